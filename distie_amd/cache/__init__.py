@@ -1,0 +1,5 @@
+from .block_pool import BlockPool, OutOfBlocks
+from .manager import GONE, CacheGroup, CacheManager, LayerCache, RequestCache, pages_needed
+
+__all__ = ["BlockPool", "OutOfBlocks", "GONE", "CacheGroup", "CacheManager", "LayerCache",
+           "RequestCache", "pages_needed"]

@@ -1,0 +1,263 @@
+"""The cache manager: pages of keys and values with a block table for each request, and
+slots for per-request state of fixed size.
+
+Layers are put into *groups* by what their mixer keeps (`PagedKV(kv_heads, head_dim,
+window)`): layers that keep every key form one group, layers that keep a window of the
+same length another. Every group has pages of its own: its own id pool, its own slabs
+`k, v : [layers of the group, pages + 1, kv_heads, block_size, head_dim]` (the last page
+is a sink that is never handed out: padding rows of a captured decode step write there,
+as in worker/src/inference/torch_engine.py:439-446) and, for each request, its own block
+table. A table is addressed by position: entry i holds the page of positions
+i*block_size .. (i+1)*block_size - 1, or -1 once a window has passed that page and it
+was given back. Pages are handed out when a step needs them (`reserve`), given back when
+a request ends (`release`), is preempted (`reset`), or a window has passed them
+(`commit`), and are used again with their stale contents, which no kernel may read.
+
+The reference has one group and Python lists of ids on each sequence
+(worker/src/inference/kv_cache.py:61-103, worker/src/inference/scheduler.py:50).
+
+Slots: every live request owns one slot id. Layers whose mixer declares `FixedState`
+get a float32 slab `[slots + 1, *shape]` each; a request's row is zeroed when the slot is
+taken. The model of this engine has no such layer, the slots exist all the same.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import torch
+
+from ..parts.base import FixedState, PagedKV
+from .block_pool import BlockPool, OutOfBlocks
+
+GONE = -1
+
+
+def pages_needed(token_count: int, block_size: int) -> int:
+    """worker/src/inference/kv_cache.py:28-33: (0,16)=0, (16,16)=1, (17,16)=2."""
+    if block_size < 1:
+        raise ValueError("block_size must be >= 1")
+    if token_count <= 0:
+        return 0
+    return (token_count + block_size - 1) // block_size
+
+
+@dataclass
+class LayerCache:
+    """What a mixer gets: its group's index and its own layer's slabs (or its state slab)."""
+
+    group: int = -1
+    k: Optional[torch.Tensor] = None
+    v: Optional[torch.Tensor] = None
+    state: Optional[torch.Tensor] = None
+
+
+@dataclass
+class CacheGroup:
+    requirement: PagedKV
+    layers: List[int]
+    pool: BlockPool
+    k: Optional[torch.Tensor] = None      # [layers, pages + 1, KH, P, D]
+    v: Optional[torch.Tensor] = None
+
+    @property
+    def sink_page(self) -> int:
+        return self.pool.num_blocks
+
+
+@dataclass
+class RequestCache:
+    slot: int
+    num_cached: int = 0
+    tables: List[List[int]] = field(default_factory=list)   # per group, by page index
+
+
+class CacheManager:
+    def __init__(self, requirements: Sequence, block_size: int, num_blocks: int, num_slots: int,
+                 device=None, dtype=torch.float32, allocate: bool = True) -> None:
+        """`requirements[l]` is what layer l's mixer keeps: PagedKV, FixedState or None.
+        `allocate=False` makes the book-keeping without the slabs (for tests of decisions)."""
+        if block_size < 1 or num_blocks < 1 or num_slots < 1:
+            raise ValueError("block_size, num_blocks and num_slots must be >= 1")
+        self.block_size = int(block_size)
+        self.num_blocks = int(num_blocks)
+        self.num_slots = int(num_slots)
+        self.device = device
+        self.dtype = dtype
+        self.groups: List[CacheGroup] = []
+        self._layer_view: Dict[int, LayerCache] = {}
+        self._state_layers: Dict[int, torch.Tensor] = {}
+        by_need: Dict[PagedKV, CacheGroup] = {}
+        for layer, need in enumerate(requirements):
+            if isinstance(need, PagedKV):
+                if need not in by_need:
+                    by_need[need] = CacheGroup(need, [], BlockPool(self.num_blocks))
+                    self.groups.append(by_need[need])
+                by_need[need].layers.append(layer)
+            elif isinstance(need, FixedState):
+                slab = torch.zeros((self.num_slots + 1, *need.shape), dtype=torch.float32, device=device) \
+                    if allocate else None
+                self._state_layers[layer] = slab
+                self._layer_view[layer] = LayerCache(state=slab)
+            elif need is None:
+                self._layer_view[layer] = LayerCache()
+            else:
+                raise TypeError(f"layer {layer}: unknown cache requirement {need!r}")
+        for index, group in enumerate(self.groups):
+            need = group.requirement
+            if allocate:
+                shape = (len(group.layers), self.num_blocks + 1, need.num_kv_heads, self.block_size, need.head_dim)
+                group.k = torch.zeros(shape, dtype=dtype, device=device)
+                group.v = torch.zeros(shape, dtype=dtype, device=device)
+            for i, layer in enumerate(group.layers):
+                self._layer_view[layer] = LayerCache(
+                    group=index, k=group.k[i] if allocate else None, v=group.v[i] if allocate else None)
+        self.slots = BlockPool(self.num_slots)
+        self._requests: Dict[Hashable, RequestCache] = {}
+
+    # ---------------------------------------------------------------- views
+    def layer(self, layer: int) -> LayerCache:
+        return self._layer_view[layer]
+
+    @property
+    def sink_slot(self) -> int:
+        return self.num_slots
+
+    def bytes(self) -> int:
+        total = 0
+        for group in self.groups:
+            if group.k is not None:
+                total += 2 * group.k.numel() * group.k.element_size()
+        return total
+
+    # ------------------------------------------------------------- requests
+    def __contains__(self, request_id) -> bool:
+        return request_id in self._requests
+
+    def request(self, request_id) -> RequestCache:
+        return self._requests[request_id]
+
+    def live(self) -> List[Hashable]:
+        return list(self._requests)
+
+    def add(self, request_id) -> RequestCache:
+        """Take a state slot for a new request; zero its state rows."""
+        if request_id in self._requests:
+            raise ValueError(f"request {request_id!r} is already in the cache")
+        try:
+            (slot,) = self.slots.allocate(1)
+        except OutOfBlocks as exc:
+            raise OutOfBlocks(f"no free state slot (all {self.num_slots} in use)") from exc
+        for slab in self._state_layers.values():
+            if slab is not None:
+                slab[slot].zero_()
+        entry = RequestCache(slot=slot, tables=[[] for _ in self.groups])
+        self._requests[request_id] = entry
+        return entry
+
+    def _first_needed_page(self, group: CacheGroup, num_cached: int) -> int:
+        """Index of the first page a query at position >= num_cached can still read."""
+        window = group.requirement.window
+        if window is None:
+            return 0
+        return max(0, num_cached - window + 1) // self.block_size
+
+    def pages_short(self, request_id, num_new: int) -> List[int]:
+        """Per group: pages that `reserve(request_id, num_new)` would have to take."""
+        entry = self._requests.get(request_id)
+        cached = entry.num_cached if entry else 0
+        out = []
+        for g, group in enumerate(self.groups):
+            held = len(entry.tables[g]) if entry else 0
+            last = pages_needed(cached + num_new, self.block_size)
+            first = max(held, self._first_needed_page(group, cached))
+            out.append(max(0, last - first))
+        return out
+
+    def can_reserve(self, request_id, num_new: int, spare: int = 0) -> bool:
+        return all(short + spare <= group.pool.num_free
+                   for short, group in zip(self.pages_short(request_id, num_new), self.groups))
+
+    def reserve(self, request_id, num_new: int) -> None:
+        """Pages for the next `num_new` positions of the request, in every group; all or
+        nothing (OutOfBlocks leaves every pool and table as it was)."""
+        if num_new < 1:
+            raise ValueError("num_new must be >= 1")
+        entry = self._requests[request_id]
+        short = self.pages_short(request_id, num_new)
+        for need, group in zip(short, self.groups):
+            if need > group.pool.num_free:
+                raise OutOfBlocks(
+                    f"out of blocks: request {request_id!r} needs {need} pages, {group.pool.num_free} free")
+        last = pages_needed(entry.num_cached + num_new, self.block_size)
+        for g, (need, group) in enumerate(zip(short, self.groups)):
+            table = entry.tables[g]
+            # pages the window has already passed are never taken
+            while len(table) < last - need:
+                table.append(GONE)
+            table.extend(group.pool.allocate(need))
+
+    def commit(self, request_id, num_new: int) -> None:
+        """The step has written `num_new` more tokens; give back what windows have passed."""
+        entry = self._requests[request_id]
+        entry.num_cached += num_new
+        for g, group in enumerate(self.groups):
+            if group.requirement.window is None:
+                continue
+            table = entry.tables[g]
+            stop = min(self._first_needed_page(group, entry.num_cached), len(table))
+            passed = [table[i] for i in range(stop) if table[i] != GONE]
+            if passed:
+                group.pool.free(passed)
+                for i in range(stop):
+                    table[i] = GONE
+
+    def _give_back_pages(self, entry: RequestCache) -> None:
+        for g, group in enumerate(self.groups):
+            held = [b for b in entry.tables[g] if b != GONE]
+            if held:
+                group.pool.free(held)
+            entry.tables[g] = []
+        entry.num_cached = 0
+
+    def reset(self, request_id) -> None:
+        """Preemption by recompute: every page back, nothing cached, the slot's state zeroed."""
+        entry = self._requests[request_id]
+        self._give_back_pages(entry)
+        for slab in self._state_layers.values():
+            if slab is not None:
+                slab[entry.slot].zero_()
+
+    def release(self, request_id) -> None:
+        """The request is over: pages and slot back."""
+        entry = self._requests.pop(request_id)
+        self._give_back_pages(entry)
+        self.slots.free([entry.slot])
+
+    # ------------------------------------------------------------ accounting
+    def free_pages(self) -> List[int]:
+        return [group.pool.num_free for group in self.groups]
+
+    def max_request_pages(self, num_tokens: int) -> int:
+        """Most pages of one group a request of `num_tokens` can hold at once."""
+        return pages_needed(num_tokens, self.block_size)
+
+    def check(self) -> None:
+        """Invariants, for tests: every page is free or in exactly one table; counts agree."""
+        for g, group in enumerate(self.groups):
+            seen = set()
+            for rid, entry in self._requests.items():
+                for page in entry.tables[g]:
+                    if page == GONE:
+                        continue
+                    if page in seen:
+                        raise AssertionError(f"page {page} of group {g} is held twice")
+                    if not group.pool.is_held(page):
+                        raise AssertionError(f"page {page} of group {g} is in a table but free")
+                    seen.add(page)
+            if len(seen) != group.pool.num_used:
+                raise AssertionError(f"group {g}: {group.pool.num_used} pages in use, {len(seen)} in tables (lost pages)")
+        slots = [e.slot for e in self._requests.values()]
+        if len(set(slots)) != len(slots) or len(slots) != self.slots.num_used:
+            raise AssertionError("state slots are held twice or lost")

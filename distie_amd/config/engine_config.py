@@ -1,0 +1,86 @@
+"""Options of the engine, typed. The reference reads the same knobs from environment
+variables ad hoc (worker/src/inference/torch_engine.py:212-226, worker/src/worker/config.py:22-57):
+WORKER_MAX_SEQS (32), WORKER_TOKEN_BUDGET (2048), WORKER_NUM_BLOCKS (1024),
+WORKER_DECODE_GRAPHS (1), WORKER_STEP_STATS (0); page size 16 (kv_cache.py:25)."""
+
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass, replace
+from typing import Optional
+
+DTYPE_NAMES = {
+    "fp32": "float32", "float32": "float32", "float": "float32",
+    "bf16": "bfloat16", "bfloat16": "bfloat16",
+}
+
+DEFAULT_BLOCK_SIZE = 16
+DEFAULT_NUM_BLOCKS = 1024
+DEFAULT_MAX_SEQS = 32
+DEFAULT_TOKEN_BUDGET = 2048
+
+
+def resolve_dtype(name: str) -> str:
+    """'auto' is bfloat16, the serving precision on the GPU (the reference's 'auto' is
+    half on the GPU: torch_engine.py:60-69). fp16 is not a precision of this engine."""
+    key = name.strip().lower()
+    if key == "auto":
+        return "bfloat16"
+    if key not in DTYPE_NAMES:
+        raise ValueError("dtype must be one of auto, " + ", ".join(sorted(DTYPE_NAMES)))
+    return DTYPE_NAMES[key]
+
+
+@dataclass(frozen=True)
+class EngineConfig:
+    dtype: str = "bfloat16"
+    block_size: int = DEFAULT_BLOCK_SIZE
+    num_blocks: Optional[int] = None        # pages of the cache; None = from max_cache_tokens or the default
+    max_cache_tokens: Optional[int] = None  # pool made for this many cached tokens
+    max_seqs: int = DEFAULT_MAX_SEQS
+    token_budget: int = DEFAULT_TOKEN_BUDGET
+    max_model_len: Optional[int] = None     # None = the model's max positions
+    use_graphs: bool = True
+    step_stats: int = 0
+    seed: int = 0
+
+    def __post_init__(self):
+        object.__setattr__(self, "dtype", resolve_dtype(self.dtype))
+        if self.block_size < 1 or self.max_seqs < 1 or self.token_budget < 1:
+            raise ValueError("block_size, max_seqs and token_budget must be >= 1")
+        if self.num_blocks is not None and self.num_blocks < 1:
+            raise ValueError("num_blocks must be >= 1")
+
+    def pages(self) -> int:
+        if self.num_blocks is not None:
+            return self.num_blocks
+        if self.max_cache_tokens is not None:
+            return max(1, -(-self.max_cache_tokens // self.block_size))
+        return DEFAULT_NUM_BLOCKS
+
+    @classmethod
+    def from_env(cls, **overrides) -> "EngineConfig":
+        """Environment variables of the reference's worker, where set."""
+        def _int(key):
+            raw = os.getenv(key, "").strip()
+            if not raw:
+                return None
+            value = int(raw)
+            if value < 1:
+                raise ValueError(f"{key} must be >= 1")
+            return value
+        env = {}
+        if _int("WORKER_MAX_SEQS"):
+            env["max_seqs"] = _int("WORKER_MAX_SEQS")
+        if _int("WORKER_TOKEN_BUDGET"):
+            env["token_budget"] = _int("WORKER_TOKEN_BUDGET")
+        if _int("WORKER_NUM_BLOCKS"):
+            env["num_blocks"] = _int("WORKER_NUM_BLOCKS")
+        raw = os.getenv("WORKER_DECODE_GRAPHS", "").strip().lower()
+        if raw:
+            env["use_graphs"] = raw not in {"0", "false", "no", "off"}
+        raw = os.getenv("WORKER_STEP_STATS", "").strip()
+        if raw:
+            env["step_stats"] = int(raw)
+        env.update({k: v for k, v in overrides.items() if v is not None})
+        return replace(cls(), **env)

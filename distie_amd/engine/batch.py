@@ -1,0 +1,127 @@
+"""From (request, its next tokens) to the flat tensors of one step.
+
+The fields are those of the reference's `build_batch`
+(worker/src/inference/qwen2/paged_attn.py:325-357): positions, slots, prefix sums, block
+table; plus the request of each token, a table and slots for every cache group, state
+slots, and the rows whose logits are wanted. Everything is packed into one int32 host
+buffer and reaches the device with one copy.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import GONE, CacheManager
+from ..kernels.interface import BatchMeta, GroupMeta
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step: its next tokens, and the places among them whose
+    logits are wanted (`want`; indexes into `tokens`)."""
+
+    request_id: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = field(default_factory=tuple)
+
+
+class BatchBuilder:
+    def __init__(self, cache: CacheManager, max_model_len: int, device, vocab_size: int) -> None:
+        self.cache = cache
+        self.device = device
+        self.vocab_size = vocab_size
+        self.max_model_len = int(max_model_len)
+        self.table_width = max(1, -(-self.max_model_len // cache.block_size))
+
+    def build(self, entries: Sequence[StepEntry], pad_requests: int = 0):
+        """-> (ids int32 [T], BatchMeta, want_rows int32 [R] or None).
+
+        Pages for the new tokens must have been reserved. `pad_requests` appends that many
+        one-token rows that write to the sink page and the sink slot (for captured steps of
+        fixed size)."""
+        if not entries:
+            raise ValueError("a step needs at least one entry")
+        cache = self.cache
+        P = cache.block_size
+        W = self.table_width
+        G = len(cache.groups)
+        B = len(entries) + pad_requests
+        T = sum(len(e.tokens) for e in entries) + pad_requests
+        R = sum(len(e.want) for e in entries)
+        if len({e.request_id for e in entries}) != len(entries):
+            raise ValueError("a request may appear once in a step")
+        # layout of the packed buffer
+        sizes = [T, T, T, B + 1, B, B, R] + [B * W] * G + [T] * G
+        offsets = np.concatenate([[0], np.cumsum(sizes)])
+        host = np.zeros(int(offsets[-1]), dtype=np.int32)
+        cut = lambda i: host[offsets[i]:offsets[i + 1]]
+        ids, positions, token_request, cu_q, kv_len, slots_state, want_rows = (cut(i) for i in range(7))
+        tables = [cut(7 + g).reshape(B, W) for g in range(G)]
+        slots = [cut(7 + G + g) for g in range(G)]
+        for t in tables:
+            t.fill(GONE)
+        t0 = 0
+        r0 = 0
+        max_q = max_kv = 1
+        host_past = np.zeros(B, dtype=np.int64)
+        for b, entry in enumerate(entries):
+            n = len(entry.tokens)
+            if n < 1:
+                raise ValueError(f"request {entry.request_id!r}: a step entry needs at least one token")
+            state = cache.request(entry.request_id)
+            past = state.num_cached
+            if past + n > self.max_model_len:
+                raise ValueError(f"request {entry.request_id!r}: {past + n} tokens exceed the limit of {self.max_model_len}")
+            toks = np.asarray(entry.tokens, dtype=np.int64)
+            if toks.min() < 0 or toks.max() >= self.vocab_size:
+                raise ValueError(f"request {entry.request_id!r}: token id outside 0..{self.vocab_size - 1}")
+            ids[t0:t0 + n] = toks
+            pos = np.arange(past, past + n, dtype=np.int64)
+            positions[t0:t0 + n] = pos
+            token_request[t0:t0 + n] = b
+            cu_q[b + 1] = t0 + n
+            kv_len[b] = past + n
+            slots_state[b] = state.slot
+            host_past[b] = past
+            for g in range(G):
+                table = np.asarray(state.tables[g], dtype=np.int64)
+                if len(table) * P < past + n:
+                    raise ValueError(f"request {entry.request_id!r}: pages were not reserved for this step")
+                tables[g][b, :len(table)] = table
+                pages = table[pos // P]
+                if (pages < 0).any():
+                    raise AssertionError("a new token would be written to a page that was given back")
+                slots[g][t0:t0 + n] = pages * P + pos % P
+            for w in entry.want:
+                if not 0 <= int(w) < n:
+                    raise ValueError(f"request {entry.request_id!r}: wanted place {w} is outside its {n} tokens")
+                want_rows[r0] = t0 + int(w)
+                r0 += 1
+            t0 += n
+            max_q = max(max_q, n)
+            max_kv = max(max_kv, past + n)
+        for b in range(len(entries), B):           # padding rows
+            positions[t0] = 0
+            token_request[t0] = b
+            cu_q[b + 1] = t0 + 1
+            kv_len[b] = 1
+            slots_state[b] = cache.sink_slot
+            for g, group in enumerate(cache.groups):
+                tables[g][b, 0] = group.sink_page
+                slots[g][t0] = group.sink_page * P
+            t0 += 1
+        dev = torch.from_numpy(host).to(self.device, non_blocking=False)
+        dcut = lambda i: dev[int(offsets[i]):int(offsets[i + 1])]
+        meta = BatchMeta(
+            num_tokens=T, num_requests=B,
+            positions=dcut(1), token_request=dcut(2), cu_q=dcut(3), kv_len=dcut(4), state_slots=dcut(5),
+            max_q=int(max_q), max_kv=int(max_kv), block_size=P,
+            groups=[GroupMeta(block_table=dcut(7 + g).view(B, W), slots=dcut(7 + G + g)) for g in range(G)],
+            host_cu_q=cu_q.copy(), host_past=host_past,
+            all_decode=(max_q == 1),
+        )
+        return dcut(0), meta, (dcut(6) if R else None)

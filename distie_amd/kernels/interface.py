@@ -1,0 +1,109 @@
+"""The kernel surface: every device operation the parts and the engine use.
+
+The product implementation is `HipOps` (hand-written HIP for gfx950, loaded from
+shared libraries built out of `distie_amd/csrc`); there is no other implementation in
+this package and no fallback: constructing `HipOps` without a GPU or without the
+libraries raises. Parts never touch torch math directly; they call these methods, so
+what runs on the device is exactly this list.
+
+Conventions: T = tokens of the step (all requests, flattened), B = requests of the
+step, `act` = the engine's activation dtype (bfloat16 or float32). The residual stream
+is always float32. Weights may be bfloat16 or float32 whatever `act` is.
+"""
+
+from __future__ import annotations
+
+import abc
+from dataclasses import dataclass, field
+from typing import List, Optional
+
+import torch
+
+
+@dataclass
+class GroupMeta:
+    """Addressing of one cache group for one step."""
+
+    block_table: torch.Tensor          # int32 [B, W]; -1 where a page was given back
+    slots: torch.Tensor                # int32 [T]; block * block_size + offset of each new token
+
+
+@dataclass
+class BatchMeta:
+    """Device tensors that describe one flattened step (the reference's BatchMeta,
+    worker/src/inference/qwen2/paged_attn.py:310-357, plus what windows, state slots and
+    wanted rows need)."""
+
+    num_tokens: int
+    num_requests: int
+    positions: torch.Tensor            # int32 [T] absolute position of each token
+    token_request: torch.Tensor        # int32 [T] index of the request each token belongs to
+    cu_q: torch.Tensor                 # int32 [B+1] prefix sums of the new-token counts
+    kv_len: torch.Tensor               # int32 [B] tokens cached after this step (past + new)
+    state_slots: torch.Tensor          # int32 [B] per-request state slot
+    max_q: int                         # host copies, for launch geometry
+    max_kv: int
+    block_size: int
+    groups: List[GroupMeta] = field(default_factory=list)
+    # host mirrors (numpy) for parts that run per request on the host side
+    host_cu_q: Optional[object] = None
+    host_past: Optional[object] = None
+    all_decode: bool = False           # every request brings exactly one token
+
+
+class Ops(abc.ABC):
+    device: torch.device
+
+    @abc.abstractmethod
+    def embed(self, ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+        """ids int32 [T], table [V, C] -> float32 [T, C]."""
+
+    @abc.abstractmethod
+    def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
+        """float32 [T, C] -> out_dtype [T, C]; statistics in float32."""
+
+    @abc.abstractmethod
+    def add_rmsnorm(self, residual: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor,
+                    eps: float, out_dtype) -> torch.Tensor:
+        """residual (float32, updated in place) += delta; returns rmsnorm(residual)."""
+
+    @abc.abstractmethod
+    def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """x [T, K] (act) times weight [N, K] transposed, plus bias [N] -> act [T, N]."""
+
+    @abc.abstractmethod
+    def linear_f32out(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+        """As `linear` without bias, result in float32 (the logits)."""
+
+    @abc.abstractmethod
+    def rope_kv_write(self, qkv: torch.Tensor, meta: BatchMeta, group: int, k_cache: torch.Tensor,
+                      v_cache: torch.Tensor, inv_freq: Optional[torch.Tensor], num_heads: int,
+                      num_kv_heads: int, head_dim: int, write: bool) -> None:
+        """Rotate q and k of qkv [T, (H+2KH)*D] in place by each token's position (angles and
+        trigonometry in float32; no rotation if inv_freq is None) and, if `write`, store the
+        rotated k and v at the token's slot of k_cache / v_cache [NB, KH, P, D]."""
+
+    @abc.abstractmethod
+    def paged_attention(self, qkv: torch.Tensor, meta: BatchMeta, group: int, k_cache: torch.Tensor,
+                        v_cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                        scale: float, window: Optional[int]) -> torch.Tensor:
+        """softmax(q k^T * scale) v over the cached keys 0..position of each token (the last
+        `window` of them on a windowed layer), read through the block table -> act [T, H*D]."""
+
+    @abc.abstractmethod
+    def silu_mul(self, gate_up: torch.Tensor) -> torch.Tensor:
+        """[T, 2I] -> silu(first half) * second half, [T, I]."""
+
+    @abc.abstractmethod
+    def gather_rows(self, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+        """x [T, C], rows int32 [R] -> x[rows]."""
+
+    @abc.abstractmethod
+    def argmax(self, logits: torch.Tensor) -> torch.Tensor:
+        """float32 [R, V] -> int32 [R], lowest index among equals."""
+
+    @abc.abstractmethod
+    def sample(self, logits: torch.Tensor, temperature: torch.Tensor, seeds: torch.Tensor,
+               counters: torch.Tensor) -> torch.Tensor:
+        """Rows with temperature <= 0: argmax. Others: one draw from softmax(logits / t)
+        with the uniform number hash(seed, counter) -> int32 [R]."""

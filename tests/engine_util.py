@@ -1,0 +1,68 @@
+"""Helpers shared by the tests: model folders in a temporary place, an engine on the CPU
+test double or on the GPU, and replays of one request under different ways of cutting."""
+
+from __future__ import annotations
+
+import torch
+
+import plain_qwen2 as plain
+from distie_amd.cache import CacheManager
+from distie_amd.config import load_model_config
+from distie_amd.engine.batch import StepEntry
+from distie_amd.engine.model import Model
+from distie_amd.engine.runner import ModelRunner
+from distie_amd.weights import load_into
+
+
+# Spread of the random weights for each tiny configuration: large enough that logits are far
+# from uniform (the top probability is 20 to 50 times the uniform one), small enough that the
+# float32 rounding of the plain implementation itself stays near 1e-5.
+STD = {64: 0.2, 96: 0.15, 240: 0.1}
+FP32_TOL = 1e-4   # the bound the reference holds for tiny models (worker/tests/test_qwen2.py:89-93)
+
+
+def oracle(weights, cfg, ids):
+    """Logits of the plain implementation in float64, as float32."""
+    return plain.forward(weights, cfg, ids, torch.float64).float()
+
+
+def make_model_dir(tmp_path, cfg, seed=0, std=None, norm_jitter=0.2, dtype=torch.float32, name="model"):
+    std = STD.get(cfg["hidden_size"], 0.1) if std is None else std
+    weights = plain.random_weights(cfg, seed, std=std, norm_jitter=norm_jitter, dtype=dtype)
+    folder = tmp_path / name
+    plain.write_model_dir(folder, cfg, weights)
+    return folder, weights
+
+
+def build_runner(model_dir, ops, dtype=torch.float32, block_size=4, num_blocks=64, num_slots=8,
+                 max_model_len=None):
+    config = load_model_config(model_dir)
+    model = Model(config.model_spec())
+    load_into(model, model_dir, ops.device, dtype)
+    cache = CacheManager(model.cache_requirements(), block_size, num_blocks, num_slots,
+                         device=ops.device, dtype=dtype)
+    return ModelRunner(model, cache, ops, dtype, max_model_len)
+
+
+def replay_whole(runner, rid, ids):
+    logits = runner.step([StepEntry(rid, list(ids), list(range(len(ids))))])
+    runner.finish(rid)
+    return logits.float().cpu()
+
+
+def replay_cut(runner, rid, ids, cuts):
+    """Feed `ids` in portions of the sizes `cuts` (the rest one token at a time)."""
+    out = []
+    at = 0
+    sizes = list(cuts)
+    while at < len(ids):
+        n = sizes.pop(0) if sizes else 1
+        n = min(n, len(ids) - at)
+        out.append(runner.step([StepEntry(rid, list(ids[at:at + n]), list(range(n)))]))
+        at += n
+    runner.finish(rid)
+    return torch.cat(out).float().cpu()
+
+
+def random_ids(cfg, n, seed):
+    return torch.randint(0, cfg["vocab_size"], (n,), generator=torch.Generator().manual_seed(seed)).tolist()
