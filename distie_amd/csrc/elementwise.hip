@@ -1,0 +1,189 @@
+// Memory-bound kernels of a step: embedding rows, RMS norm (alone and fused with the residual
+// sum), rotation + cache write, gated activation, row gather.
+//
+// Reference formulas (paths in the reference checkout):
+//   RMS norm   worker/src/inference/qwen2/model.py:85-90
+//   rotation   worker/src/inference/qwen2/model.py:98-117
+//   cache slot worker/src/inference/qwen2/paged_attn.py:341, 360-371
+//   SwiGLU     worker/src/inference/qwen2/model.py:236
+// Statistics, angles, trigonometry and the residual sum are float32 whatever the storage type.
+
+#include "common.h"
+
+// ---------------------------------------------------------------- embedding
+template <typename W>
+__global__ void embed_kernel(const int32_t* __restrict__ ids, const W* __restrict__ table,
+                             float* __restrict__ out, int width, int vocab) {
+  const int64_t t = blockIdx.x;
+  int64_t id = ids[t];
+  if (id < 0 || id >= vocab) id = 0;  // ids are validated on the host; never read outside the table
+  const W* row = table + id * width;
+  float* dst = out + t * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_float(row[i]);
+}
+
+extern "C" int distie_embed(const int32_t* ids, const void* table, int table_dtype, float* out,
+                            int tokens, int width, int vocab, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (width <= 0 || vocab <= 0) return DISTIE_BAD_ARGUMENT;
+  const int threads = width >= 1024 ? 256 : 64;
+  DISTIE_DISPATCH(table_dtype, W,
+                  embed_kernel<W><<<tokens, threads, 0, stream>>>(ids, static_cast<const W*>(table), out, width, vocab));
+  return launch_status();
+}
+
+// ---------------------------------------------------------------- RMS norm
+// One block per row. With `delta`, the row of the residual stream is first updated
+// (residual += delta, float32) and then normed: one pass less over the activations.
+template <typename D, typename W, typename O>
+__global__ void rmsnorm_kernel(float* __restrict__ residual, const D* __restrict__ delta,
+                               const W* __restrict__ weight, O* __restrict__ out, int width, float eps) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  float* x = residual + row * width;
+  float ss = 0.f;
+  if (delta != nullptr) {
+    const D* d = delta + row * width;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+      const float v = x[i] + to_float(d[i]);
+      x[i] = v;
+      ss += v * v;
+    }
+  } else {
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+      const float v = x[i];
+      ss += v * v;
+    }
+  }
+  const float total = block_sum(ss, scratch);
+  const float scale = rsqrtf(total / static_cast<float>(width) + eps);
+  O* y = out + row * width;
+  // each thread re-reads what it wrote itself
+  for (int i = threadIdx.x; i < width; i += blockDim.x) y[i] = from_float<O>(x[i] * scale * to_float(weight[i]));
+}
+
+template <typename D, typename W>
+static int rmsnorm_launch_out(float* residual, const D* delta, const W* weight, void* out, int out_dtype,
+                              int rows, int width, float eps, hipStream_t stream) {
+  const int threads = width >= 2048 ? 512 : (width >= 512 ? 256 : 64);
+  DISTIE_DISPATCH(out_dtype, O,
+                  rmsnorm_kernel<D, W, O><<<rows, threads, 0, stream>>>(residual, delta, weight, static_cast<O*>(out), width, eps));
+  return launch_status();
+}
+
+extern "C" int distie_rmsnorm(float* residual, const void* delta, int delta_dtype, const void* weight,
+                              int weight_dtype, void* out, int out_dtype, int rows, int width, float eps,
+                              hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (width <= 0) return DISTIE_BAD_ARGUMENT;
+  DISTIE_DISPATCH(weight_dtype, W, DISTIE_DISPATCH(delta_dtype, D, return rmsnorm_launch_out<D, W>(
+      residual, static_cast<const D*>(delta), static_cast<const W*>(weight), out, out_dtype, rows, width, eps, stream)));
+  return DISTIE_BAD_ARGUMENT;
+}
+
+// ---------------------------------------------------------------- rotation + cache write
+// qkv: [T, (H + 2 KH) * D]. One block per token. Pair (j, j + R/2) of every q and k head is turned by
+// angle = float(position) * inv_freq[j] (R = 2 * pairs <= D is the rotated width). The turned k and the
+// v of the token go to the cache [pages, KH, P, D] at the token's slot (slot = page * P + offset).
+template <typename T, typename C>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,
+                                     const int32_t* __restrict__ slots, C* __restrict__ k_cache,
+                                     C* __restrict__ v_cache, const float* __restrict__ inv_freq, int pairs,
+                                     int heads, int kv_heads, int dim, int block_size, int write) {
+  const int64_t t = blockIdx.x;
+  T* row = qkv + t * static_cast<int64_t>(heads + 2 * kv_heads) * dim;
+  const float pos = static_cast<float>(positions[t]);
+  const int64_t slot = write ? slots[t] : 0;
+  const int64_t page = slot / block_size;
+  const int offset = static_cast<int>(slot % block_size);
+  const int rotated_heads = heads + kv_heads;
+  if (pairs > 0) {
+    for (int i = threadIdx.x; i < rotated_heads * pairs; i += blockDim.x) {
+      const int head = i / pairs;
+      const int j = i % pairs;
+      float s, c;
+      sincosf(pos * inv_freq[j], &s, &c);
+      T* h = row + head * dim;
+      const float a = to_float(h[j]);
+      const float b = to_float(h[j + pairs]);
+      h[j] = from_float<T>(a * c - b * s);
+      h[j + pairs] = from_float<T>(b * c + a * s);
+    }
+  }
+  if (!write) return;
+  __syncthreads();
+  for (int i = threadIdx.x; i < kv_heads * dim; i += blockDim.x) {
+    const int head = i / dim;
+    const int d = i % dim;
+    const int64_t at = ((page * kv_heads + head) * block_size + offset) * dim + d;
+    k_cache[at] = from_float<C>(to_float(row[(heads + head) * dim + d]));
+    v_cache[at] = from_float<C>(to_float(row[(heads + kv_heads + head) * dim + d]));
+  }
+}
+
+extern "C" int distie_rope_kv_write(void* qkv, int dtype, const int32_t* positions, const int32_t* slots,
+                                    void* k_cache, void* v_cache, int cache_dtype, const float* inv_freq,
+                                    int pairs, int tokens, int heads, int kv_heads, int dim, int block_size,
+                                    int write, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (heads < 1 || kv_heads < 1 || dim < 1 || block_size < 1 || 2 * pairs > dim || pairs < 0) return DISTIE_BAD_ARGUMENT;
+  if (pairs > 0 && inv_freq == nullptr) return DISTIE_BAD_ARGUMENT;
+  const int work = (heads + kv_heads) * (pairs > 0 ? pairs : 1);
+  const int threads = work >= 512 ? 256 : (work >= 128 ? 128 : 64);
+  DISTIE_DISPATCH(dtype, T, DISTIE_DISPATCH(cache_dtype, C,
+      rope_kv_write_kernel<T, C><<<tokens, threads, 0, stream>>>(
+          static_cast<T*>(qkv), positions, slots, static_cast<C*>(k_cache), static_cast<C*>(v_cache), inv_freq,
+          pairs, heads, kv_heads, dim, block_size, write)));
+  return launch_status();
+}
+
+// ---------------------------------------------------------------- gated activation
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int64_t rows, int inter) {
+  const int64_t total = rows * inter;
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t r = i / inter;
+    const int c = static_cast<int>(i % inter);
+    const float g = to_float(gate_up[r * 2 * inter + c]);
+    const float u = to_float(gate_up[r * 2 * inter + inter + c]);
+    out[i] = from_float<T>(g / (1.f + expf(-g)) * u);
+  }
+}
+
+extern "C" int distie_silu_mul(const void* gate_up, void* out, int dtype, int rows, int inter, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (inter <= 0) return DISTIE_BAD_ARGUMENT;
+  const int64_t total = static_cast<int64_t>(rows) * inter;
+  const int threads = 256;
+  const int blocks = static_cast<int>(total / threads + 1 < 16384 ? total / threads + 1 : 16384);
+  DISTIE_DISPATCH(dtype, T, silu_mul_kernel<T><<<blocks, threads, 0, stream>>>(
+                                static_cast<const T*>(gate_up), static_cast<T*>(out), rows, inter));
+  return launch_status();
+}
+
+// ---------------------------------------------------------------- row gather
+__global__ void gather_rows_kernel(const uint8_t* __restrict__ src, const int32_t* __restrict__ rows,
+                                   uint8_t* __restrict__ dst, int64_t row_bytes, int src_rows) {
+  const int64_t r = blockIdx.x;
+  int64_t from = rows[r];
+  if (from < 0 || from >= src_rows) from = 0;
+  const uint8_t* s = src + from * row_bytes;
+  uint8_t* d = dst + r * row_bytes;
+  if ((row_bytes & 3) == 0) {
+    const uint32_t* s4 = reinterpret_cast<const uint32_t*>(s);
+    uint32_t* d4 = reinterpret_cast<uint32_t*>(d);
+    for (int64_t i = threadIdx.x; i < row_bytes / 4; i += blockDim.x) d4[i] = s4[i];
+  } else {
+    for (int64_t i = threadIdx.x; i < row_bytes; i += blockDim.x) d[i] = s[i];
+  }
+}
+
+extern "C" int distie_gather_rows(const void* src, const int32_t* rows, void* dst, int count, int64_t row_bytes,
+                                  int src_rows, hipStream_t stream) {
+  if (count <= 0) return 0;
+  if (row_bytes <= 0 || src_rows <= 0) return DISTIE_BAD_ARGUMENT;
+  gather_rows_kernel<<<count, 256, 0, stream>>>(static_cast<const uint8_t*>(src), rows,
+                                                static_cast<uint8_t*>(dst), row_bytes, src_rows);
+  return launch_status();
+}

@@ -1,0 +1,235 @@
+// Matrix products y[M,N] = x[M,K] * W[N,K]^T (+ bias[N]); W has the layout of the checkpoint.
+//
+//  * gemm_generic: every combination of float32 / bfloat16 for x, W and y, any M, N, K. Products
+//    and sums are float32 FMAs on the vector ALU: this is the true 32-bit path (no matrix-core
+//    mode of reduced precision), and the path for weights that a file keeps in 32-bit.
+//  * gemm_skinny_bf16: bfloat16 x and W, M <= 64 (decode). Weight-streaming on the matrix cores
+//    (v_mfma_f32_16x16x32_bf16): a wave owns 16 rows of W and a slice of K, reads W straight from
+//    memory into the A operand (every weight byte is read once), and the small x is the B operand.
+//    Slices of K are combined in a fixed order by the last wave to finish, so results do not
+//    depend on timing.
+//
+// The reference leaves these products to a library (worker/src/inference/qwen2/model.py:149-152,
+// 231-233, 301); large bfloat16 products (prefill) are left to the library here as well.
+
+#include "common.h"
+
+// ---------------------------------------------------------------- generic
+#define GT 64   // tile of M and of N
+#define GK 16   // tile of K
+
+template <typename X, typename W, typename Y>
+__global__ __launch_bounds__(256) void gemm_generic_kernel(const X* __restrict__ x, const W* __restrict__ w,
+                                                           const float* __restrict__ bias, Y* __restrict__ y,
+                                                           int M, int N, int K) {
+  __shared__ float xs[GK][GT + 4];
+  __shared__ float ws[GK][GT + 4];
+  const int tx = threadIdx.x % 16;   // columns (N)
+  const int ty = threadIdx.x / 16;   // rows (M)
+  const int64_t m0 = static_cast<int64_t>(blockIdx.y) * GT;
+  const int64_t n0 = static_cast<int64_t>(blockIdx.x) * GT;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += GK) {
+    // 64 rows x 16 k of each operand: 1024 elements, 4 per thread; k runs fastest (contiguous reads)
+    for (int e = threadIdx.x; e < GT * GK; e += 256) {
+      const int r = e / GK;
+      const int k = e % GK;
+      const bool in_k = k0 + k < K;
+      xs[k][r] = (in_k && m0 + r < M) ? to_float(x[(m0 + r) * K + k0 + k]) : 0.f;
+      ws[k][r] = (in_k && n0 + r < N) ? to_float(w[(n0 + r) * K + k0 + k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < GK; ++k) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = xs[k][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = ws[k][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t m = m0 + ty * 4 + i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t n = n0 + tx * 4 + j;
+      if (n >= N) continue;
+      const float v = acc[i][j] + (bias != nullptr ? bias[n] : 0.f);
+      y[m * N + n] = from_float<Y>(v);
+    }
+  }
+}
+
+template <typename X, typename W>
+static int gemm_generic_out(const X* x, const W* w, const float* bias, void* y, int y_dtype, int M, int N, int K,
+                            hipStream_t stream) {
+  dim3 grid((N + GT - 1) / GT, (M + GT - 1) / GT);
+  DISTIE_DISPATCH(y_dtype, Y, gemm_generic_kernel<X, W, Y><<<grid, 256, 0, stream>>>(x, w, bias, static_cast<Y*>(y), M, N, K));
+  return launch_status();
+}
+
+extern "C" int distie_gemm_generic(const void* x, int x_dtype, const void* w, int w_dtype, const float* bias,
+                                   void* y, int y_dtype, int M, int N, int K, hipStream_t stream) {
+  if (M <= 0) return 0;
+  if (N <= 0 || K <= 0) return DISTIE_BAD_ARGUMENT;
+  DISTIE_DISPATCH(x_dtype, X, DISTIE_DISPATCH(w_dtype, W, return gemm_generic_out<X, W>(
+      static_cast<const X*>(x), static_cast<const W*>(w), bias, y, y_dtype, M, N, K, stream)));
+  return DISTIE_BAD_ARGUMENT;
+}
+
+// ---------------------------------------------------------------- skinny, bfloat16, matrix cores
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+#define SK_ROWS 16          // rows of W per wave
+#define SK_KSTEP 128        // k per wave iteration: each lane reads 4 x 16 bytes = 64 contiguous bytes of its row
+
+// One wave per block. blockIdx.x: block of 16 rows of W; blockIdx.y: slice of K.
+// MB = ceil(M / 16) column blocks of x (1..4).
+// In a k-step the lane (r = lane % 16, g = lane / 16) reads W[n0 + r][k0 + 32 g + 8 j .. + 7] for j = 0..3 and the
+// same places of x's rows; MFMA j multiplies the two. Which k a lane holds does not matter as long as
+// A and B agree, and they do: both use the same function of (lane, j).
+template <int MB, typename Y>
+__global__ __launch_bounds__(64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                         const float* __restrict__ bias, Y* __restrict__ y,
+                                                         float* __restrict__ partial, unsigned int* __restrict__ counters,
+                                                         int M, int N, int K, int k_per_slice) {
+  const int lane = threadIdx.x;
+  const int r = lane % 16;
+  const int g = lane / 16;
+  const int64_t n0 = static_cast<int64_t>(blockIdx.x) * SK_ROWS;
+  const int slices = gridDim.y;
+  const int k_begin = blockIdx.y * k_per_slice;
+  const int k_end = min(K, k_begin + k_per_slice);
+
+  // rows outside W or x are read from the last valid row and their results dropped
+  const int64_t w_row = min<int64_t>(n0 + r, N - 1);
+  const bf16_t* wp = w + w_row * K;
+  const bf16_t* xp[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) xp[b] = x + static_cast<int64_t>(min(b * 16 + r, M - 1)) * K;
+
+  floatx4 acc[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) acc[b] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  int k0 = k_begin;
+  for (; k0 + SK_KSTEP <= k_end; k0 += SK_KSTEP) {
+    const int k = k0 + 32 * g;
+    bf16x8 a[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) a[j] = *reinterpret_cast<const bf16x8*>(wp + k + 8 * j);
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bf16x8 xb = *reinterpret_cast<const bf16x8*>(xp[b] + k + 8 * j);
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], xb, acc[b], 0, 0, 0);
+      }
+    }
+  }
+  // the rest of the slice (K is a multiple of 8; the slice's end need not be a multiple of 128)
+  for (; k0 < k_end; k0 += 32) {
+    const int k = k0 + 8 * g;
+    bf16x8 a = {};
+    const bool in = k < k_end;
+    if (in) a = *reinterpret_cast<const bf16x8*>(wp + k);
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      bf16x8 xb = {};
+      if (in) xb = *reinterpret_cast<const bf16x8*>(xp[b] + k);
+      acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, xb, acc[b], 0, 0, 0);
+    }
+  }
+
+  // acc[b][i] = sum for W row n0 + 4 g + i and x row 16 b + r
+  if (slices > 1) {
+    // partial[slice][m][n]; the last wave to arrive for this row block adds the slices in order
+    float* mine = partial + static_cast<int64_t>(blockIdx.y) * M * N;
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      const int m = b * 16 + r;
+      if (m >= M) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int64_t n = n0 + 4 * g + i;
+        if (n < N) mine[static_cast<int64_t>(m) * N + n] = acc[b][i];
+      }
+    }
+    __threadfence();
+    __shared__ unsigned int arrived;
+    if (lane == 0) arrived = atomicAdd(&counters[blockIdx.x], 1u);
+    __syncthreads();
+    if (arrived != static_cast<unsigned int>(slices - 1)) return;
+    __threadfence();
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      const int m = b * 16 + r;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int64_t n = n0 + 4 * g + i;
+        float total = 0.f;
+        if (m < M && n < N)
+          for (int s = 0; s < slices; ++s)
+            total += __hip_atomic_load(partial + (static_cast<int64_t>(s) * M + m) * N + n, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);  // written by other compute units: read past the local cache
+        acc[b][i] = total;
+      }
+    }
+    if (lane == 0) counters[blockIdx.x] = 0;   // ready for the next product
+  }
+#pragma unroll
+  for (int b = 0; b < MB; ++b) {
+    const int m = b * 16 + r;
+    if (m >= M) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t n = n0 + 4 * g + i;
+      if (n < N) y[static_cast<int64_t>(m) * N + n] = from_float<Y>(acc[b][i] + (bias != nullptr ? bias[n] : 0.f));
+    }
+  }
+}
+
+// The number of K slices the launcher will use for this shape (so that the caller can size `partial`).
+extern "C" int distie_gemm_skinny_slices(int M, int N, int K) {
+  const int row_blocks = (N + SK_ROWS - 1) / SK_ROWS;
+  // aim at >= 2048 waves (8 per CU) while keeping >= 256 k per slice
+  int slices = 1;
+  while (row_blocks * slices < 2048 && K / (slices * 2) >= 256 && slices < 32) slices *= 2;
+  return slices;
+}
+
+// `partial`: float32 [slices * M * N] scratch, `counters`: uint32 [ceil(N / 16)] zero before the first call
+// (the kernel leaves them zero). Both may be null if slices == 1.
+extern "C" int distie_gemm_skinny_bf16(const void* x, const void* w, const float* bias, void* y, int y_dtype,
+                                       int M, int N, int K, float* partial, unsigned int* counters,
+                                       hipStream_t stream) {
+  if (M <= 0) return 0;
+  if (M > 64 || N <= 0 || K <= 0 || K % 8 != 0) return DISTIE_BAD_ARGUMENT;
+  const int slices = distie_gemm_skinny_slices(M, N, K);
+  if (slices > 1 && (partial == nullptr || counters == nullptr)) return DISTIE_BAD_ARGUMENT;
+  int k_per_slice = (K + slices - 1) / slices;
+  k_per_slice = (k_per_slice + SK_KSTEP - 1) / SK_KSTEP * SK_KSTEP;
+  dim3 grid((N + SK_ROWS - 1) / SK_ROWS, slices);
+  const bf16_t* xb = static_cast<const bf16_t*>(x);
+  const bf16_t* wb = static_cast<const bf16_t*>(w);
+  const int mb = (M + 15) / 16;
+#define SKINNY(MB)                                                                                          \
+  DISTIE_DISPATCH(y_dtype, Y, gemm_skinny_kernel<MB, Y><<<grid, 64, 0, stream>>>(                           \
+                                  xb, wb, bias, static_cast<Y*>(y), partial, counters, M, N, K, k_per_slice))
+  switch (mb) {
+    case 1: SKINNY(1); break;
+    case 2: SKINNY(2); break;
+    case 3: SKINNY(3); break;
+    default: SKINNY(4); break;
+  }
+#undef SKINNY
+  return launch_status();
+}

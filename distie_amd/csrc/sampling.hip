@@ -1,0 +1,135 @@
+// Choosing a token from a row of float32 logits.
+//
+//   argmax: the greedy pick of the reference (worker/src/inference/model_runner.py:124-126), lowest
+//           index among equals.
+//   sample: rows with temperature <= 0 are greedy; others draw once from softmax(logits / t)
+//           (worker/src/inference/model_runner.py:127-129). The reference draws from a global
+//           generator; here the uniform number is a hash of (seed, counter) of the request, so a run
+//           can be repeated. The draw inverts the cumulative sum: the token is the first index whose
+//           cumulative weight exceeds u * total.
+
+#include "common.h"
+
+#define SAMPLE_THREADS 256
+
+struct Best {
+  float value;
+  int index;
+};
+
+__device__ __forceinline__ Best better(Best a, Best b) {
+  if (b.value > a.value || (b.value == a.value && b.index < a.index)) return b;
+  return a;
+}
+
+__device__ __forceinline__ Best block_best(Best mine, Best* scratch) {
+#pragma unroll
+  for (int o = DISTIE_WAVE / 2; o > 0; o >>= 1) {
+    Best other{__shfl_xor(mine.value, o, DISTIE_WAVE), __shfl_xor(mine.index, o, DISTIE_WAVE)};
+    mine = better(mine, other);
+  }
+  const int wave = threadIdx.x / DISTIE_WAVE;
+  const int waves = blockDim.x / DISTIE_WAVE;
+  __syncthreads();
+  if (threadIdx.x % DISTIE_WAVE == 0) scratch[wave] = mine;
+  __syncthreads();
+  Best out = scratch[0];
+  for (int w = 1; w < waves; ++w) out = better(out, scratch[w]);
+  return out;
+}
+
+__device__ __forceinline__ Best row_best(const float* row, int vocab, Best* scratch) {
+  Best mine{-INFINITY, 0x7fffffff};
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) mine = better(mine, Best{row[i], i});
+  Best out = block_best(mine, scratch);
+  if (out.index >= vocab) out.index = 0;   // a row of NaN or -inf
+  return out;
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void argmax_kernel(const float* __restrict__ logits,
+                                                                int32_t* __restrict__ out, int vocab) {
+  __shared__ Best scratch[SAMPLE_THREADS / DISTIE_WAVE];
+  const Best best = row_best(logits + static_cast<int64_t>(blockIdx.x) * vocab, vocab, scratch);
+  if (threadIdx.x == 0) out[blockIdx.x] = best.index;
+}
+
+extern "C" int distie_argmax(const float* logits, int32_t* out, int rows, int vocab, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (vocab <= 0) return DISTIE_BAD_ARGUMENT;
+  argmax_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, out, vocab);
+  return launch_status();
+}
+
+// splitmix64 of (seed, counter) -> a float in [0, 1) with 24 random bits
+__device__ __forceinline__ float uniform_of(uint64_t seed, uint64_t counter) {
+  uint64_t z = seed * 0x9E3779B97F4A7C15ull + counter * 0xD1B54A32D192ED03ull + 0x94D049BB133111EBull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  z = z ^ (z >> 31);
+  return static_cast<float>(z >> 40) * (1.0f / 16777216.0f);
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __restrict__ logits,
+                                                                const float* __restrict__ temperature,
+                                                                const int64_t* __restrict__ seeds,
+                                                                const int64_t* __restrict__ counters,
+                                                                int32_t* __restrict__ out, int vocab) {
+  __shared__ Best best_scratch[SAMPLE_THREADS / DISTIE_WAVE];
+  __shared__ float sums[SAMPLE_THREADS];
+  __shared__ float reduce_scratch[16];
+  const float* row = logits + static_cast<int64_t>(blockIdx.x) * vocab;
+  const Best best = row_best(row, vocab, best_scratch);
+  const float t = temperature[blockIdx.x];
+  if (!(t > 0.f)) {
+    if (threadIdx.x == 0) out[blockIdx.x] = best.index;
+    return;
+  }
+  // every thread owns a contiguous run of the vocabulary
+  const int per = (vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  const int begin = min(vocab, static_cast<int>(threadIdx.x) * per);
+  const int end = min(vocab, begin + per);
+  const float inv_t = 1.f / t;
+  float mine = 0.f;
+  for (int i = begin; i < end; ++i) mine += expf((row[i] - best.value) * inv_t);
+  sums[threadIdx.x] = mine;
+  const float total = block_sum(mine, reduce_scratch);
+  __syncthreads();
+  const float target = uniform_of(static_cast<uint64_t>(seeds[blockIdx.x]), static_cast<uint64_t>(counters[blockIdx.x])) * total;
+  if (threadIdx.x == 0) {
+    // find the run that holds the target, then the token inside it
+    float before = 0.f;
+    int owner = 0;
+    for (; owner < SAMPLE_THREADS - 1; ++owner) {
+      if (before + sums[owner] > target) break;
+      before += sums[owner];
+    }
+    int b = min(vocab, owner * per), e = min(vocab, b + per);
+    int pick = -1;
+    float running = before;
+    for (int i = b; i < e; ++i) {
+      running += expf((row[i] - best.value) * inv_t);
+      if (running > target) {
+        pick = i;
+        break;
+      }
+    }
+    if (pick < 0) {
+      // rounding left the target beyond the last run: take the last token with weight
+      pick = best.index;
+      for (int i = vocab - 1; i >= 0; --i)
+        if (expf((row[i] - best.value) * inv_t) > 0.f) {
+          pick = i;
+          break;
+        }
+    }
+    out[blockIdx.x] = pick;
+  }
+}
+
+extern "C" int distie_sample(const float* logits, const float* temperature, const int64_t* seeds,
+                             const int64_t* counters, int32_t* out, int rows, int vocab, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (vocab <= 0) return DISTIE_BAD_ARGUMENT;
+  sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, temperature, seeds, counters, out, vocab);
+  return launch_status();
+}

@@ -1,0 +1,250 @@
+"""`HipOps`: the kernel surface on hand-written HIP kernels for gfx950.
+
+The kernels live in shared libraries built from `distie_amd/csrc` and are called through
+ctypes with raw device pointers on torch's current HIP stream, so they take part in
+stream order and in graph capture like any other launch. torch is the allocator and the
+stream/graph owner; the only library routine on this path is the matrix product for
+large bfloat16 operands (the reference leaves its products to a library too).
+
+Constructing `HipOps` without a GPU, without hipcc-built libraries, or for a head size
+the kernels refuse, raises: there is no fallback.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Dict, Optional
+
+import torch
+
+from ..csrc import build
+from .interface import BatchMeta, Ops
+
+_F32, _BF16 = 0, 1
+_CODES = {torch.float32: _F32, torch.bfloat16: _BF16}
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+_L = ctypes.c_int64
+_F = ctypes.c_float
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _CODES[t.dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 and bfloat16 tensors, not {t.dtype}") from None
+
+
+def _check(status: int, name: str) -> None:
+    if status == 0:
+        return
+    if status < 0:
+        raise KernelError(f"{name}: the kernel refuses these sizes or types")
+    raise KernelError(f"{name}: launch failed with HIP error {status}")
+
+
+class HipOps(Ops):
+    SKINNY_MAX_ROWS = 64
+
+    def __init__(self, device="cuda:0") -> None:
+        self.device = torch.device(device)
+        if self.device.type != "cuda" or not torch.cuda.is_available():
+            raise KernelError("HipOps needs an AMD GPU (torch.cuda is not available): there is no CPU path")
+        name = torch.cuda.get_device_properties(self.device).gcnArchName
+        if not name.startswith("gfx950"):
+            raise KernelError(f"the kernels are built for gfx950 (MI355X); this device is {name}")
+        self._ops = ctypes.CDLL(str(build.ensure("ops")))
+        self._declare()
+        self._attn: Dict[int, ctypes.CDLL] = {}
+        self._partial: Optional[torch.Tensor] = None
+        self._counters = torch.zeros(16384, dtype=torch.int32, device=self.device)
+
+    # ------------------------------------------------------------ plumbing
+    def _declare(self) -> None:
+        o = self._ops
+        o.distie_embed.argtypes = [_P, _P, _I, _P, _I, _I, _I, _P]
+        o.distie_rmsnorm.argtypes = [_P, _P, _I, _P, _I, _P, _I, _I, _I, _F, _P]
+        o.distie_rope_kv_write.argtypes = [_P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P]
+        o.distie_silu_mul.argtypes = [_P, _P, _I, _I, _I, _P]
+        o.distie_gather_rows.argtypes = [_P, _P, _P, _I, _L, _I, _P]
+        o.distie_gemm_generic.argtypes = [_P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _P]
+        o.distie_gemm_skinny_slices.argtypes = [_I, _I, _I]
+        o.distie_gemm_skinny_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P]
+        o.distie_argmax.argtypes = [_P, _P, _I, _I, _P]
+        o.distie_sample.argtypes = [_P, _P, _P, _P, _P, _I, _I, _P]
+
+    def _stream(self):
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+    def attention_library(self, head_dim: int) -> ctypes.CDLL:
+        lib = self._attn.get(head_dim)
+        if lib is None:
+            if head_dim % 16 or not 16 <= head_dim <= 256:
+                raise KernelError(f"attention kernels take head sizes 16, 32, ..., 256, not {head_dim}")
+            lib = ctypes.CDLL(str(build.ensure(f"attn_d{head_dim}")))
+            lib.distie_attention_generic.argtypes = [_P, _I, _L, _P, _P, _I, _P, _P, _P, _I, _P,
+                                                     _I, _I, _I, _I, _F, _I, _P]
+            if lib.distie_attention_head_dim() != head_dim:
+                raise KernelError("attention library was built for another head size")
+            self._attn[head_dim] = lib
+        return lib
+
+    def _own(self, *tensors) -> None:
+        for t in tensors:
+            if t is None:
+                continue
+            if t.device != self.device:
+                raise KernelError(f"tensor on {t.device}, kernels run on {self.device}")
+            if not t.is_contiguous():
+                raise KernelError("kernels take contiguous tensors")
+
+    # ------------------------------------------------------------ operations
+    def embed(self, ids, table):
+        self._own(ids, table)
+        out = torch.empty((ids.shape[0], table.shape[1]), dtype=torch.float32, device=self.device)
+        _check(self._ops.distie_embed(ids.data_ptr(), table.data_ptr(), _code(table), out.data_ptr(),
+                                      ids.shape[0], table.shape[1], table.shape[0], self._stream()), "embed")
+        return out
+
+    def rmsnorm(self, x, weight, eps, out_dtype):
+        self._own(x, weight)
+        if x.dtype != torch.float32:
+            raise KernelError("rmsnorm reads the float32 residual stream")
+        out = torch.empty(x.shape, dtype=out_dtype, device=self.device)
+        _check(self._ops.distie_rmsnorm(x.data_ptr(), None, _F32, weight.data_ptr(), _code(weight),
+                                        out.data_ptr(), _CODES[out_dtype], x.shape[0], x.shape[1], eps,
+                                        self._stream()), "rmsnorm")
+        return out
+
+    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype):
+        self._own(residual, delta, weight)
+        if residual.dtype != torch.float32 or residual.shape != delta.shape:
+            raise KernelError("add_rmsnorm: residual must be float32 and shaped like delta")
+        out = torch.empty(residual.shape, dtype=out_dtype, device=self.device)
+        _check(self._ops.distie_rmsnorm(residual.data_ptr(), delta.data_ptr(), _code(delta), weight.data_ptr(),
+                                        _code(weight), out.data_ptr(), _CODES[out_dtype], residual.shape[0],
+                                        residual.shape[1], eps, self._stream()), "add_rmsnorm")
+        return out
+
+    def _linear(self, x, weight, bias, out_dtype):
+        self._own(x, weight, bias)
+        M, K = x.shape
+        N = weight.shape[0]
+        if weight.shape[1] != K:
+            raise KernelError(f"linear: x is [{M}, {K}], weight is {list(weight.shape)}")
+        if bias is not None and (bias.dtype != torch.float32 or bias.shape[0] != N):
+            raise KernelError("linear: bias must be float32 [N]")
+        both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+        if both_bf16 and M <= self.SKINNY_MAX_ROWS and K % 8 == 0:
+            out = torch.empty((M, N), dtype=out_dtype, device=self.device)
+            slices = self._ops.distie_gemm_skinny_slices(M, N, K)
+            partial = None
+            if slices > 1:
+                need = slices * M * N
+                if self._partial is None or self._partial.numel() < need:
+                    if torch.cuda.is_current_stream_capturing():
+                        raise KernelError("split-K scratch must be sized before a graph is captured")
+                    self._partial = torch.empty(max(need, 1 << 22), dtype=torch.float32, device=self.device)
+                partial = self._partial
+                if (N + 15) // 16 > self._counters.numel():
+                    raise KernelError("linear: too many rows for the split-K counters")
+            _check(self._ops.distie_gemm_skinny_bf16(
+                x.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(),
+                _CODES[out_dtype], M, N, K, partial.data_ptr() if partial is not None else None,
+                self._counters.data_ptr(), self._stream()), "gemm_skinny_bf16")
+            return out
+        if both_bf16:
+            # large bfloat16 product: the library's matrix-core kernels
+            lib_bias = None
+            if bias is not None:
+                # the library adds a bias of the activations' type; keep that copy on the tensor itself
+                lib_bias = getattr(bias, "_distie_bf16", None)
+                if lib_bias is None:
+                    lib_bias = bias._distie_bf16 = bias.to(torch.bfloat16)
+            y = torch.nn.functional.linear(x, weight, lib_bias)
+            return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
+        out = torch.empty((M, N), dtype=out_dtype, device=self.device)
+        _check(self._ops.distie_gemm_generic(
+            x.data_ptr(), _code(x), weight.data_ptr(), _code(weight), bias.data_ptr() if bias is not None else None,
+            out.data_ptr(), _CODES[out_dtype], M, N, K, self._stream()), "gemm_generic")
+        return out
+
+    def linear(self, x, weight, bias=None):
+        return self._linear(x, weight, bias, x.dtype)
+
+    def linear_f32out(self, x, weight):
+        return self._linear(x, weight, None, torch.float32)
+
+    def rope_kv_write(self, qkv, meta: BatchMeta, group, k_cache, v_cache, inv_freq, num_heads, num_kv_heads,
+                      head_dim, write):
+        self._own(qkv, k_cache, v_cache, inv_freq)
+        T = qkv.shape[0]
+        if qkv.shape[1] != (num_heads + 2 * num_kv_heads) * head_dim:
+            raise KernelError("rope_kv_write: qkv width does not match the head counts")
+        if tuple(k_cache.shape[1:]) != (num_kv_heads, meta.block_size, head_dim) or k_cache.shape != v_cache.shape:
+            raise KernelError("rope_kv_write: cache is not [pages, kv_heads, block_size, head_dim]")
+        if T != meta.num_tokens:
+            raise KernelError("rope_kv_write: qkv rows do not match the batch")
+        pairs = 0 if inv_freq is None else inv_freq.shape[0]
+        slots = meta.groups[group].slots
+        _check(self._ops.distie_rope_kv_write(
+            qkv.data_ptr(), _code(qkv), meta.positions.data_ptr(), slots.data_ptr(), k_cache.data_ptr(),
+            v_cache.data_ptr(), _code(k_cache), inv_freq.data_ptr() if inv_freq is not None else None, pairs, T,
+            num_heads, num_kv_heads, head_dim, meta.block_size, 1 if write else 0, self._stream()), "rope_kv_write")
+
+    def paged_attention(self, qkv, meta: BatchMeta, group, k_cache, v_cache, num_heads, num_kv_heads, head_dim,
+                        scale, window):
+        self._own(qkv, k_cache, v_cache)
+        lib = self.attention_library(head_dim)
+        T = qkv.shape[0]
+        table = meta.groups[group].block_table
+        if tuple(k_cache.shape[1:]) != (num_kv_heads, meta.block_size, head_dim):
+            raise KernelError("paged_attention: cache is not [pages, kv_heads, block_size, head_dim]")
+        if T != meta.num_tokens or table.shape[0] != meta.num_requests:
+            raise KernelError("paged_attention: tensors do not match the batch")
+        out = torch.empty((T, num_heads * head_dim), dtype=qkv.dtype, device=self.device)
+        _check(lib.distie_attention_generic(
+            qkv.data_ptr(), _code(qkv), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), _code(k_cache),
+            meta.positions.data_ptr(), meta.token_request.data_ptr(), table.data_ptr(), table.shape[1],
+            out.data_ptr(), T, num_heads, num_kv_heads, meta.block_size, float(scale), int(window or 0),
+            self._stream()), "attention_generic")
+        return out
+
+    def silu_mul(self, gate_up):
+        self._own(gate_up)
+        rows, two = gate_up.shape
+        out = torch.empty((rows, two // 2), dtype=gate_up.dtype, device=self.device)
+        _check(self._ops.distie_silu_mul(gate_up.data_ptr(), out.data_ptr(), _code(gate_up), rows, two // 2,
+                                         self._stream()), "silu_mul")
+        return out
+
+    def gather_rows(self, x, rows):
+        self._own(x, rows)
+        out = torch.empty((rows.shape[0], x.shape[1]), dtype=x.dtype, device=self.device)
+        _check(self._ops.distie_gather_rows(x.data_ptr(), rows.data_ptr(), out.data_ptr(), rows.shape[0],
+                                            x.shape[1] * x.element_size(), x.shape[0], self._stream()), "gather_rows")
+        return out
+
+    def argmax(self, logits):
+        self._own(logits)
+        if logits.dtype != torch.float32:
+            raise KernelError("argmax reads float32 logits")
+        out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
+        _check(self._ops.distie_argmax(logits.data_ptr(), out.data_ptr(), logits.shape[0], logits.shape[1],
+                                       self._stream()), "argmax")
+        return out
+
+    def sample(self, logits, temperature, seeds, counters):
+        self._own(logits, temperature, seeds, counters)
+        if logits.dtype != torch.float32 or temperature.dtype != torch.float32 or \
+                seeds.dtype != torch.int64 or counters.dtype != torch.int64:
+            raise KernelError("sample: logits/temperature float32, seeds/counters int64")
+        out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
+        _check(self._ops.distie_sample(logits.data_ptr(), temperature.data_ptr(), seeds.data_ptr(),
+                                       counters.data_ptr(), out.data_ptr(), logits.shape[0], logits.shape[1],
+                                       self._stream()), "sample")
+        return out

@@ -66,3 +66,25 @@ def replay_cut(runner, rid, ids, cuts):
 
 def random_ids(cfg, n, seed):
     return torch.randint(0, cfg["vocab_size"], (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+def check_logits(got, weights, cfg, ids, dtype, folder=None):
+    """float32: within FP32_TOL of the float64 oracle.
+
+    bfloat16: rounding activations to 8 bits moves the logits of these tiny models by 2 to 3 % of
+    the largest logit at the worst place and by 0.4 % in the root mean square (measured with the
+    test double, which rounds where the engine rounds; two runs that differ only in the order of
+    float32 sums drift apart by as much, because one flipped rounding flips others downstream).
+    The bounds are about twice that: 1/16 at the worst place and 1/64 in the root mean square. A
+    wrong key, page or position moves logits by far more, and the float32 runs of the same code
+    hold the tight bound."""
+    want = oracle(weights, cfg, ids)
+    diff = got - want
+    err = diff.abs().max().item()
+    scale = want.abs().max().item()
+    if dtype == torch.float32:
+        assert err < FP32_TOL, f"max error {err} vs oracle"
+        return
+    rms = diff.pow(2).mean().sqrt().item()
+    assert err < scale / 16, f"max error {err} vs oracle, largest logit {scale}"
+    assert rms < scale / 64, f"rms error {rms} vs oracle, largest logit {scale}"

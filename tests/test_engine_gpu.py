@@ -1,0 +1,108 @@
+"""The engine on the GPU against the plain implementation: whole requests, decoding,
+portions of changing size, mixed batches with page reuse; float32 and bfloat16."""
+
+import pytest
+import torch
+
+import plain_qwen2 as plain
+from distie_amd.engine.batch import StepEntry
+from engine_util import build_runner, check_logits, make_model_dir, random_ids, replay_cut, replay_whole
+
+pytestmark = pytest.mark.gpu
+
+CONFIGS = {"A": (plain.TINY_A, 4), "B": (plain.TINY_B, 8), "C": (plain.TINY_C, 16)}
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from distie_amd.kernels.hip_ops import HipOps
+
+    return HipOps("cuda:0")
+
+
+@pytest.fixture(scope="module", params=[(c, d) for c in sorted(CONFIGS) for d in DTYPES])
+def setup(request, tmp_path_factory):
+    name, dtype_name = request.param
+    cfg, block = CONFIGS[name]
+    dtype = DTYPES[dtype_name]
+    # the file holds what the engine keeps: bfloat16 weights for the bfloat16 run
+    folder, weights = make_model_dir(tmp_path_factory.mktemp(f"m{name}{dtype_name}"), cfg, seed=11, dtype=dtype)
+    return cfg, block, folder, weights, dtype
+
+
+def test_whole(setup, ops):
+    cfg, block, folder, weights, dtype = setup
+    runner = build_runner(folder, ops, dtype, block_size=block)
+    ids = random_ids(cfg, 100, 1)
+    check_logits(replay_whole(runner, "a", ids), weights, cfg, ids, dtype, folder)
+    # the first tokens of a sequence
+    check_logits(replay_whole(runner, "b", ids[:3]), weights, cfg, ids[:3], dtype, folder)
+    check_logits(replay_whole(runner, "c", ids[:1]), weights, cfg, ids[:1], dtype, folder)
+    runner.cache.check()
+
+
+def test_prompt_then_last_32_one_by_one(setup, ops):
+    cfg, block, folder, weights, dtype = setup
+    runner = build_runner(folder, ops, dtype, block_size=block)
+    ids = random_ids(cfg, 120, 2)
+    check_logits(replay_cut(runner, "a", ids, [88]), weights, cfg, ids, dtype, folder)
+
+
+@pytest.mark.parametrize("cuts", [[2, 3, 5, 7, 2, 11, 4, 33, 2, 2, 19], [64, 2, 2, 2, 30], [1, 1, 2, 70, 9]])
+def test_portions(setup, ops, cuts):
+    cfg, block, folder, weights, dtype = setup
+    runner = build_runner(folder, ops, dtype, block_size=block)
+    ids = random_ids(cfg, 110, 3)
+    check_logits(replay_cut(runner, "a", ids, cuts), weights, cfg, ids, dtype, folder)
+
+
+def test_mixed_with_page_reuse(setup, ops):
+    cfg, block, folder, weights, dtype = setup
+    lengths = [90, 120, 45, 101, 64, 77, 33]
+    pages = sum(-(-n // block) for n in sorted(lengths)[-4:])
+    runner = build_runner(folder, ops, dtype, block_size=block, num_blocks=pages, num_slots=4)
+    # poison the cache: stale contents must never be read
+    for group in runner.cache.groups:
+        group.k.fill_(float("nan"))
+        group.v.fill_(float("nan"))
+    reqs = {f"r{i}": random_ids(cfg, n, 10 + i) for i, n in enumerate(lengths)}
+    got = {r: [] for r in reqs}
+    at = {r: 0 for r in reqs}
+    waiting, live = list(reqs), []
+    gen = torch.Generator().manual_seed(5)
+    step = 0
+    while waiting or live:
+        while waiting and len(live) < 4:
+            live.append(waiting.pop(0))
+        entries = []
+        for r in live:
+            left = len(reqs[r]) - at[r]
+            n = 1 if left <= 32 else min(left - 32, int(torch.randint(2, 40, (1,), generator=gen)))
+            if step % 4 == 3 and r == live[0] and len(live) > 1:
+                continue
+            entries.append(StepEntry(r, reqs[r][at[r]:at[r] + n], list(range(n))))
+        logits = runner.step(entries)
+        row = 0
+        for e in entries:
+            n = len(e.tokens)
+            got[e.request_id].append(logits[row:row + n].float().cpu())
+            row += n
+            at[e.request_id] += n
+        for r in list(live):
+            if at[r] == len(reqs[r]):
+                runner.finish(r)
+                live.remove(r)
+        runner.cache.check()
+        step += 1
+    for r in reqs:
+        check_logits(torch.cat(got[r]), weights, cfg, reqs[r], dtype, folder)
+    assert all(f == pages for f in runner.cache.free_pages())
+
+
+def test_long_decoding(setup, ops):
+    cfg, block, folder, weights, dtype = setup
+    n = min(cfg["max_position_embeddings"], 250)
+    runner = build_runner(folder, ops, dtype, block_size=block, num_blocks=-(-n // block))
+    ids = random_ids(cfg, n, 4)
+    check_logits(replay_cut(runner, "a", ids, [5]), weights, cfg, ids, dtype, folder)

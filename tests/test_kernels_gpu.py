@@ -1,0 +1,246 @@
+"""Each HIP kernel alone against a plain torch float32/float64 reference of the same
+operation, at sizes other than the engine's tiny models (widths and vocabularies that
+are no power of two, grouped heads, odd page sizes)."""
+
+import math
+
+import pytest
+import torch
+
+from torch_ops import TorchOps, plain_sample
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from distie_amd.kernels.hip_ops import HipOps
+
+    return HipOps("cuda:0")
+
+
+def rand(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    return (torch.randn(*shape, generator=g, device="cuda") * scale).to(dtype)
+
+
+def close(got, want, dtype, scale=1.0):
+    tol = 2e-5 if dtype == torch.float32 else 1.0 / 128
+    err = (got.double() - want.double()).abs().max().item()
+    assert err <= tol * scale, f"max error {err} > {tol * scale}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(ops, dtype):
+    table = rand(301, 72, dtype=dtype)
+    ids = torch.tensor([0, 300, 5, 5, 17], dtype=torch.int32, device="cuda")
+    got = ops.embed(ids, table)
+    assert got.dtype == torch.float32
+    assert torch.equal(got, table[ids.long()].float())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width", [40, 1000, 3000])
+def test_rmsnorm_and_fused_add(ops, dtype, width):
+    x = rand(7, width, seed=1, scale=3.0)
+    w = rand(width, dtype=dtype, seed=2)
+    eps = 1e-5
+    want = x.double() * torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True) + eps) * w.double()
+    got = ops.rmsnorm(x, w, eps, dtype)
+    assert got.dtype == dtype
+    close(got, want, dtype, scale=want.abs().max().item())
+    delta = rand(7, width, dtype=dtype, seed=3)
+    res = x.clone()
+    got = ops.add_rmsnorm(res, delta, w, eps, dtype)
+    s = x.double() + delta.double()
+    assert torch.allclose(res.double(), s, atol=1e-6)
+    want = s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + eps) * w.double()
+    close(got, want, dtype, scale=want.abs().max().item())
+
+
+@pytest.mark.parametrize("xd,wd", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                   (torch.bfloat16, torch.float32), (torch.float32, torch.bfloat16)])
+@pytest.mark.parametrize("M,N,K", [(1, 100, 72), (5, 333, 250), (70, 65, 129), (200, 130, 64)])
+def test_gemm_generic(ops, xd, wd, M, N, K):
+    x, w, b = rand(M, K, dtype=xd, seed=1), rand(N, K, dtype=wd, seed=2), rand(N, seed=3)
+    want = x.double() @ w.double().T + b.double()
+    got = ops._linear(x, w, b, xd) if not (xd == wd == torch.bfloat16) else None
+    if got is None:
+        # bf16 x bf16 goes to the matrix-core kernels; call the generic kernel directly
+        got = torch.empty(M, N, dtype=xd, device="cuda")
+        assert ops._ops.distie_gemm_generic(x.data_ptr(), 1, w.data_ptr(), 1, b.data_ptr(), got.data_ptr(), 1,
+                                            M, N, K, None) == 0
+    close(got, want, xd, scale=want.abs().max().item())
+    got32 = ops.linear_f32out(x, w) if not (xd == wd == torch.bfloat16) else None
+    if got32 is not None:
+        assert got32.dtype == torch.float32
+        close(got32, x.double() @ w.double().T, torch.float32, scale=want.abs().max().item())
+
+
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(48, 128), (100, 264), (1536, 1536), (333, 8960), (2050, 72)])
+def test_gemm_skinny_bf16(ops, M, N, K):
+    x, w, b = rand(M, K, dtype=torch.bfloat16, seed=1), rand(N, K, dtype=torch.bfloat16, seed=2), rand(N, seed=3)
+    want = x.double() @ w.double().T
+    got = ops.linear_f32out(x, w)
+    close(got, want, torch.float32, scale=5 * want.abs().max().item())
+    got = ops.linear(x, w, b)
+    assert got.dtype == torch.bfloat16
+    close(got, want + b.double(), torch.bfloat16, scale=want.abs().max().item())
+    # the counters are left at zero: a second product with other sizes is right too
+    again = ops.linear_f32out(x[:1], w)
+    close(again, want[:1], torch.float32, scale=5 * want.abs().max().item())
+
+
+def test_gemm_large_bf16_uses_library_and_matches(ops):
+    x, w, b = rand(300, 136, dtype=torch.bfloat16, seed=1), rand(250, 136, dtype=torch.bfloat16, seed=2), rand(250, seed=3)
+    want = x.double() @ w.double().T + b.double()
+    close(ops.linear(x, w, b), want, torch.bfloat16, scale=want.abs().max().item())
+
+
+def make_meta(positions, token_request, cu_q, kv_len, tables, slots, block_size):
+    from distie_amd.kernels.interface import BatchMeta, GroupMeta
+
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    B = len(kv_len)
+    return BatchMeta(num_tokens=len(positions), num_requests=B, positions=i32(positions),
+                     token_request=i32(token_request), cu_q=i32(cu_q), kv_len=i32(kv_len),
+                     state_slots=i32([0] * B), max_q=max(b - a for a, b in zip(cu_q, cu_q[1:])),
+                     max_kv=max(kv_len), block_size=block_size,
+                     groups=[GroupMeta(block_table=i32(tables), slots=i32(slots))])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,dim,pairs", [(4, 2, 16, 8), (3, 1, 32, 16), (5, 5, 48, 24), (12, 2, 128, 64), (2, 2, 64, 16)])
+def test_rope_kv_write(ops, dtype, heads, kv_heads, dim, pairs):
+    P, pages = 4, 9
+    positions = [0, 1, 2, 3, 4, 100, 7]
+    token_request = [0, 0, 0, 0, 0, 1, 2]
+    slots = [3 * P + 0, 3 * P + 1, 3 * P + 2, 3 * P + 3, 0 * P + 0, 7 * P + 0, 5 * P + 3]
+    meta = make_meta(positions, token_request, [0, 5, 6, 7], [5, 101, 8], [[3, 0, -1]] * 3, slots, P)
+    qkv = rand(7, (heads + 2 * kv_heads) * dim, dtype=dtype, seed=4)
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, 2 * pairs, 2, dtype=torch.float32) / (2 * pairs)))).cuda()
+    k1 = torch.zeros(pages, kv_heads, P, dim, dtype=dtype, device="cuda")
+    v1 = torch.zeros_like(k1)
+    k2, v2, qkv2 = k1.clone(), v1.clone(), qkv.clone()
+    ops.rope_kv_write(qkv, meta, 0, k1, v1, inv_freq, heads, kv_heads, dim, True)
+    ref = TorchOps("cuda")
+    ref.rope_kv_write(qkv2, meta, 0, k2, v2, inv_freq, heads, kv_heads, dim, True)
+    close(qkv, qkv2, dtype, scale=4.0)
+    close(k1, k2, dtype, scale=4.0)
+    assert torch.equal(v1, v2)
+    # float64 check of the rotation at a far position, where the angle's rounding matters
+    view = qkv.view(7, heads + 2 * kv_heads, dim)
+    src = qkv2.new_tensor(rand(7, (heads + 2 * kv_heads) * dim, dtype=dtype, seed=4).double().cpu().numpy()).view(7, -1, dim)
+    ang = torch.tensor(100.0, dtype=torch.float32) * inv_freq.cpu()   # float32 angle, as specified
+    a, b = src[5, 0, :pairs].double().cpu(), src[5, 0, pairs:2 * pairs].double().cpu()
+    want = torch.cat([a * ang.double().cos() - b * ang.double().sin(), b * ang.double().cos() + a * ang.double().sin()])
+    close(view[5, 0, :2 * pairs].cpu(), want, dtype, scale=4.0)
+    if 2 * pairs < dim:
+        assert torch.equal(view[5, 0, 2 * pairs:], src[5, 0, 2 * pairs:].to(dtype).cuda())
+    # without writing, the cache stays as it is
+    k3 = torch.zeros_like(k1)
+    ops.rope_kv_write(qkv.clone(), meta, 0, k3, torch.zeros_like(k1), inv_freq, heads, kv_heads, dim, False)
+    assert k3.abs().sum() == 0
+
+
+def paged_case(heads, kv_heads, dim, P, lens, q_lens, dtype, seed=0):
+    """Requests with `lens` cached tokens (the last `q_lens` of them new), pages in a shuffled order."""
+    g = torch.Generator().manual_seed(seed)
+    total_pages = sum(-(-n // P) for n in lens) + 3
+    order = torch.randperm(total_pages, generator=g).tolist()
+    width = max(-(-n // P) for n in lens) + 1
+    tables, positions, token_request, cu_q, slots = [], [], [], [0], []
+    for b, (n, q) in enumerate(zip(lens, q_lens)):
+        pages = [order.pop() for _ in range(-(-n // P))]
+        tables.append(pages + [-1] * (width - len(pages)))
+        for pos in range(n - q, n):
+            positions.append(pos)
+            token_request.append(b)
+            slots.append(pages[pos // P] * P + pos % P)
+        cu_q.append(len(positions))
+    meta = make_meta(positions, token_request, cu_q, lens, tables, slots, P)
+    k = rand(total_pages, kv_heads, P, dim, dtype=dtype, seed=seed + 1)
+    v = rand(total_pages, kv_heads, P, dim, dtype=dtype, seed=seed + 2)
+    qkv = rand(len(positions), (heads + 2 * kv_heads) * dim, dtype=dtype, seed=seed + 3)
+    return meta, qkv, k, v
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,dim,P,window", [
+    (4, 2, 16, 4, None), (3, 1, 32, 8, 8), (5, 5, 48, 16, 20), (12, 2, 128, 16, None),
+    (6, 3, 64, 5, 33), (8, 1, 80, 16, None), (2, 2, 256, 32, 100)])
+def test_paged_attention(ops, dtype, heads, kv_heads, dim, P, window):
+    lens, q_lens = [70, 1, 33, 130, 200], [70, 1, 2, 1, 17]
+    meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, lens, q_lens, dtype)
+    got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
+    want = TorchOps("cuda").paged_attention(qkv.double(), meta, 0, k.double(), v.double(), heads, kv_heads, dim,
+                                            dim ** -0.5, window)
+    close(got, want, dtype, scale=1.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_finds_one_far_key(ops, dtype):
+    """One key among hundreds gets a large score: the output must be that key's value,
+    wherever the key sits (first of a page, last of a page, the window's edge)."""
+    heads, kv_heads, dim, P = 4, 2, 32, 16
+    for far, window in [(0, None), (15, None), (16, None), (287, None), (300 - 64, 64), (299, 64)]:
+        meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, [300], [1], dtype, seed=5)
+        q = qkv.view(1, heads + 2 * kv_heads, dim)
+        page = int(meta.groups[0].block_table[0, far // P])
+        k[page, :, far % P] = 0
+        k[page, :, far % P, 0] = 30.0
+        q[0, :heads] = 0
+        q[0, :heads, 0] = 30.0
+        got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
+        want = v[page, :, far % P].float().repeat_interleave(2, dim=0).reshape(1, -1)
+        close(got, want, dtype, scale=4.0)
+    # just outside the window the key must not count
+    meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, [300], [1], dtype, seed=5)
+    far = 299 - 64
+    page = int(meta.groups[0].block_table[0, far // P])
+    k[page, :, far % P, 0] = 1000.0
+    qkv.view(1, -1, dim)[0, :heads, 0] = 30.0
+    got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, 64)
+    want = TorchOps("cuda").paged_attention(qkv.double(), meta, 0, k.double(), v.double(), heads, kv_heads, dim,
+                                            dim ** -0.5, 64)
+    close(got, want, dtype, scale=4.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul_and_gather(ops, dtype):
+    gu = rand(9, 2 * 173, dtype=dtype, seed=6, scale=3.0)
+    g, u = gu[:, :173].double(), gu[:, 173:].double()
+    want = g / (1 + torch.exp(-g)) * u
+    close(ops.silu_mul(gu), want, dtype, scale=want.abs().max().item())
+    x = rand(11, 77, dtype=dtype, seed=7)
+    rows = torch.tensor([10, 0, 3, 3], dtype=torch.int32, device="cuda")
+    assert torch.equal(ops.gather_rows(x, rows), x[rows.long()])
+
+
+def test_argmax_and_sample(ops):
+    logits = rand(6, 1001, seed=8, scale=2.0)
+    logits[1, 7] = logits[1, 900] = 50.0          # equals: the lowest index wins
+    logits[2, 1000] = 60.0
+    got = ops.argmax(logits)
+    assert got.tolist() == [int(r.argmax()) for r in logits[:1]] + [7, 1000] + [int(r.argmax()) for r in logits[3:]]
+    temps = torch.tensor([0.0, 0.7, 1.0, 1.5, 0.3, 2.0], device="cuda")
+    hits = 0
+    trials = 40
+    for n in range(trials):
+        seeds = torch.arange(6, device="cuda", dtype=torch.int64) * 1000 + n
+        counters = torch.full((6,), n, device="cuda", dtype=torch.int64)
+        got = ops.sample(logits, temps, seeds, counters)
+        want = plain_sample(logits, temps, seeds, counters)
+        assert got[0] == want[0]
+        hits += int((got == want.cuda()).sum())
+    # the float32 cumulative sum may step over a boundary that float64 does not; that is rare
+    assert hits >= 6 * trials - 3
+    # the draws follow the distribution: chi-square-free check on a small vocabulary
+    small = torch.tensor([[0.0, 1.0, 2.0, -1.0]], device="cuda").repeat(4000, 1)
+    draws = ops.sample(small, torch.ones(4000, device="cuda"), torch.full((4000,), 12345, device="cuda", dtype=torch.int64),
+                       torch.arange(4000, device="cuda", dtype=torch.int64))
+    freq = torch.bincount(draws.long(), minlength=4).double() / 4000
+    assert (freq.cpu() - torch.softmax(small[0].double().cpu(), 0)).abs().max() < 0.03

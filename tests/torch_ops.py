@@ -94,6 +94,21 @@ class TorchOps(Ops):
         return logits.argmax(-1).to(torch.int32)
 
     def sample(self, logits, temperature, seeds, counters):
-        from distie_amd.sampling.sampler import reference_sample
+        return plain_sample(logits, temperature, seeds, counters)
 
-        return reference_sample(logits, temperature, seeds, counters)
+
+def plain_sample(logits, temperature, seeds, counters):
+    """argmax where t <= 0; else the first index whose cumulative softmax weight (float64)
+    exceeds u * total, u from the request's (seed, counter)."""
+    from distie_amd.sampling import uniform_of
+
+    out = []
+    for row, t, seed, counter in zip(logits.double().cpu(), temperature.tolist(), seeds.tolist(), counters.tolist()):
+        if t <= 0:
+            out.append(int(row.argmax()))
+            continue
+        w = torch.exp((row - row.max()) / t)
+        target = uniform_of(seed & ((1 << 64) - 1), counter & ((1 << 64) - 1)) * w.sum()
+        hit = (torch.cumsum(w, 0) > target).nonzero()
+        out.append(int(hit[0]) if len(hit) else int((w > 0).nonzero()[-1]))
+    return torch.tensor(out, dtype=torch.int32, device=logits.device)
