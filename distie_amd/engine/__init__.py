@@ -1,0 +1,8 @@
+from .batch import StepEntry
+from .llm import LLM, RequestOutput, Trace
+from .model import Model
+from .runner import ModelRunner
+from .scheduler import BlockPoolExhausted, Emission, Scheduler, Sequence, SeqState, StepPlan
+
+__all__ = ["StepEntry", "LLM", "RequestOutput", "Trace", "Model", "ModelRunner", "BlockPoolExhausted",
+           "Emission", "Scheduler", "Sequence", "SeqState", "StepPlan"]

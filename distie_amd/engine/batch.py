@@ -37,12 +37,20 @@ class BatchBuilder:
         self.max_model_len = int(max_model_len)
         self.table_width = max(1, -(-self.max_model_len // cache.block_size))
 
-    def build(self, entries: Sequence[StepEntry], pad_requests: int = 0):
-        """-> (ids int32 [T], BatchMeta, want_rows int32 [R] or None).
+    def layout(self, T: int, B: int, R: int):
+        """Offsets of the fields inside the packed int32 buffer of a step with T tokens, B requests
+        and R wanted rows."""
+        G = len(self.cache.groups)
+        sizes = [T, T, T, B + 1, B, B, R] + [B * self.table_width] * G + [T] * G
+        return np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+
+    def fill(self, host: np.ndarray, entries: Sequence[StepEntry], pad_requests: int = 0, want_all: bool = False):
+        """Write the step into `host` (int32, at least layout(...)[-1] long).
+        -> (offsets, T, B, R, max_q, max_kv, host_cu_q, host_past)
 
         Pages for the new tokens must have been reserved. `pad_requests` appends that many
         one-token rows that write to the sink page and the sink slot (for captured steps of
-        fixed size)."""
+        fixed size). `want_all`: every row is wanted, whatever the entries say."""
         if not entries:
             raise ValueError("a step needs at least one entry")
         cache = self.cache
@@ -51,13 +59,13 @@ class BatchBuilder:
         G = len(cache.groups)
         B = len(entries) + pad_requests
         T = sum(len(e.tokens) for e in entries) + pad_requests
-        R = sum(len(e.want) for e in entries)
+        R = T if want_all else sum(len(e.want) for e in entries)
         if len({e.request_id for e in entries}) != len(entries):
             raise ValueError("a request may appear once in a step")
-        # layout of the packed buffer
-        sizes = [T, T, T, B + 1, B, B, R] + [B * W] * G + [T] * G
-        offsets = np.concatenate([[0], np.cumsum(sizes)])
-        host = np.zeros(int(offsets[-1]), dtype=np.int32)
+        offsets = self.layout(T, B, R)
+        if host.shape[0] < offsets[-1]:
+            raise ValueError("host buffer too small for this step")
+        host[:offsets[-1]] = 0
         cut = lambda i: host[offsets[i]:offsets[i + 1]]
         ids, positions, token_request, cu_q, kv_len, slots_state, want_rows = (cut(i) for i in range(7))
         tables = [cut(7 + g).reshape(B, W) for g in range(G)]
@@ -96,11 +104,12 @@ class BatchBuilder:
                 if (pages < 0).any():
                     raise AssertionError("a new token would be written to a page that was given back")
                 slots[g][t0:t0 + n] = pages * P + pos % P
-            for w in entry.want:
-                if not 0 <= int(w) < n:
-                    raise ValueError(f"request {entry.request_id!r}: wanted place {w} is outside its {n} tokens")
-                want_rows[r0] = t0 + int(w)
-                r0 += 1
+            if not want_all:
+                for w in entry.want:
+                    if not 0 <= int(w) < n:
+                        raise ValueError(f"request {entry.request_id!r}: wanted place {w} is outside its {n} tokens")
+                    want_rows[r0] = t0 + int(w)
+                    r0 += 1
             t0 += n
             max_q = max(max_q, n)
             max_kv = max(max_kv, past + n)
@@ -114,14 +123,30 @@ class BatchBuilder:
                 tables[g][b, 0] = group.sink_page
                 slots[g][t0] = group.sink_page * P
             t0 += 1
-        dev = torch.from_numpy(host).to(self.device, non_blocking=False)
+        if want_all:
+            want_rows[:] = np.arange(T)
+        return offsets, T, B, R, int(max_q), int(max_kv), cu_q.copy(), host_past
+
+    def meta_of(self, dev: torch.Tensor, offsets, T: int, B: int, R: int, max_q: int, max_kv: int,
+                host_cu_q=None, host_past=None):
+        """Views into the device copy `dev` of a packed buffer -> (ids, BatchMeta, want_rows)."""
+        G = len(self.cache.groups)
+        W = self.table_width
         dcut = lambda i: dev[int(offsets[i]):int(offsets[i + 1])]
         meta = BatchMeta(
             num_tokens=T, num_requests=B,
             positions=dcut(1), token_request=dcut(2), cu_q=dcut(3), kv_len=dcut(4), state_slots=dcut(5),
-            max_q=int(max_q), max_kv=int(max_kv), block_size=P,
+            max_q=max_q, max_kv=max_kv, block_size=self.cache.block_size,
             groups=[GroupMeta(block_table=dcut(7 + g).view(B, W), slots=dcut(7 + G + g)) for g in range(G)],
-            host_cu_q=cu_q.copy(), host_past=host_past,
-            all_decode=(max_q == 1),
+            host_cu_q=host_cu_q, host_past=host_past, all_decode=(max_q == 1),
         )
         return dcut(0), meta, (dcut(6) if R else None)
+
+    def build(self, entries: Sequence[StepEntry]):
+        """-> (ids int32 [T], BatchMeta, want_rows int32 [R] or None), on the device, with one copy."""
+        T = sum(len(e.tokens) for e in entries)
+        R = sum(len(e.want) for e in entries)
+        host = np.empty(int(self.layout(T, len(entries), R)[-1]), dtype=np.int32)
+        offsets, T, B, R, max_q, max_kv, cu_q, past = self.fill(host, entries)
+        dev = torch.from_numpy(host).to(self.device, non_blocking=False)
+        return self.meta_of(dev, offsets, T, B, R, max_q, max_kv, cu_q, past)

@@ -48,10 +48,13 @@ class ModelRunner:
                 # nothing was written yet; pages taken for this step stay with their
                 # requests and are returned when those end
                 raise
-        logits = None
+        logits, ran = None, False
         if self.graphs is not None:
-            logits = self.graphs.try_run(entries)
-        if logits is None:
+            logits = self.graphs.try_run(entries)   # a view of the bucket's buffer: use it before the next step
+            ran = logits is not None
+            if ran and logits.shape[0] == 0:
+                logits = None
+        if not ran:
             ids, meta, want_rows = self.builder.build(entries)
             logits = self.model.forward(self.ops, ids, meta, self.cache, self.act_dtype, want_rows)
         for entry in entries:

@@ -77,6 +77,11 @@ class HipOps(Ops):
         o.distie_argmax.argtypes = [_P, _P, _I, _I, _P]
         o.distie_sample.argtypes = [_P, _P, _P, _P, _P, _I, _I, _P]
 
+    def graphs_supported(self) -> bool:
+        """Every kernel launches on torch's current stream and keeps its scratch at fixed
+        addresses, so a step can be captured into a HIP graph."""
+        return True
+
     def _stream(self):
         return torch.cuda.current_stream(self.device).cuda_stream
 

@@ -1,0 +1,168 @@
+"""Configuration, registry, weight files and their errors."""
+
+import json
+
+import pytest
+import torch
+
+import plain_qwen2 as plain
+from distie_amd.config import (ConfigError, EngineConfig, Qwen2Config, config_from_dict, known_architectures,
+                               load_model_config, register_architecture)
+from distie_amd.engine.model import Model
+from distie_amd.weights import (SafetensorsFile, WeightsError, kept_dtype, load_into, write_random_model,
+                                write_safetensors)
+from engine_util import make_model_dir
+
+
+def test_qwen2_config_reads_every_key():
+    c = config_from_dict(plain.TINY_B)
+    assert isinstance(c, Qwen2Config)
+    assert (c.num_hidden_layers, c.hidden_size, c.num_attention_heads, c.num_key_value_heads, c.head_dim) == (3, 96, 3, 1, 32)
+    assert (c.intermediate_size, c.vocab_size, c.rope_theta, c.rms_norm_eps) == (250, 323, 1e6, 1e-5)
+    assert c.tie_word_embeddings is False and c.max_position_embeddings == 256
+    assert c.layer_windows == (None, 8, 8)
+    assert c.num_key_value_groups == 3
+    a = config_from_dict(plain.TINY_A)
+    assert a.head_dim == 16 and a.layer_windows == (None, None) and a.tie_word_embeddings
+    assert config_from_dict(plain.TINY_C).layer_windows == (20, None)
+    # rope_parameters wins over rope_theta (worker/src/inference/qwen2/model.py:413-419)
+    assert config_from_dict(dict(plain.TINY_A, rope_parameters={"rope_theta": 5.0})).rope_theta == 5.0
+
+
+@pytest.mark.parametrize("change,message", [
+    ({"num_key_value_heads": 3}, "multiple of num_key_value_heads"),
+    ({"hidden_size": 70}, "hidden_size must equal"),
+    ({"hidden_size": 12, "num_attention_heads": 4, "num_key_value_heads": 2}, "even"),
+    ({"hidden_act": "gelu"}, "silu"),
+    ({"rope_parameters": {"rope_type": "yarn"}}, "RoPE type"),
+    ({"num_hidden_layers": 0}, ">= 1"),
+    ({"layer_types": ["full_attention", "chunked_attention"]}, "unknown layer type"),
+    ({"layer_types": ["full_attention"]}, "entries"),
+    ({"vocab_size": None}, "required key 'vocab_size'"),
+    ({"rms_norm_eps": None}, "rms_norm_eps"),
+    ({"max_position_embeddings": None}, "max_position_embeddings"),
+])
+def test_config_errors(change, message):
+    with pytest.raises(ConfigError, match=message):
+        config_from_dict(dict(plain.TINY_A, **change))
+
+
+def test_registry():
+    assert "Qwen2ForCausalLM" in known_architectures()
+    with pytest.raises(ConfigError, match="unknown architecture 'LlamaForCausalLM'.*Qwen2ForCausalLM"):
+        config_from_dict(dict(plain.TINY_A, architectures=["LlamaForCausalLM"]))
+    with pytest.raises(ConfigError, match="architectures"):
+        config_from_dict({k: v for k, v in plain.TINY_A.items() if k != "architectures"})
+    with pytest.raises(TypeError):
+        register_architecture("X", object)
+
+
+def test_model_spec_has_no_size_in_code():
+    spec = config_from_dict(plain.TINY_B).model_spec()
+    assert [l.mixer.params["window"] for l in spec.layers] == [None, 8, 8]
+    assert spec.layers[0].mixer.params["scale"] == 32 ** -0.5
+    assert spec.layers[2].mixer.prefix == "model.layers.2.self_attn."
+    assert [c.layer for c in spec.order] == [0, 1, 2]
+    names = Model.declare(spec)
+    assert set(names) == set(plain.tensor_shapes(plain.TINY_B))
+    assert {n: tuple(s.shape) for n, s in names.items()} == plain.tensor_shapes(plain.TINY_B)
+
+
+def test_engine_config():
+    assert EngineConfig(dtype="bf16").dtype == "bfloat16"
+    assert EngineConfig(dtype="auto").dtype == "bfloat16"
+    assert EngineConfig(dtype="fp32", max_cache_tokens=130, block_size=16).pages() == 9
+    with pytest.raises(ValueError):
+        EngineConfig(dtype="fp16")
+    with pytest.raises(ValueError):
+        EngineConfig(token_budget=0)
+
+
+def test_safetensors_round_trip_matches_the_library(tmp_path):
+    from safetensors.torch import load_file, save_file
+
+    tensors = {"a": torch.randn(3, 5), "b": torch.randn(7).to(torch.bfloat16), "c": torch.arange(6, dtype=torch.int64).view(2, 3)}
+    write_safetensors(tmp_path / "ours.safetensors", [(n, t.dtype, tuple(t.shape)) for n, t in tensors.items()],
+                      iter(tensors.items()), {"k": "v"})
+    theirs = load_file(str(tmp_path / "ours.safetensors"))
+    for n, t in tensors.items():
+        assert torch.equal(theirs[n], t)
+    save_file(tensors, str(tmp_path / "theirs.safetensors"))
+    f = SafetensorsFile(tmp_path / "theirs.safetensors")
+    assert {n: s for n, (d, s) in f.index.items()} == {"a": (3, 5), "b": (7,), "c": (2, 3)}
+    for n, t in tensors.items():
+        assert torch.equal(f.read(n), t)
+    f.close()
+
+
+def test_kept_precision():
+    bf, f32 = torch.bfloat16, torch.float32
+    assert kept_dtype(bf, bf) == bf and kept_dtype(torch.float16, bf) == bf
+    assert kept_dtype(f32, bf) == f32          # a tensor stored in 32-bit stays so
+    assert kept_dtype(bf, f32) == f32 and kept_dtype(torch.float64, f32) == f32
+    assert kept_dtype(torch.int64, bf) == torch.int32
+
+
+def test_mixed_file_keeps_each_tensors_precision(tmp_path):
+    cfg = plain.TINY_A
+    weights = plain.random_weights(cfg, 1, dtype=torch.bfloat16)
+    for name in weights:
+        if name.endswith("norm.weight"):
+            weights[name] = weights[name].float()
+    plain.write_model_dir(tmp_path / "m", cfg, weights)
+    model = Model(load_model_config(tmp_path / "m").model_spec())
+    load_into(model, tmp_path / "m", "cpu", torch.bfloat16)
+    assert model.embedding.dtype == torch.bfloat16
+    assert model.blocks[0].mixer_norm.weight.dtype == torch.float32
+    assert model.blocks[0].mixer.qkv_weight.dtype == torch.bfloat16
+    assert model.head is model.embedding       # tied: one buffer (worker/tests/test_qwen2.py:52-58)
+
+
+def test_weight_errors_list_everything(tmp_path):
+    cfg = plain.TINY_B
+    weights = plain.random_weights(cfg, 1)
+    del weights["model.layers.1.mlp.up_proj.weight"]
+    del weights["lm_head.weight"]
+    weights["model.layers.0.self_attn.q_proj.bias"] = torch.zeros(5)
+    weights["model.layers.7.extra.weight"] = torch.zeros(2)
+    plain.write_model_dir(tmp_path / "m", cfg, weights)
+    model = Model(load_model_config(tmp_path / "m").model_spec())
+    with pytest.raises(WeightsError) as info:
+        load_into(model, tmp_path / "m", "cpu", torch.float32)
+    err = info.value
+    assert err.missing == ["model.layers.1.mlp.up_proj.weight", "lm_head.weight"]
+    assert err.unexpected == ["model.layers.7.extra.weight"]
+    assert err.wrong_shape == [("model.layers.0.self_attn.q_proj.bias", (5,), (96,))]
+    text = str(err)
+    for piece in ("missing (2)", "unexpected (1)", "wrong shape (1)", "is [5], want [96]"):
+        assert piece in text
+
+
+def test_tied_head_ignores_a_copy_in_the_file(tmp_path):
+    cfg = plain.TINY_A
+    weights = plain.random_weights(cfg, 1)
+    weights["lm_head.weight"] = weights["model.embed_tokens.weight"].clone()
+    plain.write_model_dir(tmp_path / "m", cfg, weights)
+    model = Model(load_model_config(tmp_path / "m").model_spec())
+    load_into(model, tmp_path / "m", "cpu", torch.float32)
+    assert model.head is model.embedding
+
+
+def test_random_weights_mode_writes_a_model_folder(tmp_path):
+    config = config_from_dict(plain.TINY_B)
+    a = write_random_model(config, tmp_path / "a", seed=3, dtype="float32")
+    b = write_random_model(config, tmp_path / "b", seed=3, dtype="bfloat16")
+    c = write_random_model(config, tmp_path / "c", seed=4, dtype="float32")
+    wa, wb, wc = plain.read_weights(a), plain.read_weights(b), plain.read_weights(c)
+    assert {n: tuple(t.shape) for n, t in wa.items()} == plain.tensor_shapes(plain.TINY_B)
+    assert all(torch.equal(wa[n].to(torch.bfloat16), wb[n]) for n in wa)    # same numbers in every precision
+    assert not torch.equal(wa["lm_head.weight"], wc["lm_head.weight"])
+    assert torch.equal(wa["model.norm.weight"], torch.ones(96))
+    assert abs(wa["model.embed_tokens.weight"].std().item() - 0.02) < 0.002
+    assert abs(wa["model.layers.0.self_attn.q_proj.bias"].std().item() - 0.02) < 0.006
+    again = load_model_config(a)
+    assert again == config
+    assert json.loads((b / "config.json").read_text())["torch_dtype"] == "bfloat16"
+    # the plain implementation reads the folder too
+    logits = plain.forward(wa, plain.read_config(a), [1, 2, 3])
+    assert logits.shape == (3, 323)

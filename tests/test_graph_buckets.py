@@ -1,0 +1,23 @@
+"""Bucket sizes of captured decode steps (vectors of worker/tests/test_batch_decode.py:50-62)."""
+
+import pytest
+
+from distie_amd.engine.graphs import bucket_for, decode_buckets
+
+
+def test_decode_buckets():
+    assert decode_buckets(32) == (1, 2, 4, 8, 16, 24, 32)
+    assert decode_buckets(64) == (1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64)
+    assert decode_buckets(5) == (1, 2, 4, 5)
+    assert decode_buckets(1) == (1,)
+    with pytest.raises(ValueError):
+        decode_buckets(0)
+
+
+def test_bucket_for():
+    buckets = decode_buckets(32)
+    assert [bucket_for(buckets, n) for n in (1, 3, 8, 9, 17, 32)] == [1, 4, 8, 16, 24, 32]
+    with pytest.raises(ValueError):
+        bucket_for(buckets, 33)
+    with pytest.raises(ValueError):
+        bucket_for(buckets, 0)

@@ -1,0 +1,144 @@
+"""The entry point end to end on the CPU test double: greedy generation against the plain
+implementation, concurrent == sequential, a tight pool with preemption == a roomy one,
+cancel, a failing step, trace (worker/tests/test_batched_engine.py:85-144,
+worker/tests/test_torch_engine.py:100-130)."""
+
+import pytest
+import torch
+
+import plain_qwen2 as plain
+from distie_amd import LLM, SamplingParams
+from engine_util import make_model_dir, oracle, random_ids
+from torch_ops import TorchOps
+
+
+def plain_greedy(weights, cfg, prompt, n):
+    ids = list(prompt)
+    for _ in range(n):
+        ids.append(int(oracle(weights, cfg, ids)[-1].argmax()))
+    return ids[len(prompt):]
+
+
+@pytest.fixture(scope="module")
+def tiny(tmp_path_factory):
+    cfg = plain.TINY_B
+    folder, weights = make_model_dir(tmp_path_factory.mktemp("llm"), cfg, seed=21)
+    return cfg, folder, weights
+
+
+def engine(folder, **options):
+    options.setdefault("block_size", 8)
+    options.setdefault("num_blocks", 64)
+    return LLM(folder, dtype="fp32", ops=TorchOps(), **options)
+
+
+def test_greedy_generation_matches_the_plain_implementation(tiny):
+    cfg, folder, weights = tiny
+    llm = engine(folder, token_budget=7)      # prompts of 9, 23 and 40 are cut into portions of <= 7
+    prompts = [random_ids(cfg, n, 30 + n) for n in (1, 9, 23, 40)]
+    outs = llm.generate(prompts, SamplingParams(max_new_tokens=12))
+    for prompt, out in zip(prompts, outs):
+        assert out.token_ids == plain_greedy(weights, cfg, prompt, 12)
+        assert out.finished and out.finish_reason == "length"
+        assert out.time_to_first_token_ms > 0 and out.total_latency_ms >= out.time_to_first_token_ms
+    llm.cache.check()
+    assert llm.cache.free_pages() == [64, 64]
+
+
+def test_concurrent_equals_sequential_and_a_tight_pool_preempts_yet_agrees(tiny):
+    cfg, folder, weights = tiny
+    prompts = [random_ids(cfg, n, 50 + n) for n in (5, 11, 17, 8)]
+    params = SamplingParams(max_new_tokens=10)
+    together = [o.token_ids for o in engine(folder).generate(prompts, params)]
+    one = engine(folder)
+    alone = [one.generate([p], params)[0].token_ids for p in prompts]
+    assert together == alone
+    tight = engine(folder, num_blocks=8)      # 8 pages of 8 tokens for four requests of up to 27 tokens
+    outs = tight.generate(prompts, params)
+    assert [o.token_ids for o in outs] == together
+    assert sum(o.preemptions for o in outs) > 0
+    tight.cache.check()
+    assert tight.cache.free_pages() == [8, 8]
+
+
+def test_temperature_sampling_is_repeatable_and_depends_on_the_seed(tiny):
+    cfg, folder, _ = tiny
+    prompts = [random_ids(cfg, 6, 1), random_ids(cfg, 9, 2)]
+    a = engine(folder).generate(prompts, SamplingParams(max_new_tokens=12, temperature=0.7, seed=5))
+    b = engine(folder).generate(list(reversed(prompts)), SamplingParams(max_new_tokens=12, temperature=0.7, seed=5))
+    c = engine(folder).generate(prompts, SamplingParams(max_new_tokens=12, temperature=0.7, seed=6))
+    assert [o.token_ids for o in a] == [o.token_ids for o in reversed(b)]      # not a matter of batch order
+    assert [o.token_ids for o in a] != [o.token_ids for o in c]
+    greedy = engine(folder).generate(prompts, SamplingParams(max_new_tokens=12))
+    assert [o.token_ids for o in a] != [o.token_ids for o in greedy]
+
+
+def test_eos_stops_and_is_emitted(tiny):
+    cfg, folder, weights = tiny
+    prompt = random_ids(cfg, 7, 3)
+    want = plain_greedy(weights, cfg, prompt, 6)
+    out = engine(folder).generate([prompt], SamplingParams(max_new_tokens=6, eos_id=want[2]))[0]
+    assert out.token_ids == want[:3] and out.finish_reason == "stop"
+    out = engine(folder).generate([prompt], SamplingParams(max_new_tokens=6, eos_id=want[2], ignore_eos=True))[0]
+    assert out.token_ids == want
+
+
+def test_cancel_frees_blocks(tiny):
+    cfg, folder, _ = tiny
+    llm = engine(folder)
+    a = llm.add_request(random_ids(cfg, 9, 4), SamplingParams(max_new_tokens=50))
+    b = llm.add_request(random_ids(cfg, 5, 5), SamplingParams(max_new_tokens=4))
+    llm.run_step()
+    llm.abort(a)
+    while llm.has_work():
+        llm.run_step()
+    assert llm._outputs[a].finish_reason == "abort" and len(llm._outputs[a].token_ids) == 1
+    assert llm._outputs[b].finish_reason == "length"
+    assert llm.cache.free_pages() == [64, 64] and llm.cache.slots.num_free == llm.cache.num_slots
+
+
+def test_request_larger_than_the_pool(tiny):
+    cfg, folder, _ = tiny
+    llm = engine(folder, num_blocks=2)
+    with pytest.raises(RuntimeError, match="out of KV blocks"):
+        llm.generate([random_ids(cfg, 30, 6)], SamplingParams(max_new_tokens=4))
+
+
+def test_a_failing_step_reaches_its_requests_and_frees(tiny):
+    cfg, folder, _ = tiny
+    llm = engine(folder)
+    calls = {"n": 0}
+    real = llm.ops.silu_mul
+
+    def flaky(x):
+        calls["n"] += 1
+        if calls["n"] == 4:
+            raise RuntimeError("injected kernel failure")
+        return real(x)
+
+    llm.ops.silu_mul = flaky
+    outs = llm.generate([random_ids(cfg, 4, 7)], SamplingParams(max_new_tokens=5))
+    assert outs[0].finish_reason == "error" and "injected" in outs[0].error
+    assert llm.cache.free_pages() == [64, 64]
+    llm.ops.silu_mul = real
+    assert llm.generate([random_ids(cfg, 4, 7)], SamplingParams(max_new_tokens=2))[0].finish_reason == "length"
+
+
+def test_trace_free_running_and_forced(tiny):
+    cfg, folder, weights = tiny
+    llm = engine(folder)
+    prompt = random_ids(cfg, 8, 8)
+    want = plain_greedy(weights, cfg, prompt, 5)
+    trace = llm.trace(prompt, 5)
+    assert trace.token_ids == want and trace.logits.shape == (5, cfg["vocab_size"])
+    full = oracle(weights, cfg, prompt + want)
+    assert (trace.logits - full[len(prompt) - 1:len(prompt) + 4]).abs().max() < 1e-4
+    forced = [3, 1, 4, 1, 5]
+    trace = llm.trace(prompt, 5, forced_ids=forced)
+    full = oracle(weights, cfg, prompt + forced)
+    assert (trace.logits - full[len(prompt) - 1:len(prompt) + 4]).abs().max() < 1e-4
+    with pytest.raises(ValueError):
+        llm.trace([], 3)
+    with pytest.raises(ValueError):
+        llm.trace(prompt, 3, forced_ids=[1])
+    assert llm.cache.free_pages() == [64, 64]

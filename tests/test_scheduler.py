@@ -1,0 +1,237 @@
+"""The scheduler's decisions, with the real cache manager (no slabs) and no model.
+The sequences of plans restate worker/tests/test_scheduler.py:29-182, adapted where this
+scheduler cuts prompts (the reference never does)."""
+
+import pytest
+
+from distie_amd.cache import CacheManager
+from distie_amd.engine.scheduler import BlockPoolExhausted, Scheduler, Sequence, SeqState
+from distie_amd.parts import PagedKV
+from distie_amd.sampling import SamplingParams
+
+EOS = 99
+
+
+def make(pages, block=4, max_seqs=32, budget=2048, window=None, slots=8, max_model_len=None):
+    needs = [PagedKV(1, 16), PagedKV(1, 16, window)] if window else [PagedKV(1, 16)]
+    cache = CacheManager(needs, block, pages, slots, allocate=False)
+    return Scheduler(cache, max_seqs, budget, max_model_len), cache
+
+
+def seq(rid, prompt_len, max_new=8):
+    return Sequence(request_id=rid, prompt_ids=list(range(1, prompt_len + 1)),
+                    params=SamplingParams(max_new_tokens=max_new), eos_ids=(EOS,))
+
+
+def run(sched, cache, tokens):
+    """schedule, pretend the step ran (the step function advances the cache's counts), complete"""
+    plan = sched.schedule()
+    for item in plan.items:
+        cache.commit(item.seq.request_id, len(item.token_ids))
+    picks = [tokens if isinstance(tokens, int) else tokens[i] for i in range(len(plan.items))]
+    return plan, sched.complete(plan, picks)
+
+
+def names(plan):
+    return [i.seq.request_id for i in plan.items]
+
+
+def test_fifo_and_prefill_then_decode():
+    sched, cache = make(8)
+    a, b = seq("a", 5), seq("b", 2)
+    sched.submit(a)
+    sched.submit(b)
+    plan = sched.schedule()
+    assert names(plan) == ["a", "b"]
+    assert [len(i.token_ids) for i in plan.items] == [5, 2]
+    assert [i.past_len for i in plan.items] == [0, 0]
+    assert all(i.samples for i in plan.items)
+    assert len(cache.request("a").tables[0]) == 2
+    for i in plan.items:
+        cache.commit(i.seq.request_id, len(i.token_ids))
+    sched.complete(plan, [7, 8])
+    plan = sched.schedule()
+    assert [(i.token_ids, i.past_len) for i in plan.items] == [([7], 5), ([8], 2)]
+    assert plan.is_decode
+
+
+def test_max_seqs_and_token_budget_cut_prompts():
+    sched, cache = make(16, max_seqs=2, budget=6)
+    for rid in ("a", "b", "c"):
+        sched.submit(seq(rid, 4))
+    plan, _ = run(sched, cache, 7)
+    # a whole, b's first two tokens: the budget of 6 is filled, b does not sample yet
+    assert [(i.seq.request_id, i.token_ids, i.samples) for i in plan.items] == [("a", [1, 2, 3, 4], True), ("b", [1, 2], False)]
+    assert sched._ids["b"].output_ids == []
+    plan, _ = run(sched, cache, 7)
+    # decoding first, then the prompt in flight
+    assert [(i.seq.request_id, i.token_ids, i.past_len, i.samples) for i in plan.items] == \
+        [("a", [7], 4, True), ("b", [3, 4], 2, True)]
+    plan, _ = run(sched, cache, 7)
+    assert names(plan) == ["a", "b"] and sched.num_waiting == 1      # max_seqs keeps c waiting
+
+
+def test_long_prompt_is_cut_under_the_budget():
+    sched, cache = make(16, budget=4)
+    sched.submit(seq("a", 10))
+    sizes = []
+    for _ in range(3):
+        plan, out = run(sched, cache, 7)
+        sizes.append((plan.num_tokens, plan.items[0].past_len, plan.items[0].samples))
+    assert sizes == [(4, 0, False), (4, 4, False), (2, 8, True)]
+    assert out[0].token_id == 7
+    assert all(p.num_tokens <= 4 for p in [plan])
+
+
+def test_every_step_stays_within_the_budget_and_decodes_come_first():
+    sched, cache = make(64, budget=8)
+    sched.submit(seq("a", 3, max_new=20))
+    run(sched, cache, 7)
+    sched.submit(seq("b", 30, max_new=2))
+    for _ in range(6):
+        plan, _ = run(sched, cache, 7)
+        assert plan.num_tokens <= 8
+        assert plan.items[0].seq.request_id == "a" and len(plan.items[0].token_ids) == 1
+
+
+def test_waits_for_blocks():
+    sched, cache = make(2)
+    sched.submit(seq("a", 7, max_new=1))
+    sched.submit(seq("b", 4, max_new=2))
+    plan = sched.schedule()
+    assert names(plan) == ["a"] and cache.free_pages() == [0]
+    cache.commit("a", 7)
+    emitted = sched.complete(plan, [7])
+    assert emitted[0].finished and emitted[0].seq.finish_reason == "length"
+    assert names(sched.schedule()) == ["b"]
+
+
+def test_request_that_can_never_fit_is_refused():
+    sched, _ = make(2)
+    with pytest.raises(BlockPoolExhausted):
+        sched.submit(seq("a", 6, max_new=4))
+    sched2, _ = make(100, max_model_len=12)
+    with pytest.raises(ValueError, match="model length"):
+        sched2.submit(seq("a", 6, max_new=7))
+
+
+def test_rejects_duplicate_and_empty():
+    sched, _ = make(4)
+    sched.submit(seq("a", 2))
+    with pytest.raises(ValueError):
+        sched.submit(seq("a", 2))
+    with pytest.raises(ValueError):
+        sched.submit(Sequence(request_id="b", prompt_ids=[]))
+
+
+def test_eos_and_cap_free_blocks():
+    sched, cache = make(4)
+    sched.submit(seq("a", 2, max_new=5))
+    sched.submit(seq("b", 2, max_new=1))
+    plan, emitted = run(sched, cache, [EOS, 3])
+    assert [(e.seq.request_id, e.finished, e.seq.finish_reason) for e in emitted] == \
+        [("a", True, "stop"), ("b", True, "length")]
+    assert cache.free_pages() == [4] and cache.slots.num_free == 8
+    assert not sched.has_work()
+
+
+def test_ignore_eos():
+    sched, cache = make(4)
+    s = Sequence("a", [1, 2], SamplingParams(max_new_tokens=3, ignore_eos=True), eos_ids=(EOS,))
+    sched.submit(s)
+    _, emitted = run(sched, cache, EOS)
+    assert not emitted[0].finished
+
+
+def test_newest_is_preempted_and_recomputed_without_reemitting():
+    sched, cache = make(2)
+    a, b = seq("a", 3, max_new=4), seq("b", 3, max_new=4)
+    sched.submit(a)
+    sched.submit(b)
+    run(sched, cache, [10, 20])
+    run(sched, cache, [11, 21])       # 5 tokens each: page 1 is full
+    plan = sched.schedule()
+    # a needs a second page; the pool is empty, so b (newest) is preempted
+    assert names(plan) == ["a"]
+    assert b.state is SeqState.WAITING and "b" not in cache
+    assert b.output_ids == [20, 21] and b.preemptions == 1 and b.num_computed == 0
+    cache.commit("a", 1)
+    assert [e.token_id for e in sched.complete(plan, [12])] == [12]
+    cache.check()
+
+
+def test_recompute_prefills_prompt_plus_output():
+    sched, cache = make(3)
+    a, b = seq("a", 3, max_new=2), seq("b", 3)
+    sched.submit(a)
+    sched.submit(b)
+    run(sched, cache, [10, 20])
+    plan, _ = run(sched, cache, [11, 21])     # a finishes on the cap and frees its pages
+    assert len(plan.items) == 2 and cache.free_pages() == [2]
+    sched._preempt(b)
+    item = sched.schedule().items[0]
+    assert (item.seq.request_id, item.token_ids, item.past_len, item.samples) == ("b", [1, 2, 3, 20, 21], 0, True)
+
+
+def test_queue_front_after_preemption_and_no_readmission_in_that_step():
+    sched, cache = make(2)
+    for rid in ("a", "b"):
+        sched.submit(seq(rid, 3, max_new=4))
+    run(sched, cache, [1, 2])
+    run(sched, cache, [1, 2])
+    sched.submit(seq("c", 1, max_new=4))
+    plan = sched.schedule()
+    assert names(plan) == ["a"]
+    assert [s.request_id for s in sched._waiting] == ["b", "c"]
+
+
+def test_needy_request_preempts_itself_when_it_is_the_newest():
+    sched, cache = make(3)
+    a, b = seq("a", 4, max_new=8), seq("b", 4, max_new=8)
+    sched.submit(a)
+    sched.submit(b)
+    run(sched, cache, 5)                      # one page each, one page free
+    plan = sched.schedule()
+    # both need a second page: a (older) takes the free one, b is the newest and goes itself
+    assert names(plan) == ["a"] and sched._waiting[0] is b and b.preemptions == 1
+    assert cache.free_pages() == [1]
+    cache.check()
+
+
+def test_abort_running_frees_on_next_schedule():
+    sched, cache = make(4)
+    sched.submit(seq("a", 2))
+    plan = sched.schedule()
+    sched.abort("a")
+    cache.commit("a", 2)
+    assert sched.complete(plan, [5]) == []        # aborted in flight: nothing emitted
+    assert sched.schedule().items == ()
+    assert cache.free_pages() == [4] and not sched.has_work()
+
+
+def test_abort_waiting_and_unknown():
+    sched, cache = make(1)
+    sched.submit(seq("a", 3, max_new=1))
+    sched.submit(seq("b", 3, max_new=1))
+    sched.abort("b")
+    sched.abort("missing")
+    assert names(sched.schedule()) == ["a"] and sched.num_waiting == 0
+
+
+def test_failed_step_ends_its_requests_and_frees():
+    sched, cache = make(4)
+    sched.submit(seq("a", 2))
+    plan = sched.schedule()
+    failed = sched.fail(plan, RuntimeError("boom"))
+    assert [s.request_id for s in failed] == ["a"] and failed[0].finish_reason == "error"
+    assert cache.free_pages() == [4] and not sched.has_work()
+
+
+def test_windowed_group_lets_long_requests_decode_in_few_pages():
+    sched, cache = make(8, block=4, window=4, budget=8)
+    sched.submit(seq("a", 6, max_new=20))
+    for _ in range(15):
+        run(sched, cache, 7)
+        cache.check()
+    full, windowed = cache.free_pages()
+    assert full == 8 - 5 and windowed >= 8 - 2      # 20 cached: 5 pages in full, at most 2 in the window group

@@ -1,0 +1,134 @@
+"""bin/trace_run as a user drives it: a subprocess, steps on standard input, logits in files;
+and greedy generation through the entry point and the command line."""
+
+import json
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen2 as plain
+from engine_util import check_logits, make_model_dir, oracle, random_ids
+
+pytestmark = pytest.mark.gpu
+ROOT = Path(__file__).resolve().parents[1]
+
+
+class Replay:
+    def __init__(self, model, dtype, out, max_tokens):
+        self.out = Path(out)
+        self.proc = subprocess.Popen(
+            [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(model), "--dtype", dtype,
+             "--out", str(out), "--max-tokens", str(max_tokens)],
+            stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+        self.step = 0
+
+    def run(self, entries, end=()):
+        record = {"step": self.step, "entries": entries, "end": list(end)}
+        self.proc.stdin.write(json.dumps(record) + "\n")
+        self.proc.stdin.flush()
+        line = self.proc.stdout.readline().strip()
+        assert line == f"done {self.step}", line
+        path = self.out / f"{self.step}.f32"
+        self.step += 1
+        wanted = sum(len(e["want"]) for e in entries)
+        if not wanted:
+            assert not path.exists()
+            return None
+        data = np.fromfile(path, dtype="<f4")
+        return torch.from_numpy(data.reshape(wanted, -1))
+
+    def close(self):
+        self.proc.stdin.close()
+        assert self.proc.wait(timeout=60) == 0
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("B", "bfloat16"), ("C", "bfloat16")])
+def test_replay_mixed_trace(tmp_path, name, dtype):
+    cfg = {"A": plain.TINY_A, "B": plain.TINY_B, "C": plain.TINY_C}[name]
+    tdtype = getattr(torch, dtype)
+    folder, weights = make_model_dir(tmp_path, cfg, seed=31, dtype=tdtype)
+    lengths = {"p": 100, "q": 64, "r": 37, "s": 90, "t": 50}
+    reqs = {r: random_ids(cfg, n, 40 + n) for r, n in lengths.items()}
+    # four live at most: the largest four, each rounded up to 64
+    max_tokens = sum(-(-n // 64) * 64 for n in sorted(lengths.values())[-4:])
+    replay = Replay(folder, dtype, tmp_path / "out", max_tokens)
+    got = {r: [] for r in reqs}
+    at = {r: 0 for r in reqs}
+    waiting, live = list(reqs), []
+    gen = torch.Generator().manual_seed(9)
+    while waiting or live:
+        while waiting and len(live) < 4:
+            live.append(waiting.pop(0))
+        entries = []
+        for r in live:
+            left = len(reqs[r]) - at[r]
+            n = 1 if left <= 32 else min(left - 32, int(torch.randint(2, 30, (1,), generator=gen)))
+            want = list(range(n)) if r != "q" else [n - 1]
+            entries.append({"id": r, "tokens": reqs[r][at[r]:at[r] + n], "want": want})
+        logits = replay.run(entries, end=[e["id"] for e in entries if at[e["id"]] + len(e["tokens"]) == len(reqs[e["id"]])])
+        row = 0
+        for e in entries:
+            r, n = e["id"], len(e["tokens"])
+            got[r].append((at[r], e["want"], logits[row:row + len(e["want"])]))
+            row += len(e["want"])
+            at[r] += n
+        live = [r for r in live if at[r] < len(reqs[r])]
+    replay.close()
+    for r, pieces in got.items():
+        want_all = oracle(weights, cfg, reqs[r])
+        rows = [begin + w for begin, want, _ in pieces for w in want]
+        stacked = torch.cat([l for _, _, l in pieces])
+        # compare at the rows that were asked for
+        class _Sel:
+            pass
+        diff = (stacked - want_all[rows]).abs().max().item()
+        scale = want_all.abs().max().item()
+        assert diff < (1e-4 if dtype == "float32" else scale / 16), (r, diff)
+
+
+def test_replay_step_without_wanted_rows_and_a_pause(tmp_path):
+    cfg = plain.TINY_A
+    folder, weights = make_model_dir(tmp_path, cfg, seed=32)
+    ids = random_ids(cfg, 20, 1)
+    other = random_ids(cfg, 6, 2)
+    replay = Replay(folder, "float32", tmp_path / "out", 128)
+    assert replay.run([{"id": "a", "tokens": ids[:7], "want": []}]) is None
+    replay.run([{"id": "b", "tokens": other, "want": [5]}], end=["b"])          # a sits out
+    logits = replay.run([{"id": "a", "tokens": ids[7:], "want": [0, 12]}], end=["a"])
+    replay.close()
+    want = oracle(weights, cfg, ids)
+    assert (logits - want[[7, 19]]).abs().max() < 1e-4
+
+
+def test_generation_through_the_entry_point_and_the_command_line(tmp_path):
+    from distie_amd import LLM, SamplingParams
+
+    cfg = plain.TINY_B
+    folder, weights = make_model_dir(tmp_path, cfg, seed=33)
+    prompts = [random_ids(cfg, n, 60 + n) for n in (1, 9, 23, 40)]
+
+    def greedy(prompt, n):
+        ids = list(prompt)
+        for _ in range(n):
+            ids.append(int(oracle(weights, cfg, ids)[-1].argmax()))
+        return ids[len(prompt):]
+
+    want = [greedy(p, 12) for p in prompts]
+    for graphs in (False, True):
+        llm = LLM(folder, dtype="fp32", block_size=8, num_blocks=32, token_budget=7, use_graphs=graphs)
+        outs = llm.generate(prompts, SamplingParams(max_new_tokens=12))
+        assert [o.token_ids for o in outs] == want, f"graphs={graphs}"
+        llm.cache.check()
+    (tmp_path / "prompts.json").write_text(json.dumps(prompts))
+    done = subprocess.run(
+        [sys.executable, "-m", "distie_amd.cli", "generate", "--model", str(folder), "--dtype", "fp32",
+         "--prompts", str(tmp_path / "prompts.json"), "--max-new-tokens", "12", "--block-size", "8",
+         "--num-blocks", "32", "--token-budget", "7", "--out", str(tmp_path / "report.json")],
+        cwd=str(ROOT), capture_output=True, text=True, timeout=110)
+    assert done.returncode == 0, done.stderr
+    report = json.loads((tmp_path / "report.json").read_text())
+    assert [r["token_ids"] for r in report] == want
