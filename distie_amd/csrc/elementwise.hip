@@ -34,10 +34,12 @@ extern "C" int distie_embed(const int32_t* ids, const void* table, int table_dty
 
 // ---------------------------------------------------------------- RMS norm
 // One block per row. With `delta`, the row of the residual stream is first updated
-// (residual += delta, float32) and then normed: one pass less over the activations.
+// (residual += delta, float32) and then normed: one pass less over the activations. `delta` may be
+// `slices` partial sums laid side by side (`slice_stride` elements apart); they are added in order.
 template <typename D, typename W, typename O>
-__global__ void rmsnorm_kernel(float* __restrict__ residual, const D* __restrict__ delta,
-                               const W* __restrict__ weight, O* __restrict__ out, int width, float eps) {
+__global__ void rmsnorm_kernel(float* __restrict__ residual, const D* __restrict__ delta, int slices,
+                               int64_t slice_stride, const W* __restrict__ weight, O* __restrict__ out,
+                               int width, float eps) {
   __shared__ float scratch[16];
   const int64_t row = blockIdx.x;
   float* x = residual + row * width;
@@ -45,7 +47,9 @@ __global__ void rmsnorm_kernel(float* __restrict__ residual, const D* __restrict
   if (delta != nullptr) {
     const D* d = delta + row * width;
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
-      const float v = x[i] + to_float(d[i]);
+      float sum = to_float(d[i]);
+      for (int s = 1; s < slices; ++s) sum += to_float(d[s * slice_stride + i]);
+      const float v = x[i] + sum;
       x[i] = v;
       ss += v * v;
     }
@@ -63,52 +67,78 @@ __global__ void rmsnorm_kernel(float* __restrict__ residual, const D* __restrict
 }
 
 template <typename D, typename W>
-static int rmsnorm_launch_out(float* residual, const D* delta, const W* weight, void* out, int out_dtype,
-                              int rows, int width, float eps, hipStream_t stream) {
+static int rmsnorm_launch_out(float* residual, const D* delta, int slices, const W* weight, void* out,
+                              int out_dtype, int rows, int width, float eps, hipStream_t stream) {
   const int threads = width >= 2048 ? 512 : (width >= 512 ? 256 : 64);
   DISTIE_DISPATCH(out_dtype, O,
-                  rmsnorm_kernel<D, W, O><<<rows, threads, 0, stream>>>(residual, delta, weight, static_cast<O*>(out), width, eps));
+                  rmsnorm_kernel<D, W, O><<<rows, threads, 0, stream>>>(
+                      residual, delta, slices, static_cast<int64_t>(rows) * width, weight, static_cast<O*>(out), width, eps));
   return launch_status();
 }
 
-extern "C" int distie_rmsnorm(float* residual, const void* delta, int delta_dtype, const void* weight,
+// delta: null, or [slices, rows, width] of delta_dtype
+extern "C" int distie_rmsnorm(float* residual, const void* delta, int delta_dtype, int slices, const void* weight,
                               int weight_dtype, void* out, int out_dtype, int rows, int width, float eps,
                               hipStream_t stream) {
   if (rows <= 0) return 0;
-  if (width <= 0) return DISTIE_BAD_ARGUMENT;
+  if (width <= 0 || slices < 1) return DISTIE_BAD_ARGUMENT;
   DISTIE_DISPATCH(weight_dtype, W, DISTIE_DISPATCH(delta_dtype, D, return rmsnorm_launch_out<D, W>(
-      residual, static_cast<const D*>(delta), static_cast<const W*>(weight), out, out_dtype, rows, width, eps, stream)));
+      residual, static_cast<const D*>(delta), slices, static_cast<const W*>(weight), out, out_dtype, rows, width, eps,
+      stream)));
   return DISTIE_BAD_ARGUMENT;
 }
 
 // ---------------------------------------------------------------- rotation + cache write
-// qkv: [T, (H + 2 KH) * D]. One block per token. Pair (j, j + R/2) of every q and k head is turned by
-// angle = float(position) * inv_freq[j] (R = 2 * pairs <= D is the rotated width). The turned k and the
-// v of the token go to the cache [pages, KH, P, D] at the token's slot (slot = page * P + offset).
-template <typename T, typename C>
-__global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,
-                                     const int32_t* __restrict__ slots, C* __restrict__ k_cache,
-                                     C* __restrict__ v_cache, const float* __restrict__ inv_freq, int pairs,
-                                     int heads, int kv_heads, int dim, int block_size, int write) {
+// in: [slices, T, (H + 2 KH) * D] (partial sums of the q/k/v product, added in order; one slice for a
+// finished product), out: [T, (H + 2 KH) * D], which may be `in` itself. One block per token. Pair
+// (j, j + R/2) of every q and k head is turned by angle = float(position) * inv_freq[j] (R = 2 * pairs <= D
+// is the rotated width). The turned k and the v of the token go to the cache [pages, KH, P, D] at the
+// token's slot (slot = page * P + offset).
+template <typename I, typename T, typename C>
+__global__ void rope_kv_write_kernel(const I* in, int slices, int64_t slice_stride, T* out,
+                                     const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
+                                     C* __restrict__ k_cache, C* __restrict__ v_cache,
+                                     const float* __restrict__ inv_freq, int pairs, int heads, int kv_heads, int dim,
+                                     int block_size, int write) {
   const int64_t t = blockIdx.x;
-  T* row = qkv + t * static_cast<int64_t>(heads + 2 * kv_heads) * dim;
+  const int64_t width = static_cast<int64_t>(heads + 2 * kv_heads) * dim;
+  const I* src = in + t * width;
+  T* row = out + t * width;
   const float pos = static_cast<float>(positions[t]);
   const int64_t slot = write ? slots[t] : 0;
   const int64_t page = slot / block_size;
   const int offset = static_cast<int>(slot % block_size);
+  auto value = [&](int64_t i) {
+    float sum = to_float(src[i]);
+    for (int s = 1; s < slices; ++s) sum += to_float(src[s * slice_stride + i]);
+    return sum;
+  };
+  // q and k heads: every thread owns whole pairs, so `out` may alias `in`
   const int rotated_heads = heads + kv_heads;
-  if (pairs > 0) {
-    for (int i = threadIdx.x; i < rotated_heads * pairs; i += blockDim.x) {
-      const int head = i / pairs;
-      const int j = i % pairs;
-      float s, c;
-      sincosf(pos * inv_freq[j], &s, &c);
-      T* h = row + head * dim;
-      const float a = to_float(h[j]);
-      const float b = to_float(h[j + pairs]);
-      h[j] = from_float<T>(a * c - b * s);
-      h[j + pairs] = from_float<T>(b * c + a * s);
+  const int half = dim / 2;
+  for (int i = threadIdx.x; i < rotated_heads * half; i += blockDim.x) {
+    const int head = i / half;
+    const int j = i % half;
+    const int64_t lo = static_cast<int64_t>(head) * dim + j;
+    float a, b;
+    if (j < pairs) {
+      // pair (j, j + pairs)
+      const float x0 = value(lo), x1 = value(lo + pairs);
+      float sn, cs;
+      sincosf(pos * inv_freq[j], &sn, &cs);
+      a = x0 * cs - x1 * sn;
+      b = x1 * cs + x0 * sn;
+      row[lo] = from_float<T>(a);
+      row[lo + pairs] = from_float<T>(b);
     }
+  }
+  // columns of q and k beyond the rotated width, and v: copied
+  const int rot = 2 * pairs;
+  for (int64_t i = threadIdx.x; i < width; i += blockDim.x) {
+    const int head = static_cast<int>(i / dim);
+    const int d = static_cast<int>(i % dim);
+    if (head < rotated_heads && d < rot) continue;
+    row[i] = from_float<T>(value(i));
   }
   if (!write) return;
   __syncthreads();
@@ -121,44 +151,76 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restr
   }
 }
 
-extern "C" int distie_rope_kv_write(void* qkv, int dtype, const int32_t* positions, const int32_t* slots,
-                                    void* k_cache, void* v_cache, int cache_dtype, const float* inv_freq,
-                                    int pairs, int tokens, int heads, int kv_heads, int dim, int block_size,
-                                    int write, hipStream_t stream) {
+extern "C" int distie_rope_kv_write(const void* in, int in_dtype, int slices, void* out, int dtype,
+                                    const int32_t* positions, const int32_t* slots, void* k_cache, void* v_cache,
+                                    int cache_dtype, const float* inv_freq, int pairs, int tokens, int heads,
+                                    int kv_heads, int dim, int block_size, int write, hipStream_t stream) {
   if (tokens <= 0) return 0;
-  if (heads < 1 || kv_heads < 1 || dim < 1 || block_size < 1 || 2 * pairs > dim || pairs < 0) return DISTIE_BAD_ARGUMENT;
+  if (heads < 1 || kv_heads < 1 || dim < 1 || block_size < 1 || 2 * pairs > dim || pairs < 0 || slices < 1)
+    return DISTIE_BAD_ARGUMENT;
   if (pairs > 0 && inv_freq == nullptr) return DISTIE_BAD_ARGUMENT;
-  const int work = (heads + kv_heads) * (pairs > 0 ? pairs : 1);
+  if (in == out && (slices != 1 || in_dtype != dtype)) return DISTIE_BAD_ARGUMENT;
+  const int work = (heads + kv_heads) * dim / 2;
   const int threads = work >= 512 ? 256 : (work >= 128 ? 128 : 64);
-  DISTIE_DISPATCH(dtype, T, DISTIE_DISPATCH(cache_dtype, C,
-      rope_kv_write_kernel<T, C><<<tokens, threads, 0, stream>>>(
-          static_cast<T*>(qkv), positions, slots, static_cast<C*>(k_cache), static_cast<C*>(v_cache), inv_freq,
-          pairs, heads, kv_heads, dim, block_size, write)));
+  const int64_t stride = static_cast<int64_t>(tokens) * (heads + 2 * kv_heads) * dim;
+  DISTIE_DISPATCH(in_dtype, I, DISTIE_DISPATCH(dtype, T, DISTIE_DISPATCH(cache_dtype, C,
+      rope_kv_write_kernel<I, T, C><<<tokens, threads, 0, stream>>>(
+          static_cast<const I*>(in), slices, stride, static_cast<T*>(out), positions, slots,
+          static_cast<C*>(k_cache), static_cast<C*>(v_cache), inv_freq, pairs, heads, kv_heads, dim, block_size,
+          write))));
   return launch_status();
 }
 
 // ---------------------------------------------------------------- gated activation
-template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int64_t rows, int inter) {
+// gate_up: [slices, rows, 2 * inter] (partial sums added in order) -> out [rows, inter]
+template <typename I, typename T>
+__global__ void silu_mul_kernel(const I* __restrict__ gate_up, int slices, int64_t slice_stride, T* __restrict__ out,
+                                int64_t rows, int inter) {
   const int64_t total = rows * inter;
   for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
        i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
     const int64_t r = i / inter;
     const int c = static_cast<int>(i % inter);
-    const float g = to_float(gate_up[r * 2 * inter + c]);
-    const float u = to_float(gate_up[r * 2 * inter + inter + c]);
+    const I* p = gate_up + r * 2 * inter + c;
+    float g = to_float(p[0]);
+    float u = to_float(p[inter]);
+    for (int s = 1; s < slices; ++s) {
+      g += to_float(p[s * slice_stride]);
+      u += to_float(p[s * slice_stride + inter]);
+    }
     out[i] = from_float<T>(g / (1.f + expf(-g)) * u);
   }
 }
 
-extern "C" int distie_silu_mul(const void* gate_up, void* out, int dtype, int rows, int inter, hipStream_t stream) {
+extern "C" int distie_silu_mul(const void* gate_up, int in_dtype, int slices, void* out, int dtype, int rows,
+                               int inter, hipStream_t stream) {
   if (rows <= 0) return 0;
-  if (inter <= 0) return DISTIE_BAD_ARGUMENT;
+  if (inter <= 0 || slices < 1) return DISTIE_BAD_ARGUMENT;
   const int64_t total = static_cast<int64_t>(rows) * inter;
   const int threads = 256;
   const int blocks = static_cast<int>(total / threads + 1 < 16384 ? total / threads + 1 : 16384);
-  DISTIE_DISPATCH(dtype, T, silu_mul_kernel<T><<<blocks, threads, 0, stream>>>(
-                                static_cast<const T*>(gate_up), static_cast<T*>(out), rows, inter));
+  DISTIE_DISPATCH(in_dtype, I, DISTIE_DISPATCH(dtype, T, silu_mul_kernel<I, T><<<blocks, threads, 0, stream>>>(
+      static_cast<const I*>(gate_up), slices, 2 * total, static_cast<T*>(out), rows, inter)));
+  return launch_status();
+}
+
+// ---------------------------------------------------------------- sum of partial slices
+template <typename T>
+__global__ void sum_slices_kernel(const float* __restrict__ in, int slices, int64_t count, T* __restrict__ out) {
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < count;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    float sum = in[i];
+    for (int s = 1; s < slices; ++s) sum += in[s * count + i];
+    out[i] = from_float<T>(sum);
+  }
+}
+
+extern "C" int distie_sum_slices(const float* in, int slices, int64_t count, void* out, int dtype,
+                                 hipStream_t stream) {
+  if (count <= 0) return 0;
+  if (slices < 1) return DISTIE_BAD_ARGUMENT;
+  const int blocks = static_cast<int>(count / 256 + 1 < 8192 ? count / 256 + 1 : 8192);
+  DISTIE_DISPATCH(dtype, T, sum_slices_kernel<T><<<blocks, 256, 0, stream>>>(in, slices, count, static_cast<T*>(out)));
   return launch_status();
 }
 

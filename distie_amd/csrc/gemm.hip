@@ -6,8 +6,7 @@
 //  * gemm_skinny_bf16: bfloat16 x and W, M <= 64 (decode). Weight-streaming on the matrix cores
 //    (v_mfma_f32_16x16x32_bf16): a wave owns 16 rows of W and a slice of K, reads W straight from
 //    memory into the A operand (every weight byte is read once), and the small x is the B operand.
-//    Slices of K are combined in a fixed order by the last wave to finish, so results do not
-//    depend on timing.
+//    Slices of K are written side by side and added, in order, by the kernel that reads them.
 //
 // The reference leaves these products to a library (worker/src/inference/qwen2/model.py:149-152,
 // 231-233, 301); large bfloat16 products (prefill) are left to the library here as well.
@@ -89,57 +88,62 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 #define SK_ROWS 16          // rows of W per wave
-#define SK_KSTEP 128        // k per wave iteration: each lane reads 4 x 16 bytes = 64 contiguous bytes of its row
+#define SK_KSTEP 128        // k per wave iteration: four MFMAs of 32 k each
 
 // One wave per block. blockIdx.x: block of 16 rows of W; blockIdx.y: slice of K.
 // MB = ceil(M / 16) column blocks of x (1..4).
-// In a k-step the lane (r = lane % 16, g = lane / 16) reads W[n0 + r][k0 + 32 g + 8 j .. + 7] for j = 0..3 and the
-// same places of x's rows; MFMA j multiplies the two. Which k a lane holds does not matter as long as
-// A and B agree, and they do: both use the same function of (lane, j).
+// In a k-step, MFMA j works on k0 + 32 j .. + 31; the lane (r = lane % 16, g = lane / 16) holds
+// W[n0 + r][k0 + 32 j + 8 g .. + 7] and the same places of x's rows: the four lanes of a row read 64
+// contiguous bytes with one instruction. Blocks start at different k-steps of their slice and wrap
+// around, so that the waves of a launch do not all pull on the same memory channels at once.
+//
+// With more than one slice, slice s writes its float32 sums to y + s * M * N (slice 0 adds the bias):
+// the consumer adds the slices in order (the kernels that read activations here all can). A sum
+// across workgroups inside this kernel would need a device-wide release per wave, which on this
+// multi-die part costs more than the product itself.
 template <int MB, typename Y>
 __global__ __launch_bounds__(64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                          const float* __restrict__ bias, Y* __restrict__ y,
-                                                         float* __restrict__ partial, unsigned int* __restrict__ counters,
                                                          int M, int N, int K, int k_per_slice) {
   const int lane = threadIdx.x;
   const int r = lane % 16;
   const int g = lane / 16;
   const int64_t n0 = static_cast<int64_t>(blockIdx.x) * SK_ROWS;
-  const int slices = gridDim.y;
   const int k_begin = blockIdx.y * k_per_slice;
   const int k_end = min(K, k_begin + k_per_slice);
 
   // rows outside W or x are read from the last valid row and their results dropped
-  const int64_t w_row = min<int64_t>(n0 + r, N - 1);
-  const bf16_t* wp = w + w_row * K;
+  const int64_t w_row = (n0 + r < N) ? (n0 + r) : static_cast<int64_t>(N - 1);
+  const bf16_t* wp = w + w_row * K + 8 * g;
   const bf16_t* xp[MB];
 #pragma unroll
-  for (int b = 0; b < MB; ++b) xp[b] = x + static_cast<int64_t>(min(b * 16 + r, M - 1)) * K;
+  for (int b = 0; b < MB; ++b) xp[b] = x + static_cast<int64_t>(min(b * 16 + r, M - 1)) * K + 8 * g;
 
   floatx4 acc[MB];
 #pragma unroll
   for (int b = 0; b < MB; ++b) acc[b] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  int k0 = k_begin;
-  for (; k0 + SK_KSTEP <= k_end; k0 += SK_KSTEP) {
-    const int k = k0 + 32 * g;
+  const int steps = (k_end - k_begin) / SK_KSTEP;
+  int step = steps > 0 ? static_cast<int>(blockIdx.x % steps) : 0;
+  for (int it = 0; it < steps; ++it) {
+    const int k = k_begin + step * SK_KSTEP;
+    step = step + 1 == steps ? 0 : step + 1;
     bf16x8 a[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) a[j] = *reinterpret_cast<const bf16x8*>(wp + k + 8 * j);
+    for (int j = 0; j < 4; ++j) a[j] = *reinterpret_cast<const bf16x8*>(wp + k + 32 * j);
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const bf16x8 xb = *reinterpret_cast<const bf16x8*>(xp[b] + k + 8 * j);
+        const bf16x8 xb = *reinterpret_cast<const bf16x8*>(xp[b] + k + 32 * j);
         acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], xb, acc[b], 0, 0, 0);
       }
     }
   }
   // the rest of the slice (K is a multiple of 8; the slice's end need not be a multiple of 128)
-  for (; k0 < k_end; k0 += 32) {
-    const int k = k0 + 8 * g;
+  for (int k = k_begin + steps * SK_KSTEP; k < k_end; k += 32) {
     bf16x8 a = {};
-    const bool in = k < k_end;
+    const bool in = k + 8 * g < k_end;
     if (in) a = *reinterpret_cast<const bf16x8*>(wp + k);
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
@@ -150,41 +154,8 @@ __global__ __launch_bounds__(64) void gemm_skinny_kernel(const bf16_t* __restric
   }
 
   // acc[b][i] = sum for W row n0 + 4 g + i and x row 16 b + r
-  if (slices > 1) {
-    // partial[slice][m][n]; the last wave to arrive for this row block adds the slices in order
-    float* mine = partial + static_cast<int64_t>(blockIdx.y) * M * N;
-#pragma unroll
-    for (int b = 0; b < MB; ++b) {
-      const int m = b * 16 + r;
-      if (m >= M) continue;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int64_t n = n0 + 4 * g + i;
-        if (n < N) mine[static_cast<int64_t>(m) * N + n] = acc[b][i];
-      }
-    }
-    __threadfence();
-    __shared__ unsigned int arrived;
-    if (lane == 0) arrived = atomicAdd(&counters[blockIdx.x], 1u);
-    __syncthreads();
-    if (arrived != static_cast<unsigned int>(slices - 1)) return;
-    __threadfence();
-#pragma unroll
-    for (int b = 0; b < MB; ++b) {
-      const int m = b * 16 + r;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int64_t n = n0 + 4 * g + i;
-        float total = 0.f;
-        if (m < M && n < N)
-          for (int s = 0; s < slices; ++s)
-            total += __hip_atomic_load(partial + (static_cast<int64_t>(s) * M + m) * N + n, __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);  // written by other compute units: read past the local cache
-        acc[b][i] = total;
-      }
-    }
-    if (lane == 0) counters[blockIdx.x] = 0;   // ready for the next product
-  }
+  Y* out = y + static_cast<int64_t>(blockIdx.y) * M * N;
+  const bool with_bias = bias != nullptr && blockIdx.y == 0;
 #pragma unroll
   for (int b = 0; b < MB; ++b) {
     const int m = b * 16 + r;
@@ -192,38 +163,46 @@ __global__ __launch_bounds__(64) void gemm_skinny_kernel(const bf16_t* __restric
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int64_t n = n0 + 4 * g + i;
-      if (n < N) y[static_cast<int64_t>(m) * N + n] = from_float<Y>(acc[b][i] + (bias != nullptr ? bias[n] : 0.f));
+      if (n < N) out[static_cast<int64_t>(m) * N + n] = from_float<Y>(acc[b][i] + (with_bias ? bias[n] : 0.f));
     }
   }
 }
 
-// The number of K slices the launcher will use for this shape (so that the caller can size `partial`).
-extern "C" int distie_gemm_skinny_slices(int M, int N, int K) {
+// How a product is cut along K: enough waves to fill the chip (at most 8192), slices that are a
+// multiple of the k-step and at least 384 long.
+static void skinny_plan(int N, int K, int* slices, int* k_per_slice) {
   const int row_blocks = (N + SK_ROWS - 1) / SK_ROWS;
-  // aim at >= 2048 waves (8 per CU) while keeping >= 256 k per slice
-  int slices = 1;
-  while (row_blocks * slices < 2048 && K / (slices * 2) >= 256 && slices < 32) slices *= 2;
+  int want = 1;
+  while (want < 64 && row_blocks * want * 2 <= 8192 && K / (want * 2) >= 384) want *= 2;
+  int per = (K + want - 1) / want;
+  per = (per + SK_KSTEP - 1) / SK_KSTEP * SK_KSTEP;
+  *k_per_slice = per;
+  *slices = (K + per - 1) / per;
+}
+
+// The number of K slices the launcher will use for this shape.
+extern "C" int distie_gemm_skinny_slices(int M, int N, int K) {
+  (void)M;
+  int slices, per;
+  skinny_plan(N, K, &slices, &per);
   return slices;
 }
 
-// `partial`: float32 [slices * M * N] scratch, `counters`: uint32 [ceil(N / 16)] zero before the first call
-// (the kernel leaves them zero). Both may be null if slices == 1.
+// y: [M, N] of y_dtype if the shape gets one slice, else float32 [slices, M, N] (y_dtype must be float32).
 extern "C" int distie_gemm_skinny_bf16(const void* x, const void* w, const float* bias, void* y, int y_dtype,
-                                       int M, int N, int K, float* partial, unsigned int* counters,
-                                       hipStream_t stream) {
+                                       int M, int N, int K, hipStream_t stream) {
   if (M <= 0) return 0;
   if (M > 64 || N <= 0 || K <= 0 || K % 8 != 0) return DISTIE_BAD_ARGUMENT;
-  const int slices = distie_gemm_skinny_slices(M, N, K);
-  if (slices > 1 && (partial == nullptr || counters == nullptr)) return DISTIE_BAD_ARGUMENT;
-  int k_per_slice = (K + slices - 1) / slices;
-  k_per_slice = (k_per_slice + SK_KSTEP - 1) / SK_KSTEP * SK_KSTEP;
+  int slices, k_per_slice;
+  skinny_plan(N, K, &slices, &k_per_slice);
+  if (slices > 1 && y_dtype != DISTIE_F32) return DISTIE_BAD_ARGUMENT;
   dim3 grid((N + SK_ROWS - 1) / SK_ROWS, slices);
   const bf16_t* xb = static_cast<const bf16_t*>(x);
   const bf16_t* wb = static_cast<const bf16_t*>(w);
   const int mb = (M + 15) / 16;
 #define SKINNY(MB)                                                                                          \
   DISTIE_DISPATCH(y_dtype, Y, gemm_skinny_kernel<MB, Y><<<grid, 64, 0, stream>>>(                           \
-                                  xb, wb, bias, static_cast<Y*>(y), partial, counters, M, N, K, k_per_slice))
+                                  xb, wb, bias, static_cast<Y*>(y), M, N, K, k_per_slice))
   switch (mb) {
     case 1: SKINNY(1); break;
     case 2: SKINNY(2); break;

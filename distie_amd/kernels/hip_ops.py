@@ -47,6 +47,24 @@ def _check(status: int, name: str) -> None:
     raise KernelError(f"{name}: launch failed with HIP error {status}")
 
 
+class PartialSums:
+    """The result of a matrix product whose reduction was cut into slices: float32
+    [slices, rows, columns], to be added in order by whoever reads it. `linear` returns it for
+    small batches (a sum across workgroups inside the product would cost more than the product);
+    `add_rmsnorm`, `silu_mul` and `rope_kv_write` add the slices while they read, every other
+    operation sees the finished sum through `HipOps.dense`."""
+
+    def __init__(self, data: torch.Tensor, dtype: torch.dtype) -> None:
+        self.data = data
+        self.dtype = dtype                  # the dtype the finished sum would have
+        self.shape = data.shape[1:]
+        self.device = data.device
+
+    @property
+    def slices(self) -> int:
+        return self.data.shape[0]
+
+
 class HipOps(Ops):
     SKINNY_MAX_ROWS = 64
 
@@ -60,20 +78,19 @@ class HipOps(Ops):
         self._ops = ctypes.CDLL(str(build.ensure("ops")))
         self._declare()
         self._attn: Dict[int, ctypes.CDLL] = {}
-        self._partial: Optional[torch.Tensor] = None
-        self._counters = torch.zeros(16384, dtype=torch.int32, device=self.device)
 
     # ------------------------------------------------------------ plumbing
     def _declare(self) -> None:
         o = self._ops
         o.distie_embed.argtypes = [_P, _P, _I, _P, _I, _I, _I, _P]
-        o.distie_rmsnorm.argtypes = [_P, _P, _I, _P, _I, _P, _I, _I, _I, _F, _P]
-        o.distie_rope_kv_write.argtypes = [_P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P]
-        o.distie_silu_mul.argtypes = [_P, _P, _I, _I, _I, _P]
+        o.distie_rmsnorm.argtypes = [_P, _P, _I, _I, _P, _I, _P, _I, _I, _I, _F, _P]
+        o.distie_rope_kv_write.argtypes = [_P, _I, _I, _P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P]
+        o.distie_silu_mul.argtypes = [_P, _I, _I, _P, _I, _I, _I, _P]
+        o.distie_sum_slices.argtypes = [_P, _I, _L, _P, _I, _P]
         o.distie_gather_rows.argtypes = [_P, _P, _P, _I, _L, _I, _P]
         o.distie_gemm_generic.argtypes = [_P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _P]
         o.distie_gemm_skinny_slices.argtypes = [_I, _I, _I]
-        o.distie_gemm_skinny_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P]
+        o.distie_gemm_skinny_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _P]
         o.distie_argmax.argtypes = [_P, _P, _I, _I, _P]
         o.distie_sample.argtypes = [_P, _P, _P, _P, _P, _I, _I, _P]
 
@@ -120,22 +137,35 @@ class HipOps(Ops):
         if x.dtype != torch.float32:
             raise KernelError("rmsnorm reads the float32 residual stream")
         out = torch.empty(x.shape, dtype=out_dtype, device=self.device)
-        _check(self._ops.distie_rmsnorm(x.data_ptr(), None, _F32, weight.data_ptr(), _code(weight),
+        _check(self._ops.distie_rmsnorm(x.data_ptr(), None, _F32, 1, weight.data_ptr(), _code(weight),
                                         out.data_ptr(), _CODES[out_dtype], x.shape[0], x.shape[1], eps,
                                         self._stream()), "rmsnorm")
         return out
 
     def add_rmsnorm(self, residual, delta, weight, eps, out_dtype):
+        slices = 1
+        if isinstance(delta, PartialSums):
+            slices, delta = delta.slices, delta.data
         self._own(residual, delta, weight)
-        if residual.dtype != torch.float32 or residual.shape != delta.shape:
+        if residual.dtype != torch.float32 or residual.shape != delta.shape[-2:]:
             raise KernelError("add_rmsnorm: residual must be float32 and shaped like delta")
         out = torch.empty(residual.shape, dtype=out_dtype, device=self.device)
-        _check(self._ops.distie_rmsnorm(residual.data_ptr(), delta.data_ptr(), _code(delta), weight.data_ptr(),
-                                        _code(weight), out.data_ptr(), _CODES[out_dtype], residual.shape[0],
-                                        residual.shape[1], eps, self._stream()), "add_rmsnorm")
+        _check(self._ops.distie_rmsnorm(residual.data_ptr(), delta.data_ptr(), _code(delta), slices,
+                                        weight.data_ptr(), _code(weight), out.data_ptr(), _CODES[out_dtype],
+                                        residual.shape[0], residual.shape[1], eps, self._stream()), "add_rmsnorm")
         return out
 
-    def _linear(self, x, weight, bias, out_dtype):
+    def dense(self, x):
+        """The finished sum of a `PartialSums`; any other tensor as it is."""
+        if not isinstance(x, PartialSums):
+            return x
+        out = torch.empty(tuple(x.shape), dtype=x.dtype, device=self.device)
+        _check(self._ops.distie_sum_slices(x.data.data_ptr(), x.slices, out.numel(), out.data_ptr(),
+                                           _CODES[x.dtype], self._stream()), "sum_slices")
+        return out
+
+    def _linear(self, x, weight, bias, out_dtype, partial_ok=False):
+        x = self.dense(x)
         self._own(x, weight, bias)
         M, K = x.shape
         N = weight.shape[0]
@@ -145,23 +175,17 @@ class HipOps(Ops):
             raise KernelError("linear: bias must be float32 [N]")
         both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
         if both_bf16 and M <= self.SKINNY_MAX_ROWS and K % 8 == 0:
-            out = torch.empty((M, N), dtype=out_dtype, device=self.device)
             slices = self._ops.distie_gemm_skinny_slices(M, N, K)
-            partial = None
-            if slices > 1:
-                need = slices * M * N
-                if self._partial is None or self._partial.numel() < need:
-                    if torch.cuda.is_current_stream_capturing():
-                        raise KernelError("split-K scratch must be sized before a graph is captured")
-                    self._partial = torch.empty(max(need, 1 << 22), dtype=torch.float32, device=self.device)
-                partial = self._partial
-                if (N + 15) // 16 > self._counters.numel():
-                    raise KernelError("linear: too many rows for the split-K counters")
+            if slices == 1:
+                out = torch.empty((M, N), dtype=out_dtype, device=self.device)
+            else:
+                out = torch.empty((slices, M, N), dtype=torch.float32, device=self.device)
             _check(self._ops.distie_gemm_skinny_bf16(
                 x.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(),
-                _CODES[out_dtype], M, N, K, partial.data_ptr() if partial is not None else None,
-                self._counters.data_ptr(), self._stream()), "gemm_skinny_bf16")
-            return out
+                _code(out), M, N, K, self._stream()), "gemm_skinny_bf16")
+            if slices == 1:
+                return out
+            return PartialSums(out, out_dtype) if partial_ok else self.dense(PartialSums(out, out_dtype))
         if both_bf16:
             # large bfloat16 product: the library's matrix-core kernels
             lib_bias = None
@@ -179,16 +203,23 @@ class HipOps(Ops):
         return out
 
     def linear(self, x, weight, bias=None):
-        return self._linear(x, weight, bias, x.dtype)
+        """May return `PartialSums` (see there)."""
+        return self._linear(x, weight, bias, x.dtype, partial_ok=True)
 
     def linear_f32out(self, x, weight):
         return self._linear(x, weight, None, torch.float32)
 
     def rope_kv_write(self, qkv, meta: BatchMeta, group, k_cache, v_cache, inv_freq, num_heads, num_kv_heads,
                       head_dim, write):
-        self._own(qkv, k_cache, v_cache, inv_freq)
-        T = qkv.shape[0]
-        if qkv.shape[1] != (num_heads + 2 * num_kv_heads) * head_dim:
+        slices, source = 1, qkv
+        if isinstance(qkv, PartialSums):
+            slices, source = qkv.slices, qkv.data
+            out = torch.empty(tuple(qkv.shape), dtype=qkv.dtype, device=self.device)
+        else:
+            out = qkv
+        self._own(source, k_cache, v_cache, inv_freq)
+        T = out.shape[0]
+        if out.shape[1] != (num_heads + 2 * num_kv_heads) * head_dim:
             raise KernelError("rope_kv_write: qkv width does not match the head counts")
         if tuple(k_cache.shape[1:]) != (num_kv_heads, meta.block_size, head_dim) or k_cache.shape != v_cache.shape:
             raise KernelError("rope_kv_write: cache is not [pages, kv_heads, block_size, head_dim]")
@@ -197,12 +228,15 @@ class HipOps(Ops):
         pairs = 0 if inv_freq is None else inv_freq.shape[0]
         slots = meta.groups[group].slots
         _check(self._ops.distie_rope_kv_write(
-            qkv.data_ptr(), _code(qkv), meta.positions.data_ptr(), slots.data_ptr(), k_cache.data_ptr(),
-            v_cache.data_ptr(), _code(k_cache), inv_freq.data_ptr() if inv_freq is not None else None, pairs, T,
-            num_heads, num_kv_heads, head_dim, meta.block_size, 1 if write else 0, self._stream()), "rope_kv_write")
+            source.data_ptr(), _code(source), slices, out.data_ptr(), _code(out), meta.positions.data_ptr(),
+            slots.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _code(k_cache),
+            inv_freq.data_ptr() if inv_freq is not None else None, pairs, T, num_heads, num_kv_heads, head_dim,
+            meta.block_size, 1 if write else 0, self._stream()), "rope_kv_write")
+        return out
 
     def paged_attention(self, qkv, meta: BatchMeta, group, k_cache, v_cache, num_heads, num_kv_heads, head_dim,
                         scale, window):
+        qkv = self.dense(qkv)
         self._own(qkv, k_cache, v_cache)
         lib = self.attention_library(head_dim)
         T = qkv.shape[0]
@@ -220,14 +254,18 @@ class HipOps(Ops):
         return out
 
     def silu_mul(self, gate_up):
-        self._own(gate_up)
+        slices, source, dtype = 1, gate_up, gate_up.dtype
+        if isinstance(gate_up, PartialSums):
+            slices, source = gate_up.slices, gate_up.data
+        self._own(source)
         rows, two = gate_up.shape
-        out = torch.empty((rows, two // 2), dtype=gate_up.dtype, device=self.device)
-        _check(self._ops.distie_silu_mul(gate_up.data_ptr(), out.data_ptr(), _code(gate_up), rows, two // 2,
-                                         self._stream()), "silu_mul")
+        out = torch.empty((rows, two // 2), dtype=dtype, device=self.device)
+        _check(self._ops.distie_silu_mul(source.data_ptr(), _code(source), slices, out.data_ptr(), _code(out),
+                                         rows, two // 2, self._stream()), "silu_mul")
         return out
 
     def gather_rows(self, x, rows):
+        x = self.dense(x)
         self._own(x, rows)
         out = torch.empty((rows.shape[0], x.shape[1]), dtype=x.dtype, device=self.device)
         _check(self._ops.distie_gather_rows(x.data_ptr(), rows.data_ptr(), out.data_ptr(), rows.shape[0],

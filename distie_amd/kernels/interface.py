@@ -69,7 +69,12 @@ class Ops(abc.ABC):
 
     @abc.abstractmethod
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """x [T, K] (act) times weight [N, K] transposed, plus bias [N] -> act [T, N]."""
+        """x [T, K] (act) times weight [N, K] transposed, plus bias [N] -> act [T, N].
+
+        An implementation may return the product in a form of its own that only its
+        `add_rmsnorm`, `silu_mul`, `rope_kv_write`, `linear`, `paged_attention` and `gather_rows`
+        read (the HIP kernels return partial sums over slices of K for small batches); parts
+        hand the result on to those operations and do nothing else with it."""
 
     @abc.abstractmethod
     def linear_f32out(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
@@ -78,10 +83,11 @@ class Ops(abc.ABC):
     @abc.abstractmethod
     def rope_kv_write(self, qkv: torch.Tensor, meta: BatchMeta, group: int, k_cache: torch.Tensor,
                       v_cache: torch.Tensor, inv_freq: Optional[torch.Tensor], num_heads: int,
-                      num_kv_heads: int, head_dim: int, write: bool) -> None:
-        """Rotate q and k of qkv [T, (H+2KH)*D] in place by each token's position (angles and
+                      num_kv_heads: int, head_dim: int, write: bool) -> torch.Tensor:
+        """Rotate q and k of qkv [T, (H+2KH)*D] by each token's position (angles and
         trigonometry in float32; no rotation if inv_freq is None) and, if `write`, store the
-        rotated k and v at the token's slot of k_cache / v_cache [NB, KH, P, D]."""
+        rotated k and v at the token's slot of k_cache / v_cache [NB, KH, P, D]. Returns the
+        rotated qkv (the argument itself if it was rotated in place)."""
 
     @abc.abstractmethod
     def paged_attention(self, qkv: torch.Tensor, meta: BatchMeta, group: int, k_cache: torch.Tensor,

@@ -67,8 +67,8 @@ class Attention(Mixer):
 
     def forward(self, ops, x, ctx, cache, writes_cache: bool):
         qkv = ops.linear(x, self.qkv_weight, self.qkv_bias_t)
-        ops.rope_kv_write(qkv, ctx.meta, cache.group, cache.k, cache.v, self.position.rotary(),
-                          self.num_heads, self.num_kv_heads, self.head_dim, writes_cache)
+        qkv = ops.rope_kv_write(qkv, ctx.meta, cache.group, cache.k, cache.v, self.position.rotary(),
+                                self.num_heads, self.num_kv_heads, self.head_dim, writes_cache)
         mixed = ops.paged_attention(qkv, ctx.meta, cache.group, cache.k, cache.v, self.num_heads,
                                     self.num_kv_heads, self.head_dim, self.scale, self.window)
         return ops.linear(mixed, self.out_weight, self.out_bias_t)

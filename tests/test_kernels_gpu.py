@@ -86,12 +86,56 @@ def test_gemm_skinny_bf16(ops, M, N, K):
     want = x.double() @ w.double().T
     got = ops.linear_f32out(x, w)
     close(got, want, torch.float32, scale=5 * want.abs().max().item())
-    got = ops.linear(x, w, b)
+    got = ops.dense(ops.linear(x, w, b))
     assert got.dtype == torch.bfloat16
     close(got, want + b.double(), torch.bfloat16, scale=want.abs().max().item())
-    # the counters are left at zero: a second product with other sizes is right too
-    again = ops.linear_f32out(x[:1], w)
-    close(again, want[:1], torch.float32, scale=5 * want.abs().max().item())
+
+
+def test_partial_sums_are_added_by_their_readers(ops):
+    """A product over a long K comes back as slices; norm, activation and rotation add them."""
+    from distie_amd.kernels.hip_ops import PartialSums
+
+    M, K = 5, 2048
+    x = rand(M, K, dtype=torch.bfloat16, seed=1)
+    # residual add + norm
+    w = rand(96, K, dtype=torch.bfloat16, seed=2, scale=0.05)
+    part = ops.linear(x, w)
+    assert isinstance(part, PartialSums) and part.slices > 1
+    delta = x.double() @ w.double().T
+    res = rand(M, 96, seed=3)
+    want_res = res.double() + delta
+    g = rand(96, dtype=torch.bfloat16, seed=4)
+    got = ops.add_rmsnorm(res, part, g, 1e-6, torch.bfloat16)
+    assert torch.allclose(res.double(), want_res, atol=1e-4)
+    want = want_res * torch.rsqrt(want_res.pow(2).mean(-1, keepdim=True) + 1e-6) * g.double()
+    close(got, want, torch.bfloat16, scale=want.abs().max().item())
+    # gated activation
+    w = rand(2 * 88, K, dtype=torch.bfloat16, seed=5, scale=0.05)
+    part = ops.linear(x, w)
+    assert isinstance(part, PartialSums)
+    gu = x.double() @ w.double().T
+    want = gu[:, :88] / (1 + torch.exp(-gu[:, :88])) * gu[:, 88:]
+    close(ops.silu_mul(part), want, torch.bfloat16, scale=want.abs().max().item())
+    # rotation + cache write, with a bias
+    heads, kv_heads, dim, P = 3, 1, 32, 4
+    w = rand((heads + 2 * kv_heads) * dim, K, dtype=torch.bfloat16, seed=6, scale=0.05)
+    b = rand((heads + 2 * kv_heads) * dim, seed=7)
+    part = ops.linear(x, w, b)
+    assert isinstance(part, PartialSums)
+    dense = (x.double() @ w.double().T + b.double()).float()
+    meta = make_meta([7, 8, 9, 0, 30], [0, 0, 0, 1, 2], [0, 3, 4, 5], [10, 1, 31], [[2, 0, 1, -1, -1, -1, -1, -1]] * 3,
+                     [0 * P + 3, 1 * P + 0, 1 * P + 1, 5 * P, 6 * P + 2], P)
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, dim, 2, dtype=torch.float32) / dim))).cuda()
+    k1 = torch.zeros(8, kv_heads, P, dim, dtype=torch.bfloat16, device="cuda")
+    v1, k2, v2 = torch.zeros_like(k1), torch.zeros_like(k1), torch.zeros_like(k1)
+    got = ops.rope_kv_write(part, meta, 0, k1, v1, inv_freq, heads, kv_heads, dim, True)
+    want = TorchOps("cuda").rope_kv_write(dense.clone(), meta, 0, k2, v2, inv_freq, heads, kv_heads, dim, True)
+    assert got.dtype == torch.bfloat16
+    close(got, want, torch.bfloat16, scale=want.abs().max().item())
+    close(k1, k2, torch.bfloat16, scale=want.abs().max().item())
+    close(v1, v2, torch.bfloat16, scale=want.abs().max().item())
+    # any other reader sees the finished sum
+    close(ops.dense(part), dense, torch.bfloat16, scale=dense.abs().max().item())
 
 
 def test_gemm_large_bf16_uses_library_and_matches(ops):

@@ -57,6 +57,7 @@ class TorchOps(Ops):
             v = view[:, num_heads + num_kv_heads:]
             k_cache[slots // P, :, slots % P] = k.to(k_cache.dtype)
             v_cache[slots // P, :, slots % P] = v.to(v_cache.dtype)
+        return qkv
 
     def paged_attention(self, qkv, meta, group, k_cache, v_cache, num_heads, num_kv_heads, head_dim,
                         scale, window):
