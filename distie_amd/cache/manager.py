@@ -59,7 +59,7 @@ class CacheGroup:
     layers: List[int]
     pool: BlockPool
     k: Optional[torch.Tensor] = None      # [layers, pages + 1, KH, P, D]
-    v: Optional[torch.Tensor] = None
+    v: Optional[torch.Tensor] = None      # [layers, pages + 1, KH, D, P]
 
     @property
     def sink_page(self) -> int:
@@ -107,9 +107,9 @@ class CacheManager:
         for index, group in enumerate(self.groups):
             need = group.requirement
             if allocate:
-                shape = (len(group.layers), self.num_blocks + 1, need.num_kv_heads, self.block_size, need.head_dim)
-                group.k = torch.zeros(shape, dtype=dtype, device=device)
-                group.v = torch.zeros(shape, dtype=dtype, device=device)
+                lead = (len(group.layers), self.num_blocks + 1, need.num_kv_heads)
+                group.k = torch.zeros(lead + (self.block_size, need.head_dim), dtype=dtype, device=device)
+                group.v = torch.zeros(lead + (need.head_dim, self.block_size), dtype=dtype, device=device)
             for i, layer in enumerate(group.layers):
                 self._layer_view[layer] = LayerCache(
                     group=index, k=group.k[i] if allocate else None, v=group.v[i] if allocate else None)

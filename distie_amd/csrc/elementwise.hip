@@ -92,8 +92,8 @@ extern "C" int distie_rmsnorm(float* residual, const void* delta, int delta_dtyp
 // in: [slices, T, (H + 2 KH) * D] (partial sums of the q/k/v product, added in order; one slice for a
 // finished product), out: [T, (H + 2 KH) * D], which may be `in` itself. One block per token. Pair
 // (j, j + R/2) of every q and k head is turned by angle = float(position) * inv_freq[j] (R = 2 * pairs <= D
-// is the rotated width). The turned k and the v of the token go to the cache [pages, KH, P, D] at the
-// token's slot (slot = page * P + offset).
+// is the rotated width). The turned k and the v of the token go to the cache at the token's slot
+// (slot = page * P + offset): k into [pages, KH, P, D], v transposed into [pages, KH, D, P].
 template <typename I, typename T, typename C>
 __global__ void rope_kv_write_kernel(const I* in, int slices, int64_t slice_stride, T* out,
                                      const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
@@ -145,9 +145,10 @@ __global__ void rope_kv_write_kernel(const I* in, int slices, int64_t slice_stri
   for (int i = threadIdx.x; i < kv_heads * dim; i += blockDim.x) {
     const int head = i / dim;
     const int d = i % dim;
-    const int64_t at = ((page * kv_heads + head) * block_size + offset) * dim + d;
-    k_cache[at] = from_float<C>(to_float(row[(heads + head) * dim + d]));
-    v_cache[at] = from_float<C>(to_float(row[(heads + kv_heads + head) * dim + d]));
+    const int64_t base = (page * kv_heads + head) * block_size * dim;
+    k_cache[base + static_cast<int64_t>(offset) * dim + d] = from_float<C>(to_float(row[(heads + head) * dim + d]));
+    v_cache[base + static_cast<int64_t>(d) * block_size + offset] =
+        from_float<C>(to_float(row[(heads + kv_heads + head) * dim + d]));
   }
 }
 

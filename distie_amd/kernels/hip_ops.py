@@ -110,6 +110,10 @@ class HipOps(Ops):
             lib = ctypes.CDLL(str(build.ensure(f"attn_d{head_dim}")))
             lib.distie_attention_generic.argtypes = [_P, _I, _L, _P, _P, _I, _P, _P, _P, _I, _P,
                                                      _I, _I, _I, _I, _F, _I, _P]
+            lib.distie_attention_prefill_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I,
+                                                          _F, _I, _P]
+            lib.distie_attention_decode_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I,
+                                                         _I, _F, _I, _I, _I, _P]
             if lib.distie_attention_head_dim() != head_dim:
                 raise KernelError("attention library was built for another head size")
             self._attn[head_dim] = lib
@@ -123,6 +127,13 @@ class HipOps(Ops):
                 raise KernelError(f"tensor on {t.device}, kernels run on {self.device}")
             if not t.is_contiguous():
                 raise KernelError("kernels take contiguous tensors")
+
+    @staticmethod
+    def _check_cache(k_cache, v_cache, kv_heads, block_size, head_dim) -> None:
+        if tuple(k_cache.shape[1:]) != (kv_heads, block_size, head_dim) or \
+                tuple(v_cache.shape[1:]) != (kv_heads, head_dim, block_size) or k_cache.shape[0] != v_cache.shape[0]:
+            raise KernelError("cache is not k [pages, kv_heads, block_size, head_dim], "
+                              "v [pages, kv_heads, head_dim, block_size]")
 
     # ------------------------------------------------------------ operations
     def embed(self, ids, table):
@@ -221,8 +232,7 @@ class HipOps(Ops):
         T = out.shape[0]
         if out.shape[1] != (num_heads + 2 * num_kv_heads) * head_dim:
             raise KernelError("rope_kv_write: qkv width does not match the head counts")
-        if tuple(k_cache.shape[1:]) != (num_kv_heads, meta.block_size, head_dim) or k_cache.shape != v_cache.shape:
-            raise KernelError("rope_kv_write: cache is not [pages, kv_heads, block_size, head_dim]")
+        self._check_cache(k_cache, v_cache, num_kv_heads, meta.block_size, head_dim)
         if T != meta.num_tokens:
             raise KernelError("rope_kv_write: qkv rows do not match the batch")
         pairs = 0 if inv_freq is None else inv_freq.shape[0]
@@ -241,11 +251,34 @@ class HipOps(Ops):
         lib = self.attention_library(head_dim)
         T = qkv.shape[0]
         table = meta.groups[group].block_table
-        if tuple(k_cache.shape[1:]) != (num_kv_heads, meta.block_size, head_dim):
-            raise KernelError("paged_attention: cache is not [pages, kv_heads, block_size, head_dim]")
+        self._check_cache(k_cache, v_cache, num_kv_heads, meta.block_size, head_dim)
         if T != meta.num_tokens or table.shape[0] != meta.num_requests:
             raise KernelError("paged_attention: tensors do not match the batch")
         out = torch.empty((T, num_heads * head_dim), dtype=qkv.dtype, device=self.device)
+        bf16 = qkv.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16
+        if bf16 and meta.block_size % 16 == 0:
+            group = num_heads // num_kv_heads
+            if meta.all_decode and group <= lib.distie_attention_mfma_columns():
+                # keys are cut into runs, one wave each: enough waves to fill the chip when few requests decode
+                runs = max(1, min(64, 4096 // (meta.num_requests * num_kv_heads)))
+                split_len = max(64, -(-meta.max_kv // runs + 31) // 32 * 32)
+                max_splits = -(-meta.max_kv // split_len)
+                part_o = torch.empty((meta.num_requests, num_heads, max_splits, head_dim), dtype=torch.float32,
+                                     device=self.device)
+                part_ml = torch.empty((meta.num_requests, num_heads, max_splits, 2), dtype=torch.float32,
+                                      device=self.device)
+                _check(lib.distie_attention_decode_bf16(
+                    qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), meta.positions.data_ptr(),
+                    meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], out.data_ptr(), part_o.data_ptr(),
+                    part_ml.data_ptr(), meta.num_requests, num_heads, num_kv_heads, meta.block_size, float(scale),
+                    int(window or 0), split_len, max_splits, self._stream()), "attention_decode_bf16")
+                return out
+            _check(lib.distie_attention_prefill_bf16(
+                qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), meta.positions.data_ptr(),
+                meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], out.data_ptr(), T, meta.num_requests,
+                num_heads, num_kv_heads, meta.block_size, float(scale), int(window or 0), self._stream()),
+                "attention_prefill_bf16")
+            return out
         _check(lib.distie_attention_generic(
             qkv.data_ptr(), _code(qkv), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), _code(k_cache),
             meta.positions.data_ptr(), meta.token_request.data_ptr(), table.data_ptr(), table.shape[1],

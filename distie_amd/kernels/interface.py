@@ -86,7 +86,7 @@ class Ops(abc.ABC):
                       num_kv_heads: int, head_dim: int, write: bool) -> torch.Tensor:
         """Rotate q and k of qkv [T, (H+2KH)*D] by each token's position (angles and
         trigonometry in float32; no rotation if inv_freq is None) and, if `write`, store the
-        rotated k and v at the token's slot of k_cache / v_cache [NB, KH, P, D]. Returns the
+        rotated k and v at the token's slot of k_cache [NB, KH, P, D] / v_cache [NB, KH, D, P]. Returns the
         rotated qkv (the argument itself if it was rotated in place)."""
 
     @abc.abstractmethod

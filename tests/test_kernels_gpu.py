@@ -127,7 +127,8 @@ def test_partial_sums_are_added_by_their_readers(ops):
                      [0 * P + 3, 1 * P + 0, 1 * P + 1, 5 * P, 6 * P + 2], P)
     inv_freq = (1.0 / (10000.0 ** (torch.arange(0, dim, 2, dtype=torch.float32) / dim))).cuda()
     k1 = torch.zeros(8, kv_heads, P, dim, dtype=torch.bfloat16, device="cuda")
-    v1, k2, v2 = torch.zeros_like(k1), torch.zeros_like(k1), torch.zeros_like(k1)
+    v1 = torch.zeros(8, kv_heads, dim, P, dtype=torch.bfloat16, device="cuda")
+    k2, v2 = torch.zeros_like(k1), torch.zeros_like(v1)
     got = ops.rope_kv_write(part, meta, 0, k1, v1, inv_freq, heads, kv_heads, dim, True)
     want = TorchOps("cuda").rope_kv_write(dense.clone(), meta, 0, k2, v2, inv_freq, heads, kv_heads, dim, True)
     assert got.dtype == torch.bfloat16
@@ -167,7 +168,7 @@ def test_rope_kv_write(ops, dtype, heads, kv_heads, dim, pairs):
     qkv = rand(7, (heads + 2 * kv_heads) * dim, dtype=dtype, seed=4)
     inv_freq = (1.0 / (10000.0 ** (torch.arange(0, 2 * pairs, 2, dtype=torch.float32) / (2 * pairs)))).cuda()
     k1 = torch.zeros(pages, kv_heads, P, dim, dtype=dtype, device="cuda")
-    v1 = torch.zeros_like(k1)
+    v1 = torch.zeros(pages, kv_heads, dim, P, dtype=dtype, device="cuda")
     k2, v2, qkv2 = k1.clone(), v1.clone(), qkv.clone()
     ops.rope_kv_write(qkv, meta, 0, k1, v1, inv_freq, heads, kv_heads, dim, True)
     ref = TorchOps("cuda")
@@ -186,7 +187,7 @@ def test_rope_kv_write(ops, dtype, heads, kv_heads, dim, pairs):
         assert torch.equal(view[5, 0, 2 * pairs:], src[5, 0, 2 * pairs:].to(dtype).cuda())
     # without writing, the cache stays as it is
     k3 = torch.zeros_like(k1)
-    ops.rope_kv_write(qkv.clone(), meta, 0, k3, torch.zeros_like(k1), inv_freq, heads, kv_heads, dim, False)
+    ops.rope_kv_write(qkv.clone(), meta, 0, k3, torch.zeros_like(v1), inv_freq, heads, kv_heads, dim, False)
     assert k3.abs().sum() == 0
 
 
@@ -207,22 +208,44 @@ def paged_case(heads, kv_heads, dim, P, lens, q_lens, dtype, seed=0):
         cu_q.append(len(positions))
     meta = make_meta(positions, token_request, cu_q, lens, tables, slots, P)
     k = rand(total_pages, kv_heads, P, dim, dtype=dtype, seed=seed + 1)
-    v = rand(total_pages, kv_heads, P, dim, dtype=dtype, seed=seed + 2)
+    v = rand(total_pages, kv_heads, dim, P, dtype=dtype, seed=seed + 2)
     qkv = rand(len(positions), (heads + 2 * kv_heads) * dim, dtype=dtype, seed=seed + 3)
     return meta, qkv, k, v
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,kv_heads,dim,P,window", [
+ATTENTION_SHAPES = [
     (4, 2, 16, 4, None), (3, 1, 32, 8, 8), (5, 5, 48, 16, 20), (12, 2, 128, 16, None),
-    (6, 3, 64, 5, 33), (8, 1, 80, 16, None), (2, 2, 256, 32, 100)])
+    (6, 3, 64, 5, 33), (8, 1, 80, 16, None), (2, 2, 256, 32, 100), (4, 2, 16, 16, 7), (40, 2, 32, 16, None),
+    (12, 2, 128, 64, 150)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,dim,P,window", ATTENTION_SHAPES)
 def test_paged_attention(ops, dtype, heads, kv_heads, dim, P, window):
-    lens, q_lens = [70, 1, 33, 130, 200], [70, 1, 2, 1, 17]
+    """Mixed step: whole prompts, portions down to two tokens, single decoded tokens."""
+    lens, q_lens = [70, 1, 33, 130, 200, 67], [70, 1, 2, 1, 17, 66]
     meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, lens, q_lens, dtype)
     got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
     want = TorchOps("cuda").paged_attention(qkv.double(), meta, 0, k.double(), v.double(), heads, kv_heads, dim,
                                             dim ** -0.5, window)
-    close(got, want, dtype, scale=1.0)
+    close(got, want, dtype, scale=want.abs().max().item())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,dim,P,window", ATTENTION_SHAPES)
+def test_paged_attention_decode_step(ops, dtype, heads, kv_heads, dim, P, window):
+    """Every request brings one token (the split-key kernel in bfloat16), contexts from 1 to 700."""
+    lens = [1, 2, 16, 17, 64, 65, 129, 300, 700]
+    meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, lens, [1] * len(lens), dtype)
+    meta.all_decode = True
+    want = TorchOps("cuda").paged_attention(qkv.double(), meta, 0, k.double(), v.double(), heads, kv_heads, dim,
+                                            dim ** -0.5, window)
+    got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
+    close(got, want, dtype, scale=want.abs().max().item())
+    # as in a captured step: the launch is sized for the longest context the model allows
+    meta.max_kv = 4096
+    got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
+    close(got, want, dtype, scale=want.abs().max().item())
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -238,9 +261,11 @@ def test_attention_finds_one_far_key(ops, dtype):
         k[page, :, far % P, 0] = 30.0
         q[0, :heads] = 0
         q[0, :heads, 0] = 30.0
-        got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
-        want = v[page, :, far % P].float().repeat_interleave(2, dim=0).reshape(1, -1)
-        close(got, want, dtype, scale=4.0)
+        want = v[page, :, :, far % P].float().repeat_interleave(2, dim=0).reshape(1, -1)
+        for decode in (False, True):
+            meta.all_decode = decode
+            got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
+            close(got, want, dtype, scale=4.0)
     # just outside the window the key must not count
     meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, [300], [1], dtype, seed=5)
     far = 299 - 64

@@ -56,7 +56,7 @@ class TorchOps(Ops):
             k = view[:, num_heads:num_heads + num_kv_heads]
             v = view[:, num_heads + num_kv_heads:]
             k_cache[slots // P, :, slots % P] = k.to(k_cache.dtype)
-            v_cache[slots // P, :, slots % P] = v.to(v_cache.dtype)
+            v_cache[slots // P, :, :, slots % P] = v.to(v_cache.dtype)
         return qkv
 
     def paged_attention(self, qkv, meta, group, k_cache, v_cache, num_heads, num_kv_heads, head_dim,
@@ -76,7 +76,7 @@ class TorchOps(Ops):
                 pages = table[b, keys // P]
                 assert (pages >= 0).all(), "attention would read a page that was given back"
                 k = k_cache[pages, :, keys % P].float()          # [n, KH, D]
-                v = v_cache[pages, :, keys % P].float()
+                v = v_cache[pages, :, :, keys % P].float()
                 k = k.repeat_interleave(rep, dim=1)
                 v = v.repeat_interleave(rep, dim=1)
                 s = torch.einsum("hd,nhd->hn", q_all[t], k) * scale
