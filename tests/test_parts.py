@@ -1,0 +1,310 @@
+"""Each part alone against the plain implementation, and the generality of the assembly:
+a toy mixer with state of its own, defined here, is registered, built into a model beside
+attention layers and stepped; a run order that names a layer twice and lets a layer read
+another layer's cache. No file of the package changes for this.
+
+Runs on the CPU test double, and on the HIP kernels when a GPU is there."""
+
+import pytest
+import torch
+
+import plain_qwen2 as plain
+from distie_amd.cache import CacheManager
+from distie_amd.config import LayerCall, LayerSpec, ModelSpec, PartSpec, register_architecture
+from distie_amd.engine.batch import BatchBuilder, StepEntry
+from distie_amd.engine.model import Model
+from distie_amd.engine.runner import ModelRunner
+from distie_amd.parts import (FixedState, Mixer, PagedKV, ParamSpec, ResidualStream, StepContext, build_part,
+                              register_part)
+from torch_ops import TorchOps
+
+
+@pytest.fixture(scope="module", params=["cpu", pytest.param("hip", marks=pytest.mark.gpu)])
+def ops(request):
+    if request.param == "cpu":
+        return TorchOps()
+    from distie_amd.kernels.hip_ops import HipOps
+
+    return HipOps("cuda:0")
+
+
+def rnd(*shape, seed=0, scale=1.0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+def dense(ops, x):
+    return ops.dense(x) if hasattr(ops, "dense") else x
+
+
+def context(ops, requirements, lengths, block=4, dtype=torch.float32):
+    """A cache and the batch of whole sequences of the given lengths."""
+    cache = CacheManager(requirements, block, 64, 8, device=ops.device, dtype=dtype)
+    builder = BatchBuilder(cache, 512, ops.device, 1000)
+    entries = []
+    for i, n in enumerate(lengths):
+        cache.add(i)
+        cache.reserve(i, n)
+        entries.append(StepEntry(i, [0] * n, []))
+    ids, meta, _ = builder.build(entries)
+    return cache, meta
+
+
+def test_rmsnorm_part(ops):
+    part = build_part("norm", PartSpec("rmsnorm", "n.", {"size": 50, "eps": 1e-3}))
+    assert {k: v.shape for k, v in part.param_specs().items()} == {"weight": (50,)}
+    w = 1 + rnd(50, seed=1, scale=0.3)
+    part.load({"weight": w.to(ops.device)})
+    x = rnd(6, 50, seed=2, scale=2.0)
+    got = part.apply(ops, x.to(ops.device), torch.float32)
+    assert (got.cpu() - plain.rms_norm(x, w, 1e-3)).abs().max() < 1e-5
+    stream = ResidualStream(x.clone().to(ops.device))
+    stream.pending = rnd(6, 50, seed=3).to(ops.device)
+    got = part.of_stream(ops, stream, torch.float32)
+    want = x + rnd(6, 50, seed=3)
+    assert stream.pending is None and (stream.hidden.cpu() - want).abs().max() < 1e-6
+    assert (got.cpu() - plain.rms_norm(want, w, 1e-3)).abs().max() < 1e-5
+
+
+def test_rotary_part(ops):
+    part = build_part("position", PartSpec("rope", "", {"dim": 24, "theta": 500.0}))
+    assert torch.allclose(part.rotary(), plain.rope_inv_freq(24, 500.0))
+    with pytest.raises(ValueError):
+        build_part("position", PartSpec("rope", "", {"dim": 7, "theta": 500.0}))
+    assert build_part("position", PartSpec("none")).rotary() is None
+
+
+def test_swiglu_part(ops):
+    part = build_part("feed_forward", PartSpec("swiglu", "mlp.", {"hidden_size": 40, "intermediate_size": 72}))
+    w = {"gate_proj.weight": rnd(72, 40, seed=1, scale=0.2), "up_proj.weight": rnd(72, 40, seed=2, scale=0.2),
+         "down_proj.weight": rnd(40, 72, seed=3, scale=0.2)}
+    assert {k: v.shape for k, v in part.param_specs().items()} == {k: tuple(v.shape) for k, v in w.items()}
+    part.load({k: v.to(ops.device) for k, v in w.items()})
+    x = rnd(5, 40, seed=4)
+    got = dense(ops, part.forward(ops, x.to(ops.device), None))
+    want = plain.swiglu(x.double(), *(w[k].double() for k in ("gate_proj.weight", "up_proj.weight", "down_proj.weight")))
+    assert (got.cpu().double() - want).abs().max() < 1e-5
+
+
+@pytest.mark.parametrize("heads,kv_heads,dim,window,bias", [(4, 2, 16, None, True), (3, 1, 32, 5, True), (2, 2, 48, None, False)])
+def test_attention_part(ops, heads, kv_heads, dim, window, bias):
+    hidden = 40
+    spec = PartSpec("attention", "a.", {"hidden_size": hidden, "num_heads": heads, "num_kv_heads": kv_heads,
+                                        "head_dim": dim, "qkv_bias": bias, "window": window,
+                                        "position": PartSpec("rope", "", {"dim": dim, "theta": 1e4})})
+    part = build_part("mixer", spec)
+    assert part.cache_requirement() == PagedKV(kv_heads, dim, window)
+    w = {}
+    for i, (name, pspec) in enumerate(part.param_specs().items()):
+        w[name] = rnd(*pspec.shape, seed=10 + i, scale=0.2)
+    part.load({k: v.to(ops.device) for k, v in w.items()})
+    lengths = [9, 1, 14]
+    cache, meta = context(ops, [part.cache_requirement()], lengths)
+    x = rnd(sum(lengths), hidden, seed=5)
+    got = dense(ops, part.forward(ops, x.to(ops.device), StepContext(meta, torch.float32), cache.layer(0), True)).cpu()
+    cfg = {"num_attention_heads": heads, "num_key_value_heads": kv_heads, "head_dim": dim, "hidden_size": hidden,
+           "rope_theta": 1e4}
+    named = {"a." + k: v.double() for k, v in w.items()}
+    if not bias:
+        for n, rows in (("q", heads * dim), ("k", kv_heads * dim), ("v", kv_heads * dim)):
+            named[f"a.{n}_proj.bias"] = torch.zeros(rows, dtype=torch.float64)
+    at = 0
+    for n in lengths:
+        want = plain.self_attention(x[at:at + n].double(), named, "a.", torch.arange(n), cfg, window)
+        assert (got[at:at + n].double() - want).abs().max() < 1e-5
+        at += n
+
+
+def test_prenorm_block(ops):
+    """h += mixer(norm(h)); h += ffn(norm(h)), with the additions left to the next norm."""
+    calls = []
+
+    class Twice(Mixer):
+        def forward(self, ops, x, ctx, cache, writes_cache):
+            calls.append("mixer")
+            return x * 2
+
+    register_part("mixer", "test_twice", Twice)
+
+    class Half:
+        spec = PartSpec("half")
+
+        def param_specs(self):
+            return {}
+
+        def forward(self, ops, x, ctx):
+            calls.append("ffn")
+            return x * 0.5
+
+    norm = lambda: build_part("norm", PartSpec("rmsnorm", "", {"size": 8, "eps": 1e-6}))
+    n1, n2 = norm(), norm()
+    for n in (n1, n2):
+        n.load({"weight": torch.ones(8, device=ops.device)})
+    block = build_part("block", PartSpec("prenorm_residual"), build_part("mixer", PartSpec("test_twice")), Half(), n1, n2)
+    x = rnd(3, 8, seed=1)
+    stream = ResidualStream(x.clone().to(ops.device))
+    block.forward(ops, stream, StepContext(None, torch.float32), None, True)
+    rms = lambda t: plain.rms_norm(t, torch.ones(8), 1e-6)
+    h1 = x + 2 * rms(x)
+    assert calls == ["mixer", "ffn"]
+    assert (stream.hidden.cpu() - h1).abs().max() < 1e-5
+    assert (stream.pending.cpu() - 0.5 * rms(h1)).abs().max() < 1e-5
+
+
+# ---------------------------------------------------------------------------------------------
+# a toy mixer with state of its own: y_t = s_t, s_t = decay * s_{t-1} + x_t W, one state row a request
+# ---------------------------------------------------------------------------------------------
+class DecayMixer(Mixer):
+    def __init__(self, spec):
+        super().__init__(spec)
+        self.size = int(spec.params["hidden_size"])
+        self.decay = float(spec.params["decay"])
+        self.weight = None
+
+    def cache_requirement(self):
+        return FixedState((self.size,))
+
+    def param_specs(self):
+        return {"mix.weight": ParamSpec((self.size, self.size))}
+
+    def load(self, tensors):
+        self.weight = tensors["mix.weight"].float()
+
+    def forward(self, ops, x, ctx, cache, writes_cache):
+        meta = ctx.meta
+        u = x.float() @ self.weight.T
+        out = torch.empty_like(u)
+        slots = meta.state_slots.tolist()
+        cu = meta.cu_q.tolist()
+        for b in range(meta.num_requests):          # tokens of a request in order; the state carries over
+            s = cache.state[slots[b]]
+            for t in range(cu[b], cu[b + 1]):
+                s = self.decay * s + u[t]
+                out[t] = s
+            if writes_cache:
+                cache.state[slots[b]] = s
+        return out.to(x.dtype)
+
+
+class ToyConfig:
+    """An architecture of the test: attention and decay layers in turn, layer 0 run twice, and
+    the last call reads layer 0's cache."""
+
+    def __init__(self, hidden, vocab, decay):
+        self.hidden, self.vocab, self.decay = hidden, vocab, decay
+
+    @classmethod
+    def from_dict(cls, data):
+        return cls(data["hidden"], data["vocab"], data["decay"])
+
+    def model_spec(self):
+        norm = lambda p: PartSpec("rmsnorm", p, {"size": self.hidden, "eps": 1e-5})
+        ffn = lambda p: PartSpec("swiglu", p, {"hidden_size": self.hidden, "intermediate_size": 2 * self.hidden})
+
+        def attention(p):
+            return PartSpec("attention", p, {"hidden_size": self.hidden, "num_heads": 2, "num_kv_heads": 1,
+                                             "head_dim": self.hidden // 2, "qkv_bias": False,
+                                             "position": PartSpec("rope", "", {"dim": self.hidden // 2, "theta": 100.0})})
+
+        layers = []
+        for l, mixer in enumerate([attention("l0.attn."), PartSpec("test_decay", "l1.", {"hidden_size": self.hidden, "decay": self.decay}),
+                                   attention("l2.attn.")]):
+            layers.append(LayerSpec(PartSpec("prenorm_residual"), mixer, ffn(f"l{l}.ffn."), norm(f"l{l}.n1."), norm(f"l{l}.n2.")))
+        order = (LayerCall(0), LayerCall(1), LayerCall(2), LayerCall(2, cache_of=0))
+        return ModelSpec("ToyForCausalLM", self.vocab, self.hidden, 256, PartSpec("token_embedding", "emb."), layers, order,
+                         norm("final."), PartSpec("lm_head", "head.", {"tied": True}))
+
+
+def toy_plain(weights, cfg, ids):
+    """The toy model in plain torch (float64), whole sequence, no cache."""
+    w = {k: v.double() for k, v in weights.items()}
+    x = w["emb.weight"][torch.tensor(ids)]
+    n = len(ids)
+    att_cfg = {"num_attention_heads": 2, "num_key_value_heads": 1, "head_dim": cfg.hidden // 2, "rope_theta": 100.0}
+    zero = lambda rows: torch.zeros(rows, dtype=torch.float64)
+
+    def attention(x, p, kv_from=None):
+        named = dict(w)
+        for name, rows in (("q", cfg.hidden), ("k", cfg.hidden // 2), ("v", cfg.hidden // 2)):
+            named[p + f"{name}_proj.bias"] = zero(rows)
+        if kv_from is not None:      # keys and values of another layer's cache: its k/v of its own input
+            return kv_from
+        return plain.self_attention(x, named, p, torch.arange(n), att_cfg, None)
+
+    def ffn(x, p):
+        return plain.swiglu(x, w[p + "gate_proj.weight"], w[p + "up_proj.weight"], w[p + "down_proj.weight"])
+
+    rms = lambda t, p: plain.rms_norm(t, w[p + "weight"], 1e-5)
+    # layer 0 (its keys and values are kept for the last call)
+    n0 = rms(x, "l0.n1.")
+    x = x + attention(n0, "l0.attn.")
+    x = x + ffn(rms(x, "l0.n2."), "l0.ffn.")
+    # layer 1: decay mixer
+    u = rms(x, "l1.n1.") @ w["l1.mix.weight"].T
+    s = torch.zeros(cfg.hidden, dtype=torch.float64)
+    y = []
+    for t in range(n):
+        s = cfg.decay * s + u[t]
+        y.append(s)
+    x = x + torch.stack(y)
+    x = x + ffn(rms(x, "l1.n2."), "l1.ffn.")
+    # layer 2 with its own cache
+    x = x + attention(rms(x, "l2.n1."), "l2.attn.")
+    x = x + ffn(rms(x, "l2.n2."), "l2.ffn.")
+    # layer 2 again, reading layer 0's keys and values: q from layer 2's weights, k/v as layer 0 made them
+    n2 = rms(x, "l2.n1.")
+    d = cfg.hidden // 2
+    q = (n2 @ w["l2.attn.q_proj.weight"].T).view(n, 2, d)
+    k = (n0 @ w["l0.attn.k_proj.weight"].T).view(n, 1, d)
+    v = (n0 @ w["l0.attn.v_proj.weight"].T).view(n, 1, d)
+    cos, sin = plain.rope_cos_sin(torch.arange(n), d, 100.0, torch.float64)
+    mixed = plain.attention(plain.apply_rope(q, cos, sin), plain.apply_rope(k, cos, sin), v)
+    x = x + mixed.reshape(n, cfg.hidden) @ w["l2.attn.o_proj.weight"].T
+    x = x + ffn(rms(x, "l2.n2."), "l2.ffn.")
+    return plain.rms_norm(x, w["final.weight"], 1e-5) @ w["emb.weight"].T
+
+
+def test_toy_architecture_with_a_state_mixer_is_registered_built_and_stepped(ops):
+    register_part("mixer", "test_decay", DecayMixer)
+    register_architecture("ToyForCausalLM", ToyConfig)
+    from distie_amd.config import config_from_dict
+
+    cfg = config_from_dict({"architectures": ["ToyForCausalLM"], "hidden": 32, "vocab": 70, "decay": 0.8})
+    model = Model(cfg.model_spec())
+    specs = model.param_specs()
+    assert "l1.mix.weight" in specs and "l0.attn.q_proj.weight" in specs and "head.weight" not in specs
+    gen = torch.Generator().manual_seed(3)
+    weights = {n: (torch.ones(s.shape) if s.init == "ones" else torch.randn(s.shape, generator=gen) * 0.2)
+               for n, s in specs.items()}
+    model.load_tensors(lambda name: weights[name].to(ops.device))
+    needs = model.cache_requirements()
+    assert isinstance(needs[1], FixedState) and isinstance(needs[0], PagedKV)
+    cache = CacheManager(needs, 4, 32, 4, device=ops.device, dtype=torch.float32)
+    runner = ModelRunner(model, cache, ops, torch.float32, 256)
+    a = torch.randint(0, 70, (23,), generator=gen).tolist()
+    b = torch.randint(0, 70, (9,), generator=gen).tolist()
+    want_a, want_b = toy_plain(weights, cfg, a).float(), toy_plain(weights, cfg, b).float()
+    # whole
+    got = runner.step([StepEntry("a", a, list(range(23)))]).cpu()
+    assert (got - want_a).abs().max() < 1e-4
+    runner.finish("a")
+    # in portions, mixed with another request, the state slot taken again after a request ended
+    rows = {"a": [], "b": []}
+    plan = [[("a", 0, 5)], [("a", 5, 7), ("b", 0, 3)], [("a", 7, 20), ("b", 3, 4)], [("b", 4, 9), ("a", 20, 21)],
+            [("a", 21, 23)]]
+    seqs = {"a": a, "b": b}
+    for step in plan:
+        entries = [StepEntry(r, seqs[r][lo:hi], list(range(hi - lo))) for r, lo, hi in step]
+        logits = runner.step(entries).cpu()
+        at = 0
+        for r, lo, hi in step:
+            rows[r].append(logits[at:at + hi - lo])
+            at += hi - lo
+    assert (torch.cat(rows["a"]) - want_a).abs().max() < 1e-4
+    assert (torch.cat(rows["b"]) - want_b).abs().max() < 1e-4
+    runner.finish("a")
+    runner.finish("b")
+    cache.check()
+    assert cache.slots.num_free == 4
+    # a new request in a used slot starts from a zero state
+    got = runner.step([StepEntry("c", b, list(range(9)))]).cpu()
+    assert (got - want_b).abs().max() < 1e-4
