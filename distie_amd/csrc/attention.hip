@@ -400,10 +400,14 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_mfma_kernel(
   }
 }
 
-// Combines the partial results of the runs of keys of one (request, head): grid (heads, requests).
+// Combines the partial results of the runs of keys of one (request, head): grid (heads, requests), one wave.
+// The lanes first take one run each to find the maximum and the weights of the runs, then each lane owns
+// output dims and adds the runs in order, four loads in flight at a time.
 __global__ __launch_bounds__(DISTIE_WAVE) void attn_reduce_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ cu_q, bf16_t* __restrict__ out, int heads, int window, int split_len, int max_splits) {
+  __shared__ float weight_s[DISTIE_WAVE];
+  const int lane = threadIdx.x;
   const int request = blockIdx.y;
   const int head = blockIdx.x;
   const int token = cu_q[request];
@@ -412,27 +416,51 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_reduce_kernel(
   const int s_first = first / split_len;
   const int s_last = q_pos / split_len;
   const int64_t base = (static_cast<int64_t>(request) * heads + head) * max_splits;
-  float m = -INFINITY;
-  for (int s = s_first; s <= s_last; ++s) m = fmaxf(m, part_ml[2 * (base + s)]);
-  float l = 0.f;
   float acc[DIMS_PER_LANE];
 #pragma unroll
   for (int i = 0; i < DIMS_PER_LANE; ++i) acc[i] = 0.f;
-  for (int s = s_first; s <= s_last; ++s) {
-    const float w = expf(part_ml[2 * (base + s)] - m);
-    l += w * part_ml[2 * (base + s) + 1];
-    const float* po = part_o + (base + s) * D;
+  // the maximum over all runs
+  float m = -INFINITY;
+  for (int s = s_first + lane; s <= s_last; s += DISTIE_WAVE) m = fmaxf(m, part_ml[2 * (base + s)]);
+  m = wave_max(m);
+  float l = 0.f;
+  for (int s0 = s_first; s0 <= s_last; s0 += DISTIE_WAVE) {
+    const int mine = s0 + lane;
+    float w = 0.f, wl = 0.f;
+    if (mine <= s_last) {
+      w = expf(part_ml[2 * (base + mine)] - m);
+      wl = w * part_ml[2 * (base + mine) + 1];
+    }
+    l += wl;                                  // summed over the lanes at the end
+    __syncthreads();
+    weight_s[lane] = w;
+    __syncthreads();
+    const int n = min(DISTIE_WAVE, s_last - s0 + 1);
+    const float* po = part_o + (base + s0) * D;
 #pragma unroll
     for (int i = 0; i < DIMS_PER_LANE; ++i) {
-      const int d = threadIdx.x + i * DISTIE_WAVE;
-      if (d < D) acc[i] = fmaf(w, po[d], acc[i]);
+      const int d = lane + i * DISTIE_WAVE;
+      if (d >= D) continue;
+      float a = acc[i];
+      int j = 0;
+      for (; j + 4 <= n; j += 4) {
+        const float v0 = po[static_cast<int64_t>(j) * D + d], v1 = po[static_cast<int64_t>(j + 1) * D + d];
+        const float v2 = po[static_cast<int64_t>(j + 2) * D + d], v3 = po[static_cast<int64_t>(j + 3) * D + d];
+        a = fmaf(weight_s[j], v0, a);
+        a = fmaf(weight_s[j + 1], v1, a);
+        a = fmaf(weight_s[j + 2], v2, a);
+        a = fmaf(weight_s[j + 3], v3, a);
+      }
+      for (; j < n; ++j) a = fmaf(weight_s[j], po[static_cast<int64_t>(j) * D + d], a);
+      acc[i] = a;
     }
   }
+  l = wave_sum(l);
   bf16_t* o = out + (static_cast<int64_t>(token) * heads + head) * D;
   const float inv = 1.f / l;
 #pragma unroll
   for (int i = 0; i < DIMS_PER_LANE; ++i) {
-    const int d = threadIdx.x + i * DISTIE_WAVE;
+    const int d = lane + i * DISTIE_WAVE;
     if (d < D) o[d] = static_cast<bf16_t>(acc[i] * inv);
   }
 }

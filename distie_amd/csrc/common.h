@@ -52,6 +52,26 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return total;
 }
 
+// Sum of `slices` values that lie `stride` elements apart, added in order. The loads of four slices are
+// issued together, so the sum costs a few memory round trips instead of one per slice.
+template <typename T>
+__device__ __forceinline__ float sum_strided(const T* p, int slices, int64_t stride) {
+  float sum = to_float(p[0]);
+  int s = 1;
+  for (; s + 4 <= slices; s += 4) {
+    const float a = to_float(p[s * stride]);
+    const float b = to_float(p[(s + 1) * stride]);
+    const float c = to_float(p[(s + 2) * stride]);
+    const float d = to_float(p[(s + 3) * stride]);
+    sum += a;
+    sum += b;
+    sum += c;
+    sum += d;
+  }
+  for (; s < slices; ++s) sum += to_float(p[s * stride]);
+  return sum;
+}
+
 static inline int launch_status() { return static_cast<int>(hipGetLastError()); }
 
 // Calls `body` with a value of the element type that `code` names.

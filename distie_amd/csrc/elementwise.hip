@@ -47,9 +47,7 @@ __global__ void rmsnorm_kernel(float* __restrict__ residual, const D* __restrict
   if (delta != nullptr) {
     const D* d = delta + row * width;
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
-      float sum = to_float(d[i]);
-      for (int s = 1; s < slices; ++s) sum += to_float(d[s * slice_stride + i]);
-      const float v = x[i] + sum;
+      const float v = x[i] + sum_strided(d + i, slices, slice_stride);
       x[i] = v;
       ss += v * v;
     }
@@ -69,7 +67,9 @@ __global__ void rmsnorm_kernel(float* __restrict__ residual, const D* __restrict
 template <typename D, typename W>
 static int rmsnorm_launch_out(float* residual, const D* delta, int slices, const W* weight, void* out,
                               int out_dtype, int rows, int width, float eps, hipStream_t stream) {
-  const int threads = width >= 2048 ? 512 : (width >= 512 ? 256 : 64);
+  // with slices to add, a thread's work is a chain of loads: spread a row over more threads
+  int threads = width >= 2048 ? 512 : (width >= 512 ? 256 : 64);
+  if (slices > 1) threads = width >= 1024 ? 1024 : (width >= 512 ? 512 : threads);
   DISTIE_DISPATCH(out_dtype, O,
                   rmsnorm_kernel<D, W, O><<<rows, threads, 0, stream>>>(
                       residual, delta, slices, static_cast<int64_t>(rows) * width, weight, static_cast<O*>(out), width, eps));
@@ -108,11 +108,7 @@ __global__ void rope_kv_write_kernel(const I* in, int slices, int64_t slice_stri
   const int64_t slot = write ? slots[t] : 0;
   const int64_t page = slot / block_size;
   const int offset = static_cast<int>(slot % block_size);
-  auto value = [&](int64_t i) {
-    float sum = to_float(src[i]);
-    for (int s = 1; s < slices; ++s) sum += to_float(src[s * slice_stride + i]);
-    return sum;
-  };
+  auto value = [&](int64_t i) { return sum_strided(src + i, slices, slice_stride); };
   // q and k heads: every thread owns whole pairs, so `out` may alias `in`
   const int rotated_heads = heads + kv_heads;
   const int half = dim / 2;
@@ -162,7 +158,8 @@ extern "C" int distie_rope_kv_write(const void* in, int in_dtype, int slices, vo
   if (pairs > 0 && inv_freq == nullptr) return DISTIE_BAD_ARGUMENT;
   if (in == out && (slices != 1 || in_dtype != dtype)) return DISTIE_BAD_ARGUMENT;
   const int work = (heads + kv_heads) * dim / 2;
-  const int threads = work >= 512 ? 256 : (work >= 128 ? 128 : 64);
+  int threads = work >= 512 ? 256 : (work >= 128 ? 128 : 64);
+  if (slices > 1 && work >= 512) threads = work >= 1024 ? 1024 : 512;
   const int64_t stride = static_cast<int64_t>(tokens) * (heads + 2 * kv_heads) * dim;
   DISTIE_DISPATCH(in_dtype, I, DISTIE_DISPATCH(dtype, T, DISTIE_DISPATCH(cache_dtype, C,
       rope_kv_write_kernel<I, T, C><<<tokens, threads, 0, stream>>>(
@@ -183,12 +180,8 @@ __global__ void silu_mul_kernel(const I* __restrict__ gate_up, int slices, int64
     const int64_t r = i / inter;
     const int c = static_cast<int>(i % inter);
     const I* p = gate_up + r * 2 * inter + c;
-    float g = to_float(p[0]);
-    float u = to_float(p[inter]);
-    for (int s = 1; s < slices; ++s) {
-      g += to_float(p[s * slice_stride]);
-      u += to_float(p[s * slice_stride + inter]);
-    }
+    const float g = sum_strided(p, slices, slice_stride);
+    const float u = sum_strided(p + inter, slices, slice_stride);
     out[i] = from_float<T>(g / (1.f + expf(-g)) * u);
   }
 }
@@ -210,9 +203,7 @@ template <typename T>
 __global__ void sum_slices_kernel(const float* __restrict__ in, int slices, int64_t count, T* __restrict__ out) {
   for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < count;
        i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-    float sum = in[i];
-    for (int s = 1; s < slices; ++s) sum += in[s * count + i];
-    out[i] = from_float<T>(sum);
+    out[i] = from_float<T>(sum_strided(in + i, slices, count));
   }
 }
 
