@@ -190,6 +190,7 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_mfma_kernel(
     request = blockIdx.z;
     kh = blockIdx.y;
     token0 = cu_q[request];
+    if (cu_q[request + 1] - token0 != 1) return;      // a portion of a prompt: the tiled kernel's
     columns = group;
     const int q_pos = positions[token0];
     const int first = window > 0 ? max(0, q_pos - window + 1) : 0;
@@ -411,6 +412,7 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_reduce_kernel(
   const int request = blockIdx.y;
   const int head = blockIdx.x;
   const int token = cu_q[request];
+  if (cu_q[request + 1] - token != 1) return;
   const int q_pos = positions[token];
   const int first = window > 0 ? max(0, q_pos - window + 1) : 0;
   const int s_first = first / split_len;
@@ -469,8 +471,8 @@ constexpr int MFMA_MAX_MB = (D <= 128) ? 4 : 2;     // registers: the output til
 
 extern "C" int distie_attention_mfma_columns() { return 16 * MFMA_MAX_MB; }
 
-// Prefill and mixed steps. bfloat16 only; block_size must be a multiple of 16.
-extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, const void* k_cache, const void* v_cache,
+// The register-only kernel in prefill mode (kept for comparison). bfloat16 only; block_size a multiple of 16.
+extern "C" int distie_attention_prefill_simple_bf16(const void* qkv, int64_t q_stride, const void* k_cache, const void* v_cache,
                                              const int32_t* positions, const int32_t* cu_q, const int32_t* block_table,
                                              int table_width, void* out, int tokens, int num_requests, int heads,
                                              int kv_heads, int block_size, float scale, int window,
@@ -489,7 +491,7 @@ extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, 
   return launch_status();
 }
 
-// Steps in which every request brings one token. part_o: float32 [requests, heads, max_splits, D],
+// The requests of a step that bring one token (others are skipped). part_o: float32 [requests, heads, max_splits, D],
 // part_ml: float32 [requests, heads, max_splits, 2]; max_splits * split_len must cover every position.
 extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, const void* k_cache, const void* v_cache,
                                             const int32_t* positions, const int32_t* cu_q, const int32_t* block_table,
@@ -524,5 +526,289 @@ extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, c
   if (status != 0) return status;
   attn_reduce_kernel<<<dim3(heads, num_requests), DISTIE_WAVE, 0, stream>>>(
       part_o, part_ml, positions, cu_q, static_cast<bf16_t*>(out), heads, window, split_len, max_splits);
+  return launch_status();
+}
+
+
+// ===================================================================================================
+//  * attn_prefill: the tiled kernel for portions of prompts. A workgroup of four waves owns PF_BM
+//    consecutive new tokens of one request and one head; it walks over the keys 64 at a time. The K tile
+//    [64, D] and the V^T tile [D, 64] are put into LDS once per workgroup (global loads of the next tile
+//    are in flight while the current one is used) and every wave multiplies its own 16 * PF_MB query
+//    columns against them with the same two products and the same register layout as attn_mfma.
+//    Requests that bring fewer than `min_q_len` tokens are left to the decode kernel.
+// ===================================================================================================
+constexpr int PF_BN = 64;                               // keys per tile
+constexpr int PF_WAVES = 4;
+constexpr int PF_THREADS = PF_WAVES * DISTIE_WAVE;
+constexpr int PF_MB = (D <= 128) ? 2 : 1;               // blocks of 16 query columns per wave
+constexpr int PF_WAVE_COLS = 16 * PF_MB;
+constexpr int PF_BM = PF_WAVES * PF_WAVE_COLS;          // query tokens per workgroup
+constexpr int PF_K_STRIDE = D + 8;                      // elements; the padding spreads rows over the banks
+constexpr int PF_V_STRIDE = PF_BN + 8;
+constexpr int PF_K_CHUNKS = PF_BN * D / 8;              // 16-byte pieces of a K tile
+constexpr int PF_V_CHUNKS = D * PF_BN / 8;
+constexpr int PF_K_PER_THREAD = (PF_K_CHUNKS + PF_THREADS - 1) / PF_THREADS;
+constexpr int PF_V_PER_THREAD = (PF_V_CHUNKS + PF_THREADS - 1) / PF_THREADS;
+
+__global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
+    const bf16_t* __restrict__ qkv, int64_t q_stride, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ positions, const int32_t* __restrict__ cu_q,
+    const int32_t* __restrict__ block_table, int table_width, bf16_t* __restrict__ out, int num_requests, int heads,
+    int kv_heads, int block_size, float scale, int window, int min_q_len) {
+  __shared__ __attribute__((aligned(16))) bf16_t k_lds[PF_BN * PF_K_STRIDE];
+  __shared__ __attribute__((aligned(16))) bf16_t v_lds[D * PF_V_STRIDE];
+  const int tid = threadIdx.x;
+  const int wave = tid / DISTIE_WAVE;
+  const int lane = tid % DISTIE_WAVE;
+  const int r = lane % 16;
+  const int g = lane / 16;
+  const int group = heads / kv_heads;
+
+  // ---- which tokens: blockIdx.x counts tiles of PF_BM tokens over the requests that are served here
+  int tile = blockIdx.x;
+  int request = 0, begin = 0, end = 0;
+  for (; request < num_requests; ++request) {
+    begin = cu_q[request];
+    end = cu_q[request + 1];
+    if (end - begin < min_q_len) continue;
+    const int tiles = (end - begin + PF_BM - 1) / PF_BM;
+    if (tile < tiles) break;
+    tile -= tiles;
+  }
+  if (request >= num_requests) return;
+  const int head = blockIdx.y;
+  const int kh = head / group;
+  const int token0 = begin + tile * PF_BM;
+  const int columns = min(PF_BM, end - token0);           // of the workgroup
+  const int pos0 = positions[token0];                     // the tokens of a portion have consecutive positions
+  const int key_begin = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int key_end = pos0 + columns - 1;
+  const int32_t* table = block_table + static_cast<int64_t>(request) * table_width;
+
+  // ---- this wave's columns
+  const int wave_col0 = wave * PF_WAVE_COLS;
+  const int wave_cols = max(0, min(PF_WAVE_COLS, columns - wave_col0));
+  const int wave_last = pos0 + wave_col0 + wave_cols - 1;
+  const int wave_first = window > 0 ? max(0, pos0 + wave_col0 - window + 1) : 0;
+  int col_pos[PF_MB];
+  bf16x8 q_reg[PF_MB][DK32 > 0 ? DK32 : 1];
+  shortx4 q_tail[PF_MB];
+#pragma unroll
+  for (int mb = 0; mb < PF_MB; ++mb) {
+    const int col = min(wave_col0 + 16 * mb + r, columns - 1);    // columns past the end repeat the last; dropped later
+    col_pos[mb] = pos0 + col;
+    const bf16_t* q = qkv + (token0 + col) * q_stride + static_cast<int64_t>(head) * D;
+#pragma unroll
+    for (int dk = 0; dk < DK32; ++dk) q_reg[mb][dk] = *reinterpret_cast<const bf16x8*>(q + 32 * dk + 8 * g);
+    if (DK_TAIL) q_tail[mb] = *reinterpret_cast<const shortx4*>(q + (D - 16) + 4 * g);
+  }
+  floatx4 o_acc[PF_MB][DB16];
+  float m_run[PF_MB], l_run[PF_MB];
+#pragma unroll
+  for (int mb = 0; mb < PF_MB; ++mb) {
+    m_run[mb] = -INFINITY;
+    l_run[mb] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DB16; ++db) o_acc[mb][db] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // ---- staging of one tile in registers: 16-byte pieces of K rows and of V^T rows
+  uint4 k_stage[PF_K_PER_THREAD], v_stage[PF_V_PER_THREAD];
+  auto fetch = [&](int k0) {
+    // the four blocks of 16 keys of the tile: live if they overlap the keys this workgroup reads
+    int64_t base[4];
+    int offset[4];
+    bool live[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int key = k0 + 16 * b;
+      live[b] = key <= key_end && key + 15 >= key_begin;
+      base[b] = 0;
+      offset[b] = 0;
+      if (live[b]) {
+        const int page = table[key / block_size];
+        base[b] = (static_cast<int64_t>(page) * kv_heads + kh) * block_size * D;
+        offset[b] = key % block_size;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < PF_K_PER_THREAD; ++i) {
+      const int c = tid + i * PF_THREADS;
+      k_stage[i] = uint4{0u, 0u, 0u, 0u};
+      if (c < PF_K_CHUNKS) {
+        const int row = c / (D / 8);
+        const int piece = c % (D / 8);
+        const int b = row / 16;
+        if (live[b])
+          k_stage[i] = *reinterpret_cast<const uint4*>(k_cache + base[b] + static_cast<int64_t>(offset[b] + row % 16) * D + 8 * piece);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < PF_V_PER_THREAD; ++i) {
+      const int c = tid + i * PF_THREADS;
+      v_stage[i] = uint4{0u, 0u, 0u, 0u};
+      if (c < PF_V_CHUNKS) {
+        const int d = c / 8;
+        const int piece = c % 8;              // 8 keys each
+        const int b = piece / 2;
+        if (live[b]) {
+          uint4 raw = *reinterpret_cast<const uint4*>(v_cache + base[b] + static_cast<int64_t>(d) * block_size + offset[b] + 8 * (piece % 2));
+          // slots after the last key of this workgroup were not written by this request: cleared (0 * NaN)
+          const int written = key_end - (k0 + 8 * piece) + 1;
+          if (written < 8) {
+            uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              w[e] = written >= 2 * e + 2 ? w[e] : (written == 2 * e + 1 ? (w[e] & 0x0000ffffu) : 0u);
+            raw = uint4{w[0], w[1], w[2], w[3]};
+          }
+          v_stage[i] = raw;
+        }
+      }
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < PF_K_PER_THREAD; ++i) {
+      const int c = tid + i * PF_THREADS;
+      if (c < PF_K_CHUNKS) *reinterpret_cast<uint4*>(k_lds + (c / (D / 8)) * PF_K_STRIDE + 8 * (c % (D / 8))) = k_stage[i];
+    }
+#pragma unroll
+    for (int i = 0; i < PF_V_PER_THREAD; ++i) {
+      const int c = tid + i * PF_THREADS;
+      if (c < PF_V_CHUNKS) *reinterpret_cast<uint4*>(v_lds + (c / 8) * PF_V_STRIDE + 8 * (c % 8)) = v_stage[i];
+    }
+  };
+
+  const int tile0 = key_begin / PF_BN * PF_BN;
+  fetch(tile0);
+  for (int k0 = tile0; k0 <= key_end; k0 += PF_BN) {
+    __syncthreads();                       // every wave is done with the tile in LDS
+    stash();
+    __syncthreads();
+    if (k0 + PF_BN <= key_end) fetch(k0 + PF_BN);      // in flight while this tile is used
+    if (wave_cols <= 0 || k0 > wave_last || k0 + PF_BN - 1 < wave_first) continue;
+
+    // ---- scores: 64 keys x the wave's columns
+    floatx4 s[PF_MB][4];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+#pragma unroll
+      for (int mb = 0; mb < PF_MB; ++mb) s[mb][kb] = floatx4{0.f, 0.f, 0.f, 0.f};
+      const bf16_t* k_row = k_lds + (16 * kb + r) * PF_K_STRIDE;
+#pragma unroll
+      for (int dk = 0; dk < DK32; ++dk) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(k_row + 32 * dk + 8 * g);
+#pragma unroll
+        for (int mb = 0; mb < PF_MB; ++mb)
+          s[mb][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q_reg[mb][dk], s[mb][kb], 0, 0, 0);
+      }
+      if (DK_TAIL) {
+        const shortx4 a = *reinterpret_cast<const shortx4*>(k_row + (D - 16) + 4 * g);
+#pragma unroll
+        for (int mb = 0; mb < PF_MB; ++mb) {
+          const floatx4 tail = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, q_tail[mb], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) s[mb][kb][i] += tail[i];
+        }
+      }
+    }
+    // ---- softmax step per column
+    bf16x8 p_reg[PF_MB][2];
+    float alpha[PF_MB];
+#pragma unroll
+    for (int mb = 0; mb < PF_MB; ++mb) {
+      const int last = col_pos[mb];
+      const int first = window > 0 ? max(0, last - window + 1) : 0;
+      float best = -INFINITY;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = k0 + 16 * kb + 4 * g + i;
+          const float v = (key >= first && key <= last) ? s[mb][kb][i] * scale : -INFINITY;
+          s[mb][kb][i] = v;
+          best = fmaxf(best, v);
+        }
+      best = fmaxf(best, __shfl_xor(best, 16, DISTIE_WAVE));
+      best = fmaxf(best, __shfl_xor(best, 32, DISTIE_WAVE));
+      const float m_new = fmaxf(m_run[mb], best);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      alpha[mb] = expf(m_run[mb] - m_safe);
+      float sum = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float p = expf(s[mb][kb][i] - m_safe);
+          sum += p;
+          p_reg[mb][kb / 2][4 * (kb % 2) + i] = static_cast<bf16_t>(p);
+        }
+      l_run[mb] = l_run[mb] * alpha[mb] + sum;
+      m_run[mb] = m_new;
+    }
+#pragma unroll
+    for (int mb = 0; mb < PF_MB; ++mb) {
+      float a4[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a4[i] = __shfl(alpha[mb], 4 * g + i, DISTIE_WAVE);
+#pragma unroll
+      for (int db = 0; db < DB16; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o_acc[mb][db][i] *= a4[i];
+    }
+    // ---- O += P . V: two steps of 32 keys, each the pair of 16-key blocks (2 ks, 2 ks + 1)
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int db = 0; db < DB16; ++db) {
+        const bf16_t* v_row = v_lds + (16 * db + r) * PF_V_STRIDE + 32 * ks + 4 * g;
+        const uint2 lo = *reinterpret_cast<const uint2*>(v_row);
+        const uint2 hi = *reinterpret_cast<const uint2*>(v_row + 16);
+        const uintx4 words = {lo.x, lo.y, hi.x, hi.y};
+        const bf16x8 v = __builtin_bit_cast(bf16x8, words);
+#pragma unroll
+        for (int mb = 0; mb < PF_MB; ++mb)
+          o_acc[mb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_reg[mb][ks], v, o_acc[mb][db], 0, 0, 0);
+      }
+  }
+
+  // ---- write: the lane holds columns 4g..4g+3 of each block, output dim 16 db + r
+#pragma unroll
+  for (int mb = 0; mb < PF_MB; ++mb) {
+    l_run[mb] += __shfl_xor(l_run[mb], 16, DISTIE_WAVE);
+    l_run[mb] += __shfl_xor(l_run[mb], 32, DISTIE_WAVE);
+  }
+#pragma unroll
+  for (int mb = 0; mb < PF_MB; ++mb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int col = 16 * mb + 4 * g + i;
+      const float l_col = __shfl(l_run[mb], 4 * g + i, DISTIE_WAVE);
+      if (col >= wave_cols) continue;
+      bf16_t* o = out + (static_cast<int64_t>(token0 + wave_col0 + col) * heads + head) * D;
+      const float inv = 1.f / l_col;
+#pragma unroll
+      for (int db = 0; db < DB16; ++db) o[16 * db + r] = static_cast<bf16_t>(o_acc[mb][db][i] * inv);
+    }
+}
+
+// Portions of prompts (and whole mixed steps). bfloat16 only; block_size must be a multiple of 16. Requests that
+// bring fewer than min_q_len tokens are skipped (the decode kernel serves them).
+extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, const void* k_cache, const void* v_cache,
+                                             const int32_t* positions, const int32_t* cu_q, const int32_t* block_table,
+                                             int table_width, void* out, int tokens, int num_requests, int heads,
+                                             int kv_heads, int block_size, float scale, int window, int min_q_len,
+                                             hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size % 16 != 0 || table_width < 1 || window < 0 ||
+      num_requests < 1 || heads > 65535 || min_q_len < 1)
+    return DISTIE_BAD_ARGUMENT;
+  const int tiles = (tokens + PF_BM - 1) / PF_BM + num_requests;     // an upper bound; spare blocks leave at once
+  attn_prefill_kernel<<<dim3(tiles, heads), PF_THREADS, 0, stream>>>(
+      static_cast<const bf16_t*>(qkv), q_stride, static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),
+      positions, cu_q, block_table, table_width, static_cast<bf16_t*>(out), num_requests, heads, kv_heads, block_size,
+      scale, window, min_q_len);
   return launch_status();
 }

@@ -53,10 +53,61 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void argmax_kernel(const float* __r
   if (threadIdx.x == 0) out[blockIdx.x] = best.index;
 }
 
-extern "C" int distie_argmax(const float* logits, int32_t* out, int rows, int vocab, hipStream_t stream) {
+// Large vocabularies: a row is cut into `parts` pieces (grid: parts x rows), each block writes the best of its
+// piece, and a second launch takes the best of the pieces (lowest index among equals, as everywhere).
+__global__ __launch_bounds__(SAMPLE_THREADS) void argmax_pieces_kernel(const float* __restrict__ logits,
+                                                                       float* __restrict__ piece_value,
+                                                                       int32_t* __restrict__ piece_index, int vocab,
+                                                                       int piece_len) {
+  __shared__ Best scratch[SAMPLE_THREADS / DISTIE_WAVE];
+  const float* row = logits + static_cast<int64_t>(blockIdx.y) * vocab;
+  const int begin = blockIdx.x * piece_len;
+  const int end = min(vocab, begin + piece_len);
+  Best mine{-INFINITY, 0x7fffffff};
+  for (int i = begin + threadIdx.x; i < end; i += blockDim.x) mine = better(mine, Best{row[i], i});
+  const Best best = block_best(mine, scratch);
+  if (threadIdx.x == 0) {
+    piece_value[blockIdx.y * gridDim.x + blockIdx.x] = best.value;
+    piece_index[blockIdx.y * gridDim.x + blockIdx.x] = best.index;
+  }
+}
+
+__global__ __launch_bounds__(DISTIE_WAVE) void argmax_combine_kernel(const float* __restrict__ piece_value,
+                                                                     const int32_t* __restrict__ piece_index,
+                                                                     int32_t* __restrict__ out, int parts, int vocab) {
+  Best mine{-INFINITY, 0x7fffffff};
+  for (int i = threadIdx.x; i < parts; i += DISTIE_WAVE)
+    mine = better(mine, Best{piece_value[blockIdx.x * parts + i], piece_index[blockIdx.x * parts + i]});
+#pragma unroll
+  for (int o = DISTIE_WAVE / 2; o > 0; o >>= 1) {
+    Best other{__shfl_xor(mine.value, o, DISTIE_WAVE), __shfl_xor(mine.index, o, DISTIE_WAVE)};
+    mine = better(mine, other);
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = mine.index < vocab ? mine.index : 0;
+}
+
+// pieces a row is cut into (1 = the single-launch kernel); the caller sizes the scratch from it
+extern "C" int distie_argmax_parts(int rows, int vocab) {
+  if (vocab < 16384) return 1;
+  int parts = 1024 / (rows < 1 ? 1 : rows);
+  if (parts > vocab / 4096) parts = vocab / 4096;
+  return parts < 2 ? 1 : (parts > 64 ? 64 : parts);
+}
+
+// scratch: float [rows * parts] and int32 [rows * parts]; may be null when distie_argmax_parts is 1
+extern "C" int distie_argmax(const float* logits, int32_t* out, int rows, int vocab, float* piece_value,
+                             int32_t* piece_index, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (vocab <= 0) return DISTIE_BAD_ARGUMENT;
-  argmax_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, out, vocab);
+  const int parts = distie_argmax_parts(rows, vocab);
+  if (parts == 1) {
+    argmax_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, out, vocab);
+    return launch_status();
+  }
+  if (piece_value == nullptr || piece_index == nullptr) return DISTIE_BAD_ARGUMENT;
+  const int piece_len = (vocab + parts - 1) / parts;
+  argmax_pieces_kernel<<<dim3(parts, rows), SAMPLE_THREADS, 0, stream>>>(logits, piece_value, piece_index, vocab, piece_len);
+  argmax_combine_kernel<<<rows, DISTIE_WAVE, 0, stream>>>(piece_value, piece_index, out, parts, vocab);
   return launch_status();
 }
 

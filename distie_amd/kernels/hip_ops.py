@@ -91,7 +91,8 @@ class HipOps(Ops):
         o.distie_gemm_generic.argtypes = [_P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _P]
         o.distie_gemm_skinny_slices.argtypes = [_I, _I, _I]
         o.distie_gemm_skinny_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _P]
-        o.distie_argmax.argtypes = [_P, _P, _I, _I, _P]
+        o.distie_argmax.argtypes = [_P, _P, _I, _I, _P, _P, _P]
+        o.distie_argmax_parts.argtypes = [_I, _I]
         o.distie_sample.argtypes = [_P, _P, _P, _P, _P, _I, _I, _P]
 
     def graphs_supported(self) -> bool:
@@ -111,7 +112,9 @@ class HipOps(Ops):
             lib.distie_attention_generic.argtypes = [_P, _I, _L, _P, _P, _I, _P, _P, _P, _I, _P,
                                                      _I, _I, _I, _I, _F, _I, _P]
             lib.distie_attention_prefill_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I,
-                                                          _F, _I, _P]
+                                                          _F, _I, _I, _P]
+            lib.distie_attention_prefill_simple_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I,
+                                                                 _I, _F, _I, _P]
             lib.distie_attention_decode_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I,
                                                          _I, _F, _I, _I, _I, _P]
             if lib.distie_attention_head_dim() != head_dim:
@@ -258,9 +261,14 @@ class HipOps(Ops):
         bf16 = qkv.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16
         if bf16 and meta.block_size % 16 == 0:
             group = num_heads // num_kv_heads
-            if meta.all_decode and group <= lib.distie_attention_mfma_columns():
-                # keys are cut into runs, one wave each: enough waves to fill the chip when few requests decode
-                runs = max(1, min(64, 4096 // (meta.num_requests * num_kv_heads)))
+            singles = meta.num_requests if meta.all_decode else 0
+            if not meta.all_decode and meta.host_cu_q is not None:
+                singles = int((meta.host_cu_q[1:] - meta.host_cu_q[:-1] == 1).sum())
+            split_decode = singles > 0 and group <= lib.distie_attention_mfma_columns()
+            if split_decode:
+                # requests that bring one token: keys are cut into runs, one wave each, so that the chip is
+                # filled even when few requests decode
+                runs = max(1, min(64, 4096 // (singles * num_kv_heads)))
                 split_len = max(64, -(-meta.max_kv // runs + 31) // 32 * 32)
                 max_splits = -(-meta.max_kv // split_len)
                 part_o = torch.empty((meta.num_requests, num_heads, max_splits, head_dim), dtype=torch.float32,
@@ -272,12 +280,19 @@ class HipOps(Ops):
                     meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], out.data_ptr(), part_o.data_ptr(),
                     part_ml.data_ptr(), meta.num_requests, num_heads, num_kv_heads, meta.block_size, float(scale),
                     int(window or 0), split_len, max_splits, self._stream()), "attention_decode_bf16")
-                return out
-            _check(lib.distie_attention_prefill_bf16(
-                qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), meta.positions.data_ptr(),
-                meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], out.data_ptr(), T, meta.num_requests,
-                num_heads, num_kv_heads, meta.block_size, float(scale), int(window or 0), self._stream()),
-                "attention_prefill_bf16")
+            if singles < meta.num_requests:
+                # portions of prompts (and single tokens too, if the decode kernel did not take them)
+                _check(lib.distie_attention_prefill_bf16(
+                    qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), meta.positions.data_ptr(),
+                    meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], out.data_ptr(), T, meta.num_requests,
+                    num_heads, num_kv_heads, meta.block_size, float(scale), int(window or 0),
+                    2 if split_decode else 1, self._stream()), "attention_prefill_bf16")
+            elif not split_decode:
+                _check(lib.distie_attention_prefill_bf16(
+                    qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), meta.positions.data_ptr(),
+                    meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], out.data_ptr(), T, meta.num_requests,
+                    num_heads, num_kv_heads, meta.block_size, float(scale), int(window or 0), 1, self._stream()),
+                    "attention_prefill_bf16")
             return out
         _check(lib.distie_attention_generic(
             qkv.data_ptr(), _code(qkv), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), _code(k_cache),
@@ -309,9 +324,16 @@ class HipOps(Ops):
         self._own(logits)
         if logits.dtype != torch.float32:
             raise KernelError("argmax reads float32 logits")
-        out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
-        _check(self._ops.distie_argmax(logits.data_ptr(), out.data_ptr(), logits.shape[0], logits.shape[1],
-                                       self._stream()), "argmax")
+        rows, vocab = logits.shape
+        out = torch.empty(rows, dtype=torch.int32, device=self.device)
+        parts = self._ops.distie_argmax_parts(rows, vocab)
+        values = indexes = None
+        if parts > 1:
+            values = torch.empty(rows * parts, dtype=torch.float32, device=self.device)
+            indexes = torch.empty(rows * parts, dtype=torch.int32, device=self.device)
+        _check(self._ops.distie_argmax(logits.data_ptr(), out.data_ptr(), rows, vocab,
+                                       values.data_ptr() if parts > 1 else None,
+                                       indexes.data_ptr() if parts > 1 else None, self._stream()), "argmax")
         return out
 
     def sample(self, logits, temperature, seeds, counters):

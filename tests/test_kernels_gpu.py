@@ -4,6 +4,7 @@ are no power of two, grouped heads, odd page sizes)."""
 
 import math
 
+import numpy as np
 import pytest
 import torch
 
@@ -154,7 +155,8 @@ def make_meta(positions, token_request, cu_q, kv_len, tables, slots, block_size)
                      token_request=i32(token_request), cu_q=i32(cu_q), kv_len=i32(kv_len),
                      state_slots=i32([0] * B), max_q=max(b - a for a, b in zip(cu_q, cu_q[1:])),
                      max_kv=max(kv_len), block_size=block_size,
-                     groups=[GroupMeta(block_table=i32(tables), slots=i32(slots))])
+                     groups=[GroupMeta(block_table=i32(tables), slots=i32(slots))],
+                     host_cu_q=np.asarray(cu_q), all_decode=all(b - a == 1 for a, b in zip(cu_q, cu_q[1:])))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -232,12 +234,29 @@ def test_paged_attention(ops, dtype, heads, kv_heads, dim, P, window):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,dim,P,window", [(4, 2, 16, 16, None), (3, 1, 48, 16, 100), (12, 2, 128, 16, None),
+                                                         (2, 1, 256, 32, 300), (6, 2, 64, 64, 70)])
+def test_paged_attention_long_portions(ops, dtype, heads, kv_heads, dim, P, window):
+    """Portions that span several tiles of queries and of keys, with and without a past; and the
+    tiled kernel taking the single tokens too."""
+    lens, q_lens = [520, 260, 131, 400], [300, 260, 1, 129]
+    meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, lens, q_lens, dtype, seed=3)
+    want = TorchOps("cuda").paged_attention(qkv.double(), meta, 0, k.double(), v.double(), heads, kv_heads, dim,
+                                            dim ** -0.5, window)
+    got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
+    close(got, want, dtype, scale=want.abs().max().item())
+    meta.host_cu_q = None
+    got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
+    close(got, want, dtype, scale=want.abs().max().item())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,kv_heads,dim,P,window", ATTENTION_SHAPES)
 def test_paged_attention_decode_step(ops, dtype, heads, kv_heads, dim, P, window):
     """Every request brings one token (the split-key kernel in bfloat16), contexts from 1 to 700."""
     lens = [1, 2, 16, 17, 64, 65, 129, 300, 700]
     meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, lens, [1] * len(lens), dtype)
-    meta.all_decode = True
+    assert meta.all_decode
     want = TorchOps("cuda").paged_attention(qkv.double(), meta, 0, k.double(), v.double(), heads, kv_heads, dim,
                                             dim ** -0.5, window)
     got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
@@ -264,6 +283,7 @@ def test_attention_finds_one_far_key(ops, dtype):
         want = v[page, :, :, far % P].float().repeat_interleave(2, dim=0).reshape(1, -1)
         for decode in (False, True):
             meta.all_decode = decode
+            meta.host_cu_q = np.asarray([0, 1]) if decode else None      # None: the tiled kernel takes the single token
             got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
             close(got, want, dtype, scale=4.0)
     # just outside the window the key must not count
@@ -295,6 +315,10 @@ def test_argmax_and_sample(ops):
     logits[2, 1000] = 60.0
     got = ops.argmax(logits)
     assert got.tolist() == [int(r.argmax()) for r in logits[:1]] + [7, 1000] + [int(r.argmax()) for r in logits[3:]]
+    big = rand(3, 151936, seed=9)
+    big[1, 151935] = big[1, 70000] = 9.0           # equals in different pieces of the row
+    big[2, 4096] = 8.0
+    assert ops.argmax(big).tolist() == [int(big[0].argmax()), 70000, 4096]
     temps = torch.tensor([0.0, 0.7, 1.0, 1.5, 0.3, 2.0], device="cuda")
     hits = 0
     trials = 40
