@@ -167,6 +167,9 @@ typedef __attribute__((__vector_size__(4 * sizeof(short)))) short shortx4;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t uintx4;
 
+// 2^x in one instruction (v_exp_f32; float32, about 1 ulp; -inf gives 0)
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 constexpr int DK32 = D / 32;            // full 32-wide steps of the q.k product
 constexpr bool DK_TAIL = (D % 32) != 0; // one more step of 16
 constexpr int DB16 = D / 16;            // 16-wide blocks of the output
@@ -182,6 +185,7 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_mfma_kernel(
   const int r = lane % 16;
   const int g = lane / 16;
   const int group = heads / kv_heads;
+  const float scale_log2 = scale * 1.4426950408889634f;      // scores in units of log 2: weights are exp2
 
   // ---- which columns and which keys
   int request, kh, head0 = 0, token0 = 0, columns;
@@ -308,7 +312,7 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_mfma_kernel(
         for (int i = 0; i < 4; ++i) {
           const int key = tile + 16 * ct + 4 * g + i;
           const bool seen = live[ct] && key >= max(col_first[mb], key_begin) && key <= min(col_last[mb], key_end);
-          const float v = seen ? s[mb][ct][i] * scale : -INFINITY;
+          const float v = seen ? s[mb][ct][i] * scale_log2 : -INFINITY;
           s[mb][ct][i] = v;
           best = fmaxf(best, v);
         }
@@ -316,13 +320,13 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_mfma_kernel(
       best = fmaxf(best, __shfl_xor(best, 32, DISTIE_WAVE));
       const float m_new = fmaxf(m_run[mb], best);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;     // no key seen yet: every weight is 0
-      alpha[mb] = expf(m_run[mb] - m_safe);                      // 0 while m_run is -inf
+      alpha[mb] = fast_exp2(m_run[mb] - m_safe);                 // 0 while m_run is -inf
       float sum = 0.f;
 #pragma unroll
       for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float p = expf(s[mb][ct][i] - m_safe);
+          const float p = fast_exp2(s[mb][ct][i] - m_safe);
           sum += p;
           p_reg[mb][4 * ct + i] = static_cast<bf16_t>(p);
         }
@@ -430,7 +434,7 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_reduce_kernel(
     const int mine = s0 + lane;
     float w = 0.f, wl = 0.f;
     if (mine <= s_last) {
-      w = expf(part_ml[2 * (base + mine)] - m);
+      w = fast_exp2(part_ml[2 * (base + mine)] - m);          // the maxima are in units of log 2
       wl = w * part_ml[2 * (base + mine) + 1];
     }
     l += wl;                                  // summed over the lanes at the end
@@ -551,7 +555,7 @@ constexpr int PF_V_CHUNKS = D * PF_BN / 8;
 constexpr int PF_K_PER_THREAD = (PF_K_CHUNKS + PF_THREADS - 1) / PF_THREADS;
 constexpr int PF_V_PER_THREAD = (PF_V_CHUNKS + PF_THREADS - 1) / PF_THREADS;
 
-__global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
+__global__ __launch_bounds__(PF_THREADS, 2) void attn_prefill_kernel(
     const bf16_t* __restrict__ qkv, int64_t q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ positions, const int32_t* __restrict__ cu_q,
     const int32_t* __restrict__ block_table, int table_width, bf16_t* __restrict__ out, int num_requests, int heads,
@@ -564,6 +568,7 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
   const int r = lane % 16;
   const int g = lane / 16;
   const int group = heads / kv_heads;
+  const float scale_log2 = scale * 1.4426950408889634f;      // scores in units of log 2: weights are exp2
 
   // ---- which tokens: blockIdx.x counts tiles of PF_BM tokens over the requests that are served here
   int tile = blockIdx.x;
@@ -727,7 +732,7 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = k0 + 16 * kb + 4 * g + i;
-          const float v = (key >= first && key <= last) ? s[mb][kb][i] * scale : -INFINITY;
+          const float v = (key >= first && key <= last) ? s[mb][kb][i] * scale_log2 : -INFINITY;
           s[mb][kb][i] = v;
           best = fmaxf(best, v);
         }
@@ -735,13 +740,13 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
       best = fmaxf(best, __shfl_xor(best, 32, DISTIE_WAVE));
       const float m_new = fmaxf(m_run[mb], best);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      alpha[mb] = expf(m_run[mb] - m_safe);
+      alpha[mb] = fast_exp2(m_run[mb] - m_safe);
       float sum = 0.f;
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float p = expf(s[mb][kb][i] - m_safe);
+          const float p = fast_exp2(s[mb][kb][i] - m_safe);
           sum += p;
           p_reg[mb][kb / 2][4 * (kb % 2) + i] = static_cast<bf16_t>(p);
         }

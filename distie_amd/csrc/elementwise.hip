@@ -94,8 +94,28 @@ extern "C" int distie_rmsnorm(float* residual, const void* delta, int delta_dtyp
 // (j, j + R/2) of every q and k head is turned by angle = float(position) * inv_freq[j] (R = 2 * pairs <= D
 // is the rotated width). The turned k and the v of the token go to the cache at the token's slot
 // (slot = page * P + offset): k into [pages, KH, P, D], v transposed into [pages, KH, D, P].
+// cos and sin of every (token, pair), once per step: all layers of a step turn by the same angles
+__global__ void rope_table_kernel(const int32_t* __restrict__ positions, const float* __restrict__ inv_freq,
+                                  float2* __restrict__ table, int pairs) {
+  const int64_t t = blockIdx.x;
+  const float pos = static_cast<float>(positions[t]);
+  for (int j = threadIdx.x; j < pairs; j += blockDim.x) {
+    float sn, cs;
+    sincosf(pos * inv_freq[j], &sn, &cs);
+    table[t * pairs + j] = float2{cs, sn};
+  }
+}
+
+extern "C" int distie_rope_table(const int32_t* positions, const float* inv_freq, void* table, int tokens, int pairs,
+                                 hipStream_t stream) {
+  if (tokens <= 0 || pairs <= 0) return 0;
+  rope_table_kernel<<<tokens, 64, 0, stream>>>(positions, inv_freq, static_cast<float2*>(table), pairs);
+  return launch_status();
+}
+
 template <typename I, typename T, typename C>
 __global__ void rope_kv_write_kernel(const I* in, int slices, int64_t slice_stride, T* out,
+                                     const float2* __restrict__ table,
                                      const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
                                      C* __restrict__ k_cache, C* __restrict__ v_cache,
                                      const float* __restrict__ inv_freq, int pairs, int heads, int kv_heads, int dim,
@@ -121,7 +141,13 @@ __global__ void rope_kv_write_kernel(const I* in, int slices, int64_t slice_stri
       // pair (j, j + pairs)
       const float x0 = value(lo), x1 = value(lo + pairs);
       float sn, cs;
-      sincosf(pos * inv_freq[j], &sn, &cs);
+      if (table != nullptr) {
+        const float2 e = table[t * pairs + j];
+        cs = e.x;
+        sn = e.y;
+      } else {
+        sincosf(pos * inv_freq[j], &sn, &cs);
+      }
       a = x0 * cs - x1 * sn;
       b = x1 * cs + x0 * sn;
       row[lo] = from_float<T>(a);
@@ -148,7 +174,8 @@ __global__ void rope_kv_write_kernel(const I* in, int slices, int64_t slice_stri
   }
 }
 
-extern "C" int distie_rope_kv_write(const void* in, int in_dtype, int slices, void* out, int dtype,
+// table: float2 [tokens, pairs] from distie_rope_table, or null (the angles are then computed here)
+extern "C" int distie_rope_kv_write(const void* in, int in_dtype, int slices, void* out, int dtype, const void* table,
                                     const int32_t* positions, const int32_t* slots, void* k_cache, void* v_cache,
                                     int cache_dtype, const float* inv_freq, int pairs, int tokens, int heads,
                                     int kv_heads, int dim, int block_size, int write, hipStream_t stream) {
@@ -163,7 +190,8 @@ extern "C" int distie_rope_kv_write(const void* in, int in_dtype, int slices, vo
   const int64_t stride = static_cast<int64_t>(tokens) * (heads + 2 * kv_heads) * dim;
   DISTIE_DISPATCH(in_dtype, I, DISTIE_DISPATCH(dtype, T, DISTIE_DISPATCH(cache_dtype, C,
       rope_kv_write_kernel<I, T, C><<<tokens, threads, 0, stream>>>(
-          static_cast<const I*>(in), slices, stride, static_cast<T*>(out), positions, slots,
+          static_cast<const I*>(in), slices, stride, static_cast<T*>(out), static_cast<const float2*>(table),
+          positions, slots,
           static_cast<C*>(k_cache), static_cast<C*>(v_cache), inv_freq, pairs, heads, kv_heads, dim, block_size,
           write))));
   return launch_status();
@@ -186,10 +214,42 @@ __global__ void silu_mul_kernel(const I* __restrict__ gate_up, int slices, int64
   }
 }
 
+// bfloat16 in and out, one slice, inter a multiple of 8: 16-byte loads and stores
+__global__ void silu_mul_bf16x8_kernel(const uint4* __restrict__ gate_up, uint4* __restrict__ out, int64_t rows,
+                                       int inter8) {
+  const int64_t total = rows * inter8;
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t r = i / inter8;
+    const int c = static_cast<int>(i % inter8);
+    const uint4 g4 = gate_up[r * 2 * inter8 + c];
+    const uint4 u4 = gate_up[r * 2 * inter8 + inter8 + c];
+    const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float g0 = __uint_as_float(gw[e] << 16), g1 = __uint_as_float(gw[e] & 0xffff0000u);
+      const float u0 = __uint_as_float(uw[e] << 16), u1 = __uint_as_float(uw[e] & 0xffff0000u);
+      const bf16_t lo = static_cast<bf16_t>(g0 / (1.f + expf(-g0)) * u0);
+      const bf16_t hi = static_cast<bf16_t>(g1 / (1.f + expf(-g1)) * u1);
+      ow[e] = static_cast<uint32_t>(__builtin_bit_cast(uint16_t, lo)) |
+              (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, hi)) << 16);
+    }
+    out[i] = uint4{ow[0], ow[1], ow[2], ow[3]};
+  }
+}
+
 extern "C" int distie_silu_mul(const void* gate_up, int in_dtype, int slices, void* out, int dtype, int rows,
                                int inter, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (inter <= 0 || slices < 1) return DISTIE_BAD_ARGUMENT;
+  if (in_dtype == DISTIE_BF16 && dtype == DISTIE_BF16 && slices == 1 && inter % 8 == 0) {
+    const int64_t pieces = static_cast<int64_t>(rows) * (inter / 8);
+    const int blocks8 = static_cast<int>(pieces / 256 + 1 < 16384 ? pieces / 256 + 1 : 16384);
+    silu_mul_bf16x8_kernel<<<blocks8, 256, 0, stream>>>(static_cast<const uint4*>(gate_up), static_cast<uint4*>(out),
+                                                        rows, inter / 8);
+    return launch_status();
+  }
   const int64_t total = static_cast<int64_t>(rows) * inter;
   const int threads = 256;
   const int blocks = static_cast<int>(total / threads + 1 < 16384 ? total / threads + 1 : 16384);

@@ -84,7 +84,8 @@ class HipOps(Ops):
         o = self._ops
         o.distie_embed.argtypes = [_P, _P, _I, _P, _I, _I, _I, _P]
         o.distie_rmsnorm.argtypes = [_P, _P, _I, _I, _P, _I, _P, _I, _I, _I, _F, _P]
-        o.distie_rope_kv_write.argtypes = [_P, _I, _I, _P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P]
+        o.distie_rope_kv_write.argtypes = [_P, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P]
+        o.distie_rope_table.argtypes = [_P, _P, _P, _I, _I, _P]
         o.distie_silu_mul.argtypes = [_P, _I, _I, _P, _I, _I, _I, _P]
         o.distie_sum_slices.argtypes = [_P, _I, _L, _P, _I, _P]
         o.distie_gather_rows.argtypes = [_P, _P, _P, _I, _L, _I, _P]
@@ -240,8 +241,19 @@ class HipOps(Ops):
             raise KernelError("rope_kv_write: qkv rows do not match the batch")
         pairs = 0 if inv_freq is None else inv_freq.shape[0]
         slots = meta.groups[group].slots
+        table = None
+        if pairs:
+            # cosines and sines of the step's positions: computed by the first layer that asks, used by all
+            key = ("rope", inv_freq.data_ptr(), pairs)
+            table = meta.scratch.get(key)
+            if table is None:
+                table = torch.empty((T, pairs, 2), dtype=torch.float32, device=self.device)
+                _check(self._ops.distie_rope_table(meta.positions.data_ptr(), inv_freq.data_ptr(), table.data_ptr(),
+                                                   T, pairs, self._stream()), "rope_table")
+                meta.scratch[key] = table
         _check(self._ops.distie_rope_kv_write(
-            source.data_ptr(), _code(source), slices, out.data_ptr(), _code(out), meta.positions.data_ptr(),
+            source.data_ptr(), _code(source), slices, out.data_ptr(), _code(out),
+            table.data_ptr() if table is not None else None, meta.positions.data_ptr(),
             slots.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _code(k_cache),
             inv_freq.data_ptr() if inv_freq is not None else None, pairs, T, num_heads, num_kv_heads, head_dim,
             meta.block_size, 1 if write else 0, self._stream()), "rope_kv_write")

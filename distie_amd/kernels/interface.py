@@ -49,6 +49,7 @@ class BatchMeta:
     host_cu_q: Optional[object] = None
     host_past: Optional[object] = None
     all_decode: bool = False           # every request brings exactly one token
+    scratch: dict = field(default_factory=dict)   # what an implementation computes once per step (cos/sin tables)
 
 
 class Ops(abc.ABC):

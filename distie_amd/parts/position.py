@@ -10,6 +10,9 @@ import torch
 from .base import PositionEncoding, register_part
 
 
+_SHARED = {}
+
+
 class RotaryPosition(PositionEncoding):
     def __init__(self, spec) -> None:
         super().__init__(spec)
@@ -22,7 +25,12 @@ class RotaryPosition(PositionEncoding):
         self.inv_freq = 1.0 / (self.theta ** exponent)
 
     def to_device(self, device) -> None:
-        self.inv_freq = self.inv_freq.to(device)
+        # layers with the same rotation share one table, so that what a step derives from it
+        # (cosines and sines of the step's positions) is derived once
+        key = (self.dim, self.theta, str(device))
+        if key not in _SHARED:
+            _SHARED[key] = self.inv_freq.to(device)
+        self.inv_freq = _SHARED[key]
 
     def rotary(self):
         return self.inv_freq
