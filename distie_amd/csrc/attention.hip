@@ -10,6 +10,7 @@
 // Formula: worker/src/inference/qwen2/model.py:154-161; softmax and all sums in float32.
 //
 //  * attn_generic: one wave per (token, head); any types; the true 32-bit path and the fallback.
+//  * attn_decode + attn_reduce, attn_prefill: bfloat16 on the matrix cores (described further down).
 
 #include "common.h"
 
@@ -145,22 +146,22 @@ extern "C" int distie_attention_generic(const void* qkv, int dtype, int64_t q_st
 }
 
 // ===================================================================================================
-//  * attn_mfma: bfloat16 on the matrix cores, for pages of a multiple of 16 tokens. One wave works on
-//    16 * MB "columns" and a run of keys, 32 keys at a time:
-//        S^T[key, col] = K[key, :] . q[col, :]        (v_mfma_f32_16x16x32_bf16, K rows straight from the page)
-//        online softmax over keys, per column, in float32
+//  Matrix-core kernels (bfloat16, pages of a multiple of 16 tokens). Both work on 16-wide blocks of
+//  "columns" against blocks of 16 keys with two products:
+//        S^T[key, col] = K[key, :] . q[col, :]        (v_mfma_f32_16x16x32_bf16, K rows as the A operand)
+//        online softmax over keys, per column, in float32 (weights as 2^x: scores are scaled by log2 e)
 //        O[col, d]  += P[col, key] . V^T[d, key]      (values are stored transposed inside a page, so the
 //                                                      summed index, the key, is contiguous for the B operand)
-//    A lane holds, of a 16 x 16 score tile, keys 4g..4g+3 of column r (r = lane % 16, g = lane / 16): exactly
-//    the shape of the A operand of the second product if its 32 summed keys are taken in the order
-//    (tile 0: 4g..4g+3, tile 1: 4g..4g+3); the values are read in the same order, so no data moves
-//    between lanes except the maxima and the rescaling factors.
-//    - prefill mode: columns = 16 * MB consecutive new tokens of one request, one head; all their keys;
-//      writes the normalised output.
-//    - decode mode: columns = the G query heads that share one kv head, of a request that brings one
-//      token; the keys are cut into runs of `split_len`, one wave each (this is where the parallelism
-//      comes from when few requests decode); writes unnormalised partial results that
-//      attn_reduce_kernel combines.
+//  A lane holds, of a 16 x 16 score tile, keys 4g..4g+3 of column r (r = lane % 16, g = lane / 16): exactly
+//  the shape of the A operand of the second product if its 32 summed keys are taken in the order
+//  (block 0: 4g..4g+3, block 1: 4g..4g+3); the values are read in the same order, so no data moves
+//  between lanes except the maxima and the rescaling factors.
+//
+//  * attn_decode: requests that bring one token. Columns = the G query heads that share one kv head. The
+//    keys are cut into runs of `split_len`, one wave each (this is where the parallelism comes from when
+//    few requests decode); a wave takes its run in chunks of DC_KEYS keys and issues every load of a chunk
+//    (pages, K rows, V^T rows) before it computes, so a chunk costs one trip to memory. It writes
+//    unnormalised partial results that attn_reduce combines.
 // ===================================================================================================
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short shortx4;
@@ -173,85 +174,43 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 constexpr int DK32 = D / 32;            // full 32-wide steps of the q.k product
 constexpr bool DK_TAIL = (D % 32) != 0; // one more step of 16
 constexpr int DB16 = D / 16;            // 16-wide blocks of the output
+constexpr int DC_BLOCKS = (D <= 128) ? 4 : 2;   // blocks of 16 keys whose loads are in flight together
+constexpr int DC_KEYS = 16 * DC_BLOCKS;
 
-template <int MB, bool DECODE>
-__global__ __launch_bounds__(DISTIE_WAVE) void attn_mfma_kernel(
+template <int MB>
+__global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ qkv, int64_t q_stride, const bf16_t* __restrict__ k_cache,
-    const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ positions, const int32_t* __restrict__ cu_q,
-    const int32_t* __restrict__ block_table, int table_width, bf16_t* __restrict__ out,
-    float* __restrict__ part_o, float* __restrict__ part_ml, int num_requests, int heads, int kv_heads,
-    int block_size, float scale, int window, int split_len, int max_splits) {
+    const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ kv_len, const int32_t* __restrict__ cu_q,
+    const int32_t* __restrict__ block_table, int table_width, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int heads, int kv_heads, int block_size, float scale, int window, int split_len,
+    int max_splits) {
   const int lane = threadIdx.x;
   const int r = lane % 16;
   const int g = lane / 16;
   const int group = heads / kv_heads;
-  const float scale_log2 = scale * 1.4426950408889634f;      // scores in units of log 2: weights are exp2
-
-  // ---- which columns and which keys
-  int request, kh, head0 = 0, token0 = 0, columns;
-  int key_begin, key_end;    // inclusive run of keys of this wave
-  if (DECODE) {
-    request = blockIdx.z;
-    kh = blockIdx.y;
-    token0 = cu_q[request];
-    if (cu_q[request + 1] - token0 != 1) return;      // a portion of a prompt: the tiled kernel's
-    columns = group;
-    const int q_pos = positions[token0];
-    const int first = window > 0 ? max(0, q_pos - window + 1) : 0;
-    key_begin = max(first, static_cast<int>(blockIdx.x) * split_len);
-    key_end = min(q_pos, static_cast<int>(blockIdx.x + 1) * split_len - 1);
-    if (key_begin > key_end) return;
-  } else {
-    // blockIdx.x counts tiles of 16 * MB tokens over all requests, in order
-    int tile = blockIdx.x;
-    request = 0;
-    int begin = 0, end = 0;
-    for (; request < num_requests; ++request) {
-      begin = cu_q[request];
-      end = cu_q[request + 1];
-      const int tiles = (end - begin + 16 * MB - 1) / (16 * MB);
-      if (tile < tiles) break;
-      tile -= tiles;
-    }
-    if (request >= num_requests) return;
-    head0 = blockIdx.y;
-    kh = head0 / group;
-    token0 = begin + tile * 16 * MB;
-    columns = min(16 * MB, end - token0);
-    const int pos_first = positions[token0];
-    const int pos_last = positions[token0 + columns - 1];
-    key_begin = window > 0 ? max(0, pos_first - window + 1) : 0;
-    key_end = pos_last;
-  }
+  const float scale_log2 = scale * 1.4426950408889634f;
+  const int request = blockIdx.z;
+  const int kh = blockIdx.y;
+  const int token = cu_q[request];
+  if (cu_q[request + 1] - token != 1) return;        // a portion of a prompt: the tiled kernel's
+  const int q_pos = kv_len[request] - 1;              // the new token is the last one cached
+  const int first = window > 0 ? max(0, q_pos - window + 1) : 0;
+  const int key_begin = max(first, static_cast<int>(blockIdx.x) * split_len);
+  const int key_end = min(q_pos, static_cast<int>(blockIdx.x + 1) * split_len - 1);
+  if (key_begin > key_end) return;
   const int32_t* table = block_table + static_cast<int64_t>(request) * table_width;
 
-  // ---- per column of this lane (column 16 mb + r): its query row, the keys it may see
-  const bf16_t* q_ptr[MB];
-  int col_last[MB], col_first[MB];
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb) {
-    const int col = min(16 * mb + r, columns - 1);     // columns past the end repeat the last one; dropped later
-    int token, head;
-    if (DECODE) {
-      token = token0;
-      head = kh * group + col;
-    } else {
-      token = token0 + col;
-      head = head0;
-    }
-    q_ptr[mb] = qkv + token * q_stride + static_cast<int64_t>(head) * D + 8 * g;
-    col_last[mb] = positions[token];
-    col_first[mb] = window > 0 ? max(0, col_last[mb] - window + 1) : 0;
-  }
+  // ---- the query of this lane's column (head kh * G + 16 mb + r; columns past the group repeat the last)
   bf16x8 q_reg[MB][DK32 > 0 ? DK32 : 1];
   shortx4 q_tail[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
+    const int col = min(16 * mb + r, group - 1);
+    const bf16_t* q = qkv + token * q_stride + static_cast<int64_t>(kh * group + col) * D;
 #pragma unroll
-    for (int dk = 0; dk < DK32; ++dk) q_reg[mb][dk] = *reinterpret_cast<const bf16x8*>(q_ptr[mb] + 32 * dk);
-    if (DK_TAIL) q_tail[mb] = *reinterpret_cast<const shortx4*>(q_ptr[mb] - 8 * g + (D - 16) + 4 * g);
+    for (int dk = 0; dk < DK32; ++dk) q_reg[mb][dk] = *reinterpret_cast<const bf16x8*>(q + 32 * dk + 8 * g);
+    if (DK_TAIL) q_tail[mb] = *reinterpret_cast<const shortx4*>(q + (D - 16) + 4 * g);
   }
-
   floatx4 o_acc[MB][DB16];
   float m_run[MB], l_run[MB];
 #pragma unroll
@@ -262,73 +221,91 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_mfma_kernel(
     for (int db = 0; db < DB16; ++db) o_acc[mb][db] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int tile = key_begin / 32 * 32; tile <= key_end; tile += 32) {
-    // ---- scores of 32 keys (two tiles of 16) for every column
-    floatx4 s[MB][2];
-    const bf16_t* v_base[2];
-    bool live[2];
+  for (int chunk = key_begin / DC_KEYS * DC_KEYS; chunk <= key_end; chunk += DC_KEYS) {
+    // ---- every load of the chunk first
+    bool live[DC_BLOCKS];
+    bf16x8 k_reg[DC_BLOCKS][DK32 > 0 ? DK32 : 1];
+    shortx4 k_tail[DC_BLOCKS];
+    uint2 v_reg[DC_BLOCKS][DB16];
 #pragma unroll
-    for (int ct = 0; ct < 2; ++ct) {
-      const int key0 = tile + 16 * ct;
-      live[ct] = key0 <= key_end && key0 + 15 >= key_begin;   // a tile outside the run may have no page
+    for (int b = 0; b < DC_BLOCKS; ++b) {
+      const int key0 = chunk + 16 * b;
+      live[b] = key0 <= key_end && key0 + 15 >= key_begin;      // a block outside the run may have no page
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) s[mb][ct] = floatx4{0.f, 0.f, 0.f, 0.f};
-      v_base[ct] = v_cache;
-      if (!live[ct]) continue;
+      for (int dk = 0; dk < DK32; ++dk) k_reg[b][dk] = bf16x8{};
+      k_tail[b] = shortx4{};
+#pragma unroll
+      for (int db = 0; db < DB16; ++db) v_reg[b][db] = uint2{0u, 0u};
+      if (!live[b]) continue;
       const int page = table[key0 / block_size];
       const int64_t page_base = (static_cast<int64_t>(page) * kv_heads + kh) * block_size * D;
       const int offset = key0 % block_size;
       const bf16_t* k_row = k_cache + page_base + static_cast<int64_t>(offset + r) * D;
-      v_base[ct] = v_cache + page_base + offset;
 #pragma unroll
-      for (int dk = 0; dk < DK32; ++dk) {
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(k_row + 32 * dk + 8 * g);
+      for (int dk = 0; dk < DK32; ++dk) k_reg[b][dk] = *reinterpret_cast<const bf16x8*>(k_row + 32 * dk + 8 * g);
+      if (DK_TAIL) k_tail[b] = *reinterpret_cast<const shortx4*>(k_row + (D - 16) + 4 * g);
+      // Slots after the run's last key were never written by this request: what a former owner of the page
+      // left there must not even be multiplied by a weight of zero (0 * NaN), so those values are cleared.
+      const int written = key_end - (key0 + 4 * g) + 1;          // of this lane's four keys
+      const uint32_t keep_lo = written >= 2 ? 0xffffffffu : (written == 1 ? 0x0000ffffu : 0u);
+      const uint32_t keep_hi = written >= 4 ? 0xffffffffu : (written == 3 ? 0x0000ffffu : 0u);
+      const bf16_t* v_col = v_cache + page_base + offset + 4 * g;
+#pragma unroll
+      for (int db = 0; db < DB16; ++db) {
+        const uint2 raw = *reinterpret_cast<const uint2*>(v_col + static_cast<int64_t>(16 * db + r) * block_size);
+        v_reg[b][db] = uint2{raw.x & keep_lo, raw.y & keep_hi};
+      }
+    }
+    // ---- scores
+    floatx4 s[MB][DC_BLOCKS];
+#pragma unroll
+    for (int b = 0; b < DC_BLOCKS; ++b) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) s[mb][b] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int dk = 0; dk < DK32; ++dk)
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          s[mb][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q_reg[mb][dk], s[mb][ct], 0, 0, 0);
-      }
+          s[mb][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_reg[b][dk], q_reg[mb][dk], s[mb][b], 0, 0, 0);
       if (DK_TAIL) {
         // The last 16 dims go through the 16-deep instruction into an accumulator of their own, added on the
         // vector ALU: chained straight onto the 32-deep instruction's accumulator, the first two of its
         // four registers were read before they were written (results depended on timing).
-        const shortx4 a = *reinterpret_cast<const shortx4*>(k_row + (D - 16) + 4 * g);
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
-          const floatx4 tail = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, q_tail[mb], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+          const floatx4 tail = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(k_tail[b], q_tail[mb], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) s[mb][ct][i] += tail[i];
+          for (int i = 0; i < 4; ++i) s[mb][b][i] += tail[i];
         }
       }
     }
-    // ---- softmax step, per column
-    bf16x8 p_reg[MB];
+    // ---- softmax step per column
+    bf16x8 p_reg[MB][DC_BLOCKS / 2];
     float alpha[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       float best = -INFINITY;
 #pragma unroll
-      for (int ct = 0; ct < 2; ++ct)
+      for (int b = 0; b < DC_BLOCKS; ++b)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int key = tile + 16 * ct + 4 * g + i;
-          const bool seen = live[ct] && key >= max(col_first[mb], key_begin) && key <= min(col_last[mb], key_end);
-          const float v = seen ? s[mb][ct][i] * scale_log2 : -INFINITY;
-          s[mb][ct][i] = v;
+          const int key = chunk + 16 * b + 4 * g + i;
+          const float v = (key >= key_begin && key <= key_end) ? s[mb][b][i] * scale_log2 : -INFINITY;
+          s[mb][b][i] = v;
           best = fmaxf(best, v);
         }
       best = fmaxf(best, __shfl_xor(best, 16, DISTIE_WAVE));
       best = fmaxf(best, __shfl_xor(best, 32, DISTIE_WAVE));
-      const float m_new = fmaxf(m_run[mb], best);
-      const float m_safe = m_new == -INFINITY ? 0.f : m_new;     // no key seen yet: every weight is 0
-      alpha[mb] = fast_exp2(m_run[mb] - m_safe);                 // 0 while m_run is -inf
+      const float m_new = fmaxf(m_run[mb], best);      // finite: every chunk of the run holds a key
+      alpha[mb] = fast_exp2(m_run[mb] - m_new);        // 0 while m_run is -inf
       float sum = 0.f;
 #pragma unroll
-      for (int ct = 0; ct < 2; ++ct)
+      for (int b = 0; b < DC_BLOCKS; ++b)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float p = fast_exp2(s[mb][ct][i] - m_safe);
+          const float p = fast_exp2(s[mb][b][i] - m_new);
           sum += p;
-          p_reg[mb][4 * ct + i] = static_cast<bf16_t>(p);
+          p_reg[mb][b / 2][4 * (b % 2) + i] = static_cast<bf16_t>(p);
         }
       l_run[mb] = l_run[mb] * alpha[mb] + sum;      // the lanes of a column each keep a part of the sum
       m_run[mb] = m_new;
@@ -344,202 +321,161 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_mfma_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) o_acc[mb][db][i] *= a4[i];
     }
-    // ---- O += P . V
-    // Slots after the run's last key were never written by this request: what a former owner of the page
-    // left there must not even be multiplied by a weight of zero (0 * NaN), so those values are cleared.
-    uint32_t keep[2][2];
+    // ---- O += P . V, 32 keys (two blocks) a step; the vector is put together as whole 32-bit words
 #pragma unroll
-    for (int ct = 0; ct < 2; ++ct) {
-      const int written = key_end - (tile + 16 * ct + 4 * g) + 1;     // of this lane's four keys
-      keep[ct][0] = written >= 2 ? 0xffffffffu : (written == 1 ? 0x0000ffffu : 0u);
-      keep[ct][1] = written >= 4 ? 0xffffffffu : (written == 3 ? 0x0000ffffu : 0u);
-    }
+    for (int ks = 0; ks < DC_BLOCKS / 2; ++ks)
 #pragma unroll
-    for (int db = 0; db < DB16; ++db) {
-      // four keys (8 bytes) of each live tile; the vector is put together as whole 32-bit words
-      uintx4 words = {0u, 0u, 0u, 0u};
+      for (int db = 0; db < DB16; ++db) {
+        const uintx4 words = {v_reg[2 * ks][db].x, v_reg[2 * ks][db].y, v_reg[2 * ks + 1][db].x, v_reg[2 * ks + 1][db].y};
+        const bf16x8 v = __builtin_bit_cast(bf16x8, words);
 #pragma unroll
-      for (int ct = 0; ct < 2; ++ct) {
-        if (!live[ct]) continue;
-        const uint2 raw = *reinterpret_cast<const uint2*>(v_base[ct] + static_cast<int64_t>(16 * db + r) * block_size + 4 * g);
-        words[2 * ct] = raw.x & keep[ct][0];
-        words[2 * ct + 1] = raw.y & keep[ct][1];
+        for (int mb = 0; mb < MB; ++mb)
+          o_acc[mb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_reg[mb][ks], v, o_acc[mb][db], 0, 0, 0);
       }
-      const bf16x8 v = __builtin_bit_cast(bf16x8, words);
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-        o_acc[mb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_reg[mb], v, o_acc[mb][db], 0, 0, 0);
-    }
   }
 
-  // ---- finish: sums over the lanes of a column, then write
+  // ---- sums over the lanes of a column, then the partial result of this run
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     l_run[mb] += __shfl_xor(l_run[mb], 16, DISTIE_WAVE);
     l_run[mb] += __shfl_xor(l_run[mb], 32, DISTIE_WAVE);
   }
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) {
+  for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int col = 16 * mb + 4 * g + i;
       const float l_col = __shfl(l_run[mb], 4 * g + i, DISTIE_WAVE);
       const float m_col = __shfl(m_run[mb], 4 * g + i, DISTIE_WAVE);
-      if (col >= columns) continue;
-      if (DECODE) {
-        const int64_t slot = (static_cast<int64_t>(request) * heads + kh * group + col) * max_splits + blockIdx.x;
-        float* po = part_o + slot * D;
+      if (col >= group) continue;
+      const int64_t slot = (static_cast<int64_t>(request) * heads + kh * group + col) * max_splits + blockIdx.x;
+      float* po = part_o + slot * D;
 #pragma unroll
-        for (int db = 0; db < DB16; ++db) po[16 * db + r] = o_acc[mb][db][i];
-        if (r == 0) {
-          part_ml[2 * slot] = m_col;
-          part_ml[2 * slot + 1] = l_col;
-        }
-      } else {
-        bf16_t* o = out + (static_cast<int64_t>(token0 + col) * heads + head0) * D;
-        const float inv = 1.f / l_col;
-#pragma unroll
-        for (int db = 0; db < DB16; ++db) o[16 * db + r] = static_cast<bf16_t>(o_acc[mb][db][i] * inv);
+      for (int db = 0; db < DB16; ++db) po[16 * db + r] = o_acc[mb][db][i];
+      if (r == 0) {
+        part_ml[2 * slot] = m_col;
+        part_ml[2 * slot + 1] = l_col;
       }
     }
-  }
 }
 
-// Combines the partial results of the runs of keys of one (request, head): grid (heads, requests), one wave.
-// The lanes first take one run each to find the maximum and the weights of the runs, then each lane owns
-// output dims and adds the runs in order, four loads in flight at a time.
-__global__ __launch_bounds__(DISTIE_WAVE) void attn_reduce_kernel(
-    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int32_t* __restrict__ positions,
+// Combines the partial results of the runs of keys of one (request, head): grid (heads, requests), four waves.
+// All threads first find the maximum and the weight of every run; then each wave adds a quarter of the runs
+// (in order, four loads in flight at a time) for the output dims its lanes own, and the four sums are added
+// in order through LDS.
+constexpr int RD_WAVES = 4;
+constexpr int RD_THREADS = RD_WAVES * DISTIE_WAVE;
+constexpr int RD_MAX_RUNS = 1024;
+
+__global__ __launch_bounds__(RD_THREADS) void attn_reduce_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int32_t* __restrict__ kv_len,
     const int32_t* __restrict__ cu_q, bf16_t* __restrict__ out, int heads, int window, int split_len, int max_splits) {
-  __shared__ float weight_s[DISTIE_WAVE];
-  const int lane = threadIdx.x;
+  __shared__ float weight_s[RD_MAX_RUNS];
+  __shared__ float sum_s[RD_WAVES][D];
+  __shared__ float scratch[32];
+  const int tid = threadIdx.x;
+  const int wave = tid / DISTIE_WAVE;
+  const int lane = tid % DISTIE_WAVE;
   const int request = blockIdx.y;
   const int head = blockIdx.x;
   const int token = cu_q[request];
   if (cu_q[request + 1] - token != 1) return;
-  const int q_pos = positions[token];
+  const int q_pos = kv_len[request] - 1;
   const int first = window > 0 ? max(0, q_pos - window + 1) : 0;
   const int s_first = first / split_len;
-  const int s_last = q_pos / split_len;
-  const int64_t base = (static_cast<int64_t>(request) * heads + head) * max_splits;
-  float acc[DIMS_PER_LANE];
-#pragma unroll
-  for (int i = 0; i < DIMS_PER_LANE; ++i) acc[i] = 0.f;
-  // the maximum over all runs
+  const int runs = q_pos / split_len - s_first + 1;
+  const int64_t base = (static_cast<int64_t>(request) * heads + head) * max_splits + s_first;
+  // the maximum over all runs (in units of log 2), then every run's weight
   float m = -INFINITY;
-  for (int s = s_first + lane; s <= s_last; s += DISTIE_WAVE) m = fmaxf(m, part_ml[2 * (base + s)]);
+  for (int j = tid; j < runs; j += RD_THREADS) m = fmaxf(m, part_ml[2 * (base + j)]);
   m = wave_max(m);
+  if (lane == 0) scratch[wave] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3]));
   float l = 0.f;
-  for (int s0 = s_first; s0 <= s_last; s0 += DISTIE_WAVE) {
-    const int mine = s0 + lane;
-    float w = 0.f, wl = 0.f;
-    if (mine <= s_last) {
-      w = fast_exp2(part_ml[2 * (base + mine)] - m);          // the maxima are in units of log 2
-      wl = w * part_ml[2 * (base + mine) + 1];
-    }
-    l += wl;                                  // summed over the lanes at the end
-    __syncthreads();
-    weight_s[lane] = w;
-    __syncthreads();
-    const int n = min(DISTIE_WAVE, s_last - s0 + 1);
-    const float* po = part_o + (base + s0) * D;
-#pragma unroll
-    for (int i = 0; i < DIMS_PER_LANE; ++i) {
-      const int d = lane + i * DISTIE_WAVE;
-      if (d >= D) continue;
-      float a = acc[i];
-      int j = 0;
-      for (; j + 4 <= n; j += 4) {
-        const float v0 = po[static_cast<int64_t>(j) * D + d], v1 = po[static_cast<int64_t>(j + 1) * D + d];
-        const float v2 = po[static_cast<int64_t>(j + 2) * D + d], v3 = po[static_cast<int64_t>(j + 3) * D + d];
-        a = fmaf(weight_s[j], v0, a);
-        a = fmaf(weight_s[j + 1], v1, a);
-        a = fmaf(weight_s[j + 2], v2, a);
-        a = fmaf(weight_s[j + 3], v3, a);
-      }
-      for (; j < n; ++j) a = fmaf(weight_s[j], po[static_cast<int64_t>(j) * D + d], a);
-      acc[i] = a;
-    }
+  for (int j = tid; j < runs; j += RD_THREADS) {
+    const float w = fast_exp2(part_ml[2 * (base + j)] - m);
+    weight_s[j] = w;
+    l += w * part_ml[2 * (base + j) + 1];
   }
-  l = wave_sum(l);
+  l = block_sum(l, scratch + 16);           // has the barrier that publishes the weights
+  const float* po = part_o + base * D;
+#pragma unroll
+  for (int i = 0; i < DIMS_PER_LANE; ++i) {
+    const int d = lane + i * DISTIE_WAVE;
+    if (d >= D) continue;
+    float a = 0.f;
+    int j = wave;
+    for (; j + 3 * RD_WAVES < runs; j += 4 * RD_WAVES) {
+      const float v0 = po[static_cast<int64_t>(j) * D + d], v1 = po[static_cast<int64_t>(j + RD_WAVES) * D + d];
+      const float v2 = po[static_cast<int64_t>(j + 2 * RD_WAVES) * D + d], v3 = po[static_cast<int64_t>(j + 3 * RD_WAVES) * D + d];
+      a = fmaf(weight_s[j], v0, a);
+      a = fmaf(weight_s[j + RD_WAVES], v1, a);
+      a = fmaf(weight_s[j + 2 * RD_WAVES], v2, a);
+      a = fmaf(weight_s[j + 3 * RD_WAVES], v3, a);
+    }
+    for (; j < runs; j += RD_WAVES) a = fmaf(weight_s[j], po[static_cast<int64_t>(j) * D + d], a);
+    sum_s[wave][d] = a;
+  }
+  __syncthreads();
+  if (wave != 0) return;
   bf16_t* o = out + (static_cast<int64_t>(token) * heads + head) * D;
   const float inv = 1.f / l;
 #pragma unroll
   for (int i = 0; i < DIMS_PER_LANE; ++i) {
     const int d = lane + i * DISTIE_WAVE;
-    if (d < D) o[d] = static_cast<bf16_t>(acc[i] * inv);
+    if (d < D) o[d] = static_cast<bf16_t>((((sum_s[0][d] + sum_s[1][d]) + sum_s[2][d]) + sum_s[3][d]) * inv);
   }
 }
 
-constexpr int MFMA_MAX_MB = (D <= 128) ? 4 : 2;     // registers: the output tile is 16 * MB x D floats a wave
+constexpr int DECODE_MAX_MB = (D <= 128) ? 4 : 2;   // registers: the output tile is 16 * MB x D floats a wave
 
-extern "C" int distie_attention_mfma_columns() { return 16 * MFMA_MAX_MB; }
+// most query heads per kv head the decode kernel takes
+extern "C" int distie_attention_decode_columns() { return 16 * DECODE_MAX_MB; }
 
-// The register-only kernel in prefill mode (kept for comparison). bfloat16 only; block_size a multiple of 16.
-extern "C" int distie_attention_prefill_simple_bf16(const void* qkv, int64_t q_stride, const void* k_cache, const void* v_cache,
-                                             const int32_t* positions, const int32_t* cu_q, const int32_t* block_table,
-                                             int table_width, void* out, int tokens, int num_requests, int heads,
-                                             int kv_heads, int block_size, float scale, int window,
-                                             hipStream_t stream) {
-  if (tokens <= 0) return 0;
-  if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size % 16 != 0 || table_width < 1 || window < 0 ||
-      num_requests < 1 || heads > 65535)
-    return DISTIE_BAD_ARGUMENT;
-  constexpr int MB = MFMA_MAX_MB;
-  const int tiles = (tokens + 16 * MB - 1) / (16 * MB) + num_requests;     // an upper bound; spare blocks leave at once
-  dim3 grid(tiles, heads);
-  attn_mfma_kernel<MB, false><<<grid, DISTIE_WAVE, 0, stream>>>(
-      static_cast<const bf16_t*>(qkv), q_stride, static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),
-      positions, cu_q, block_table, table_width, static_cast<bf16_t*>(out), nullptr, nullptr, num_requests, heads,
-      kv_heads, block_size, scale, window, 0, 0);
-  return launch_status();
-}
-
-// The requests of a step that bring one token (others are skipped). part_o: float32 [requests, heads, max_splits, D],
-// part_ml: float32 [requests, heads, max_splits, 2]; max_splits * split_len must cover every position.
+// The requests of a step that bring one token (others are skipped). kv_len: tokens cached after the step, per
+// request. part_o: float32 [requests, heads, max_splits, D], part_ml: float32 [requests, heads, max_splits, 2];
+// max_splits * split_len must cover every position.
 extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, const void* k_cache, const void* v_cache,
-                                            const int32_t* positions, const int32_t* cu_q, const int32_t* block_table,
+                                            const int32_t* kv_len, const int32_t* cu_q, const int32_t* block_table,
                                             int table_width, void* out, float* part_o, float* part_ml,
                                             int num_requests, int heads, int kv_heads, int block_size, float scale,
                                             int window, int split_len, int max_splits, hipStream_t stream) {
   if (num_requests <= 0) return 0;
   const int group = kv_heads > 0 ? heads / kv_heads : 0;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size % 16 != 0 || table_width < 1 || window < 0 ||
-      split_len < 32 || split_len % 32 != 0 || max_splits < 1 || group > 16 * MFMA_MAX_MB || kv_heads > 65535 ||
-      num_requests > 65535)
+      split_len < DC_KEYS || split_len % DC_KEYS != 0 || max_splits < 1 || max_splits > RD_MAX_RUNS ||
+      group > 16 * DECODE_MAX_MB || kv_heads > 65535 || num_requests > 65535 || heads > 65535)
     return DISTIE_BAD_ARGUMENT;
   dim3 grid(max_splits, kv_heads, num_requests);
   const bf16_t* q = static_cast<const bf16_t*>(qkv);
   const bf16_t* kc = static_cast<const bf16_t*>(k_cache);
   const bf16_t* vc = static_cast<const bf16_t*>(v_cache);
-#define DECODE_LAUNCH(MB)                                                                                              \
-  attn_mfma_kernel<MB, true><<<grid, DISTIE_WAVE, 0, stream>>>(q, q_stride, kc, vc, positions, cu_q, block_table,      \
-                                                               table_width, nullptr, part_o, part_ml, num_requests,   \
-                                                               heads, kv_heads, block_size, scale, window, split_len, \
-                                                               max_splits)
+#define DECODE_LAUNCH(MB)                                                                                             \
+  attn_decode_kernel<MB><<<grid, DISTIE_WAVE, 0, stream>>>(q, q_stride, kc, vc, kv_len, cu_q, block_table, table_width, \
+                                                           part_o, part_ml, heads, kv_heads, block_size, scale, window, \
+                                                           split_len, max_splits)
   if (group <= 16) {
     DECODE_LAUNCH(1);
   } else if (group <= 32) {
     DECODE_LAUNCH(2);
   } else {
-    if (MFMA_MAX_MB < 4) return DISTIE_BAD_ARGUMENT;
-    DECODE_LAUNCH(MFMA_MAX_MB);
+    DECODE_LAUNCH(DECODE_MAX_MB);
   }
 #undef DECODE_LAUNCH
   int status = launch_status();
   if (status != 0) return status;
-  attn_reduce_kernel<<<dim3(heads, num_requests), DISTIE_WAVE, 0, stream>>>(
-      part_o, part_ml, positions, cu_q, static_cast<bf16_t*>(out), heads, window, split_len, max_splits);
+  attn_reduce_kernel<<<dim3(heads, num_requests), RD_THREADS, 0, stream>>>(
+      part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, split_len, max_splits);
   return launch_status();
 }
-
 
 // ===================================================================================================
 //  * attn_prefill: the tiled kernel for portions of prompts. A workgroup of four waves owns PF_BM
 //    consecutive new tokens of one request and one head; it walks over the keys 64 at a time. The K tile
 //    [64, D] and the V^T tile [D, 64] are put into LDS once per workgroup (global loads of the next tile
 //    are in flight while the current one is used) and every wave multiplies its own 16 * PF_MB query
-//    columns against them with the same two products and the same register layout as attn_mfma.
+//    columns against them with the same two products and the same register layout as attn_decode.
 //    Requests that bring fewer than `min_q_len` tokens are left to the decode kernel.
 // ===================================================================================================
 constexpr int PF_BN = 64;                               // keys per tile

@@ -114,8 +114,6 @@ class HipOps(Ops):
                                                      _I, _I, _I, _I, _F, _I, _P]
             lib.distie_attention_prefill_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I,
                                                           _F, _I, _I, _P]
-            lib.distie_attention_prefill_simple_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I,
-                                                                 _I, _F, _I, _P]
             lib.distie_attention_decode_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I,
                                                          _I, _F, _I, _I, _I, _P]
             if lib.distie_attention_head_dim() != head_dim:
@@ -276,19 +274,19 @@ class HipOps(Ops):
             singles = meta.num_requests if meta.all_decode else 0
             if not meta.all_decode and meta.host_cu_q is not None:
                 singles = int((meta.host_cu_q[1:] - meta.host_cu_q[:-1] == 1).sum())
-            split_decode = singles > 0 and group <= lib.distie_attention_mfma_columns()
+            split_decode = singles > 0 and group <= lib.distie_attention_decode_columns()
             if split_decode:
                 # requests that bring one token: keys are cut into runs, one wave each, so that the chip is
                 # filled even when few requests decode
                 runs = max(1, min(64, 4096 // (singles * num_kv_heads)))
-                split_len = max(64, -(-meta.max_kv // runs + 31) // 32 * 32)
+                split_len = max(64, -(-(-(-meta.max_kv // runs)) // 64) * 64)
                 max_splits = -(-meta.max_kv // split_len)
                 part_o = torch.empty((meta.num_requests, num_heads, max_splits, head_dim), dtype=torch.float32,
                                      device=self.device)
                 part_ml = torch.empty((meta.num_requests, num_heads, max_splits, 2), dtype=torch.float32,
                                       device=self.device)
                 _check(lib.distie_attention_decode_bf16(
-                    qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), meta.positions.data_ptr(),
+                    qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), meta.kv_len.data_ptr(),
                     meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], out.data_ptr(), part_o.data_ptr(),
                     part_ml.data_ptr(), meta.num_requests, num_heads, num_kv_heads, meta.block_size, float(scale),
                     int(window or 0), split_len, max_splits, self._stream()), "attention_decode_bf16")
