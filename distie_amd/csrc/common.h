@@ -53,22 +53,22 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 }
 
 // Sum of `slices` values that lie `stride` elements apart, added in order. The loads of four slices are
-// issued together, so the sum costs a few memory round trips instead of one per slice.
+// issued together (the last group re-reads the last slice where it has fewer than four and does not add
+// it), so the sum costs a few memory round trips instead of one per slice.
 template <typename T>
 __device__ __forceinline__ float sum_strided(const T* p, int slices, int64_t stride) {
-  float sum = to_float(p[0]);
-  int s = 1;
-  for (; s + 4 <= slices; s += 4) {
+  float sum = 0.f;
+  for (int s = 0; s < slices; s += 4) {
+    const int last = slices - 1;
     const float a = to_float(p[s * stride]);
-    const float b = to_float(p[(s + 1) * stride]);
-    const float c = to_float(p[(s + 2) * stride]);
-    const float d = to_float(p[(s + 3) * stride]);
+    const float b = to_float(p[min(s + 1, last) * stride]);
+    const float c = to_float(p[min(s + 2, last) * stride]);
+    const float d = to_float(p[min(s + 3, last) * stride]);
     sum += a;
-    sum += b;
-    sum += c;
-    sum += d;
+    if (s + 1 <= last) sum += b;
+    if (s + 2 <= last) sum += c;
+    if (s + 3 <= last) sum += d;
   }
-  for (; s < slices; ++s) sum += to_float(p[s * stride]);
   return sum;
 }
 

@@ -43,23 +43,43 @@ __global__ void rmsnorm_kernel(float* __restrict__ residual, const D* __restrict
   __shared__ float scratch[16];
   const int64_t row = blockIdx.x;
   float* x = residual + row * width;
-  float ss = 0.f;
-  if (delta != nullptr) {
-    const D* d = delta + row * width;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) {
-      const float v = x[i] + sum_strided(d + i, slices, slice_stride);
-      x[i] = v;
-      ss += v * v;
-    }
-  } else {
-    for (int i = threadIdx.x; i < width; i += blockDim.x) {
-      const float v = x[i];
-      ss += v * v;
-    }
-  }
-  const float total = block_sum(ss, scratch);
-  const float scale = rsqrtf(total / static_cast<float>(width) + eps);
   O* y = out + row * width;
+  const D* d = delta != nullptr ? delta + row * width : nullptr;
+  constexpr int KEEP = 4;                       // elements a thread keeps in registers between the passes
+  if (width <= KEEP * static_cast<int>(blockDim.x)) {
+    float v[KEEP];
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < KEEP; ++e) {
+      const int i = threadIdx.x + e * blockDim.x;
+      v[e] = 0.f;
+      if (i < width) {
+        v[e] = x[i];
+        if (d != nullptr) {
+          v[e] += sum_strided(d + i, slices, slice_stride);
+          x[i] = v[e];
+        }
+        ss += v[e] * v[e];
+      }
+    }
+    const float scale = rsqrtf(block_sum(ss, scratch) / static_cast<float>(width) + eps);
+#pragma unroll
+    for (int e = 0; e < KEEP; ++e) {
+      const int i = threadIdx.x + e * blockDim.x;
+      if (i < width) y[i] = from_float<O>(v[e] * scale * to_float(weight[i]));
+    }
+    return;
+  }
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = x[i];
+    if (d != nullptr) {
+      v += sum_strided(d + i, slices, slice_stride);
+      x[i] = v;
+    }
+    ss += v * v;
+  }
+  const float scale = rsqrtf(block_sum(ss, scratch) / static_cast<float>(width) + eps);
   // each thread re-reads what it wrote itself
   for (int i = threadIdx.x; i < width; i += blockDim.x) y[i] = from_float<O>(x[i] * scale * to_float(weight[i]));
 }
@@ -129,52 +149,52 @@ __global__ void rope_kv_write_kernel(const I* in, int slices, int64_t slice_stri
   const int64_t page = slot / block_size;
   const int offset = static_cast<int>(slot % block_size);
   auto value = [&](int64_t i) { return sum_strided(src + i, slices, slice_stride); };
-  // q and k heads: every thread owns whole pairs, so `out` may alias `in`
+  // q and k heads: every thread owns whole pairs, so `out` may alias `in`. A thread that turns a pair of a k
+  // head, or copies a value of a v head, also stores it into the cache.
   const int rotated_heads = heads + kv_heads;
   const int half = dim / 2;
-  for (int i = threadIdx.x; i < rotated_heads * half; i += blockDim.x) {
-    const int head = i / half;
-    const int j = i % half;
+  const int rot = 2 * pairs;
+  for (int i = threadIdx.x; i < rotated_heads * pairs; i += blockDim.x) {
+    const int head = i / pairs;
+    const int j = i % pairs;
     const int64_t lo = static_cast<int64_t>(head) * dim + j;
-    float a, b;
-    if (j < pairs) {
-      // pair (j, j + pairs)
-      const float x0 = value(lo), x1 = value(lo + pairs);
-      float sn, cs;
-      if (table != nullptr) {
-        const float2 e = table[t * pairs + j];
-        cs = e.x;
-        sn = e.y;
-      } else {
-        sincosf(pos * inv_freq[j], &sn, &cs);
-      }
-      a = x0 * cs - x1 * sn;
-      b = x1 * cs + x0 * sn;
-      row[lo] = from_float<T>(a);
-      row[lo + pairs] = from_float<T>(b);
+    const float x0 = value(lo), x1 = value(lo + pairs);
+    float sn, cs;
+    if (table != nullptr) {
+      const float2 e = table[t * pairs + j];
+      cs = e.x;
+      sn = e.y;
+    } else {
+      sincosf(pos * inv_freq[j], &sn, &cs);
+    }
+    const T a = from_float<T>(x0 * cs - x1 * sn);
+    const T b = from_float<T>(x1 * cs + x0 * sn);
+    row[lo] = a;
+    row[lo + pairs] = b;
+    if (write && head >= heads) {
+      const int64_t at = ((page * kv_heads + (head - heads)) * block_size + offset) * dim;
+      k_cache[at + j] = from_float<C>(to_float(a));
+      k_cache[at + j + pairs] = from_float<C>(to_float(b));
     }
   }
+  (void)half;
   // columns of q and k beyond the rotated width, and v: copied
-  const int rot = 2 * pairs;
   for (int64_t i = threadIdx.x; i < width; i += blockDim.x) {
     const int head = static_cast<int>(i / dim);
     const int d = static_cast<int>(i % dim);
     if (head < rotated_heads && d < rot) continue;
-    row[i] = from_float<T>(value(i));
-  }
-  if (!write) return;
-  __syncthreads();
-  for (int i = threadIdx.x; i < kv_heads * dim; i += blockDim.x) {
-    const int head = i / dim;
-    const int d = i % dim;
-    const int64_t base = (page * kv_heads + head) * block_size * dim;
-    k_cache[base + static_cast<int64_t>(offset) * dim + d] = from_float<C>(to_float(row[(heads + head) * dim + d]));
-    v_cache[base + static_cast<int64_t>(d) * block_size + offset] =
-        from_float<C>(to_float(row[(heads + kv_heads + head) * dim + d]));
+    const T v = from_float<T>(value(i));
+    row[i] = v;
+    if (!write || head < heads) continue;
+    if (head < rotated_heads) {
+      k_cache[((page * kv_heads + (head - heads)) * block_size + offset) * dim + d] = from_float<C>(to_float(v));
+    } else {
+      v_cache[(page * kv_heads + (head - rotated_heads)) * block_size * dim + static_cast<int64_t>(d) * block_size + offset] =
+          from_float<C>(to_float(v));
+    }
   }
 }
 
-// table: float2 [tokens, pairs] from distie_rope_table, or null (the angles are then computed here)
 extern "C" int distie_rope_kv_write(const void* in, int in_dtype, int slices, void* out, int dtype, const void* table,
                                     const int32_t* positions, const int32_t* slots, void* k_cache, void* v_cache,
                                     int cache_dtype, const float* inv_freq, int pairs, int tokens, int heads,

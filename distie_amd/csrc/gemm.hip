@@ -125,7 +125,31 @@ __global__ __launch_bounds__(64) void gemm_skinny_kernel(const bf16_t* __restric
 
   const int steps = (k_end - k_begin) / SK_KSTEP;
   int step = steps > 0 ? static_cast<int>(blockIdx.x % steps) : 0;
-  for (int it = 0; it < steps; ++it) {
+  // Three k-steps at a time with every load issued before the first product: a wave that owns only a few
+  // steps (small layers, many slices) then pays one trip to memory instead of one per step.
+  constexpr int UN = MB == 1 ? 3 : 1;
+  int it = 0;
+  for (; it + UN <= steps; it += UN) {
+    bf16x8 a[UN][4], xb[UN][MB][4];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int k = k_begin + step * SK_KSTEP;
+      step = step + 1 == steps ? 0 : step + 1;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) a[u][j] = *reinterpret_cast<const bf16x8*>(wp + k + 32 * j);
+#pragma unroll
+      for (int b = 0; b < MB; ++b)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xb[u][b][j] = *reinterpret_cast<const bf16x8*>(xp[b] + k + 32 * j);
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u)
+#pragma unroll
+      for (int b = 0; b < MB; ++b)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][j], xb[u][b][j], acc[b], 0, 0, 0);
+  }
+  for (; it < steps; ++it) {
     const int k = k_begin + step * SK_KSTEP;
     step = step + 1 == steps ? 0 : step + 1;
     bf16x8 a[4];

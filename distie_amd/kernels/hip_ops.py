@@ -66,7 +66,7 @@ class PartialSums:
 
 
 class HipOps(Ops):
-    SKINNY_MAX_ROWS = 64
+    SKINNY_MAX_ROWS = 16       # above this the library's tiles are faster than streaming with x from memory
 
     def __init__(self, device="cuda:0") -> None:
         self.device = torch.device(device)
@@ -207,8 +207,11 @@ class HipOps(Ops):
                 lib_bias = getattr(bias, "_distie_bf16", None)
                 if lib_bias is None:
                     lib_bias = bias._distie_bf16 = bias.to(torch.bfloat16)
-            y = torch.nn.functional.linear(x, weight, lib_bias)
-            return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
+            if out_dtype == torch.float32:
+                # the library writes its float32 sums unrounded (the logits)
+                y = torch.mm(x, weight.t(), out_dtype=torch.float32)
+                return y if bias is None else y + bias
+            return torch.nn.functional.linear(x, weight, lib_bias)
         out = torch.empty((M, N), dtype=out_dtype, device=self.device)
         _check(self._ops.distie_gemm_generic(
             x.data_ptr(), _code(x), weight.data_ptr(), _code(weight), bias.data_ptr() if bias is not None else None,
