@@ -481,9 +481,10 @@ extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, c
 constexpr int PF_BN = 64;                               // keys per tile
 constexpr int PF_WAVES = 4;
 constexpr int PF_THREADS = PF_WAVES * DISTIE_WAVE;
-constexpr int PF_MB = (D <= 128) ? 2 : 1;               // blocks of 16 query columns per wave
+constexpr int PF_MB = 1;                                // blocks of 16 query columns per wave
 constexpr int PF_WAVE_COLS = 16 * PF_MB;
 constexpr int PF_BM = PF_WAVES * PF_WAVE_COLS;          // query tokens per workgroup
+constexpr int PF_DEPTH = 2;                             // key tiles whose loads are in flight
 constexpr int PF_K_STRIDE = D + 8;                      // elements; the padding spreads rows over the banks
 constexpr int PF_V_STRIDE = PF_BN + 8;
 constexpr int PF_K_CHUNKS = PF_BN * D / 8;              // 16-byte pieces of a K tile
@@ -491,7 +492,7 @@ constexpr int PF_V_CHUNKS = D * PF_BN / 8;
 constexpr int PF_K_PER_THREAD = (PF_K_CHUNKS + PF_THREADS - 1) / PF_THREADS;
 constexpr int PF_V_PER_THREAD = (PF_V_CHUNKS + PF_THREADS - 1) / PF_THREADS;
 
-__global__ __launch_bounds__(PF_THREADS, 2) void attn_prefill_kernel(
+__global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_kernel(
     const bf16_t* __restrict__ qkv, int64_t q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ positions, const int32_t* __restrict__ cu_q,
     const int32_t* __restrict__ block_table, int table_width, bf16_t* __restrict__ out, int num_requests, int heads,
@@ -506,8 +507,9 @@ __global__ __launch_bounds__(PF_THREADS, 2) void attn_prefill_kernel(
   const int group = heads / kv_heads;
   const float scale_log2 = scale * 1.4426950408889634f;      // scores in units of log 2: weights are exp2
 
-  // ---- which tokens: blockIdx.x counts tiles of PF_BM tokens over the requests that are served here
-  int tile = blockIdx.x;
+  // ---- which tokens: tiles of PF_BM tokens over the requests that are served here, the last first: the late
+  // tokens of a portion see the most keys, and the longest work should start first
+  int tile = gridDim.y - 1 - blockIdx.y;
   int request = 0, begin = 0, end = 0;
   for (; request < num_requests; ++request) {
     begin = cu_q[request];
@@ -518,7 +520,7 @@ __global__ __launch_bounds__(PF_THREADS, 2) void attn_prefill_kernel(
     tile -= tiles;
   }
   if (request >= num_requests) return;
-  const int head = blockIdx.y;
+  const int head = blockIdx.x;                            // heads vary fastest: the heavy tiles of all heads start first
   const int kh = head / group;
   const int token0 = begin + tile * PF_BM;
   const int columns = min(PF_BM, end - token0);           // of the workgroup
@@ -555,81 +557,87 @@ __global__ __launch_bounds__(PF_THREADS, 2) void attn_prefill_kernel(
   }
 
   // ---- staging of one tile in registers: 16-byte pieces of K rows and of V^T rows
-  uint4 k_stage[PF_K_PER_THREAD], v_stage[PF_V_PER_THREAD];
-  auto fetch = [&](int k0) {
-    // the four blocks of 16 keys of the tile: live if they overlap the keys this workgroup reads
+  // PF_DEPTH tiles are in flight: a tile's trip from memory is longer than the work on a tile
+  uint4 k_stages[PF_DEPTH][PF_K_PER_THREAD], v_stages[PF_DEPTH][PF_V_PER_THREAD];
+  // Every thread issues the same number of loads for every tile, with no branch around them: pieces that
+  // belong to no page read the start of the cache instead and are cleared when they are stored.
+  auto block_live = [&](int key) { return key <= key_end && key + 15 >= key_begin; };
+  auto fetch = [&](int k0, uint4 (&k_stage)[PF_K_PER_THREAD], uint4 (&v_stage)[PF_V_PER_THREAD]) {
     int64_t base[4];
     int offset[4];
-    bool live[4];
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       const int key = k0 + 16 * b;
-      live[b] = key <= key_end && key + 15 >= key_begin;
-      base[b] = 0;
-      offset[b] = 0;
-      if (live[b]) {
-        const int page = table[key / block_size];
-        base[b] = (static_cast<int64_t>(page) * kv_heads + kh) * block_size * D;
-        offset[b] = key % block_size;
-      }
+      const bool live = block_live(key);
+      const int page = live ? table[key / block_size] : 0;
+      base[b] = live ? (static_cast<int64_t>(page) * kv_heads + kh) * block_size * D : 0;
+      offset[b] = live ? key % block_size : 0;
     }
 #pragma unroll
     for (int i = 0; i < PF_K_PER_THREAD; ++i) {
-      const int c = tid + i * PF_THREADS;
-      k_stage[i] = uint4{0u, 0u, 0u, 0u};
-      if (c < PF_K_CHUNKS) {
-        const int row = c / (D / 8);
-        const int piece = c % (D / 8);
-        const int b = row / 16;
-        if (live[b])
-          k_stage[i] = *reinterpret_cast<const uint4*>(k_cache + base[b] + static_cast<int64_t>(offset[b] + row % 16) * D + 8 * piece);
-      }
+      const int c = min(tid + i * PF_THREADS, PF_K_CHUNKS - 1);
+      const int row = c / (D / 8);
+      const int piece = c % (D / 8);
+      const int b = row / 16;
+      const int64_t base_b = b == 0 ? base[0] : (b == 1 ? base[1] : (b == 2 ? base[2] : base[3]));
+      const int offset_b = b == 0 ? offset[0] : (b == 1 ? offset[1] : (b == 2 ? offset[2] : offset[3]));
+      k_stage[i] = *reinterpret_cast<const uint4*>(k_cache + base_b + static_cast<int64_t>(offset_b + row % 16) * D + 8 * piece);
     }
 #pragma unroll
     for (int i = 0; i < PF_V_PER_THREAD; ++i) {
-      const int c = tid + i * PF_THREADS;
-      v_stage[i] = uint4{0u, 0u, 0u, 0u};
-      if (c < PF_V_CHUNKS) {
-        const int d = c / 8;
-        const int piece = c % 8;              // 8 keys each
-        const int b = piece / 2;
-        if (live[b]) {
-          uint4 raw = *reinterpret_cast<const uint4*>(v_cache + base[b] + static_cast<int64_t>(d) * block_size + offset[b] + 8 * (piece % 2));
-          // slots after the last key of this workgroup were not written by this request: cleared (0 * NaN)
-          const int written = key_end - (k0 + 8 * piece) + 1;
-          if (written < 8) {
-            uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              w[e] = written >= 2 * e + 2 ? w[e] : (written == 2 * e + 1 ? (w[e] & 0x0000ffffu) : 0u);
-            raw = uint4{w[0], w[1], w[2], w[3]};
-          }
-          v_stage[i] = raw;
-        }
-      }
+      const int c = min(tid + i * PF_THREADS, PF_V_CHUNKS - 1);
+      const int d = c / 8;
+      const int piece = c % 8;              // 8 keys each
+      const int b = piece / 2;
+      const int64_t base_b = b == 0 ? base[0] : (b == 1 ? base[1] : (b == 2 ? base[2] : base[3]));
+      const int offset_b = b == 0 ? offset[0] : (b == 1 ? offset[1] : (b == 2 ? offset[2] : offset[3]));
+      v_stage[i] = *reinterpret_cast<const uint4*>(v_cache + base_b + static_cast<int64_t>(d) * block_size + offset_b + 8 * (piece % 2));
     }
   };
-  auto stash = [&]() {
+  auto stash = [&](int k0, const uint4 (&k_stage)[PF_K_PER_THREAD], const uint4 (&v_stage)[PF_V_PER_THREAD]) {
+    if (k0 >= key_begin && k0 + PF_BN - 1 <= key_end) {
+      // every key of the tile is one this workgroup reads: nothing to clear
+#pragma unroll
+      for (int i = 0; i < PF_K_PER_THREAD; ++i) {
+        const int c = tid + i * PF_THREADS;
+        if (c < PF_K_CHUNKS) *reinterpret_cast<uint4*>(k_lds + (c / (D / 8)) * PF_K_STRIDE + 8 * (c % (D / 8))) = k_stage[i];
+      }
+#pragma unroll
+      for (int i = 0; i < PF_V_PER_THREAD; ++i) {
+        const int c = tid + i * PF_THREADS;
+        if (c < PF_V_CHUNKS) *reinterpret_cast<uint4*>(v_lds + (c / 8) * PF_V_STRIDE + 8 * (c % 8)) = v_stage[i];
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < PF_K_PER_THREAD; ++i) {
       const int c = tid + i * PF_THREADS;
-      if (c < PF_K_CHUNKS) *reinterpret_cast<uint4*>(k_lds + (c / (D / 8)) * PF_K_STRIDE + 8 * (c % (D / 8))) = k_stage[i];
+      if (c < PF_K_CHUNKS) {
+        const int row = c / (D / 8);
+        const uint4 raw = block_live(k0 + row / 16 * 16) ? k_stage[i] : uint4{0u, 0u, 0u, 0u};
+        *reinterpret_cast<uint4*>(k_lds + row * PF_K_STRIDE + 8 * (c % (D / 8))) = raw;
+      }
     }
 #pragma unroll
     for (int i = 0; i < PF_V_PER_THREAD; ++i) {
       const int c = tid + i * PF_THREADS;
-      if (c < PF_V_CHUNKS) *reinterpret_cast<uint4*>(v_lds + (c / 8) * PF_V_STRIDE + 8 * (c % 8)) = v_stage[i];
+      if (c < PF_V_CHUNKS) {
+        // slots after the last key of this workgroup were not written by this request, and blocks outside the
+        // keys of this workgroup were not read: cleared (a weight of zero times NaN would still be NaN)
+        const int first_key = k0 + 8 * (c % 8);
+        const int written = block_live(first_key / 16 * 16) ? key_end - first_key + 1 : 0;
+        const uint32_t w[4] = {v_stage[i].x, v_stage[i].y, v_stage[i].z, v_stage[i].w};
+        uint32_t m[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          m[e] = written >= 2 * e + 2 ? w[e] : (written == 2 * e + 1 ? (w[e] & 0x0000ffffu) : 0u);
+        *reinterpret_cast<uint4*>(v_lds + (c / 8) * PF_V_STRIDE + 8 * (c % 8)) = uint4{m[0], m[1], m[2], m[3]};
+      }
     }
   };
 
-  const int tile0 = key_begin / PF_BN * PF_BN;
-  fetch(tile0);
-  for (int k0 = tile0; k0 <= key_end; k0 += PF_BN) {
-    __syncthreads();                       // every wave is done with the tile in LDS
-    stash();
-    __syncthreads();
-    if (k0 + PF_BN <= key_end) fetch(k0 + PF_BN);      // in flight while this tile is used
-    if (wave_cols <= 0 || k0 > wave_last || k0 + PF_BN - 1 < wave_first) continue;
+  auto compute = [&](int k0) {
+    if (wave_cols <= 0 || k0 > wave_last || k0 + PF_BN - 1 < wave_first) return;
 
     // ---- scores: 64 keys x the wave's columns
     floatx4 s[PF_MB][4];
@@ -655,7 +663,10 @@ __global__ __launch_bounds__(PF_THREADS, 2) void attn_prefill_kernel(
         }
       }
     }
-    // ---- softmax step per column
+    // ---- softmax step per column. A tile whose keys every column of the wave sees needs no mask: that is
+    // every tile but those on the diagonal and at a window's edge.
+    const bool tile_open = k0 + PF_BN - 1 <= pos0 + wave_col0 &&
+                           (window <= 0 || k0 >= pos0 + wave_col0 + wave_cols - window);
     bf16x8 p_reg[PF_MB][2];
     float alpha[PF_MB];
 #pragma unroll
@@ -663,15 +674,26 @@ __global__ __launch_bounds__(PF_THREADS, 2) void attn_prefill_kernel(
       const int last = col_pos[mb];
       const int first = window > 0 ? max(0, last - window + 1) : 0;
       float best = -INFINITY;
+      if (tile_open) {
 #pragma unroll
-      for (int kb = 0; kb < 4; ++kb)
+        for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = k0 + 16 * kb + 4 * g + i;
-          const float v = (key >= first && key <= last) ? s[mb][kb][i] * scale_log2 : -INFINITY;
-          s[mb][kb][i] = v;
-          best = fmaxf(best, v);
-        }
+          for (int i = 0; i < 4; ++i) {
+            const float v = s[mb][kb][i] * scale_log2;
+            s[mb][kb][i] = v;
+            best = fmaxf(best, v);
+          }
+      } else {
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = k0 + 16 * kb + 4 * g + i;
+            const float v = (key >= first && key <= last) ? s[mb][kb][i] * scale_log2 : -INFINITY;
+            s[mb][kb][i] = v;
+            best = fmaxf(best, v);
+          }
+      }
       best = fmaxf(best, __shfl_xor(best, 16, DISTIE_WAVE));
       best = fmaxf(best, __shfl_xor(best, 32, DISTIE_WAVE));
       const float m_new = fmaxf(m_run[mb], best);
@@ -713,8 +735,24 @@ __global__ __launch_bounds__(PF_THREADS, 2) void attn_prefill_kernel(
         for (int mb = 0; mb < PF_MB; ++mb)
           o_acc[mb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_reg[mb][ks], v, o_acc[mb][db], 0, 0, 0);
       }
-  }
+  };
 
+  // PF_DEPTH tiles of loads are in flight (tiles past the last key load the start of the cache and are not used)
+  const int tile0 = key_begin / PF_BN * PF_BN;
+#pragma unroll
+  for (int d = 0; d < PF_DEPTH; ++d) fetch(tile0 + d * PF_BN, k_stages[d], v_stages[d]);
+  for (int k0 = tile0; k0 <= key_end; k0 += PF_DEPTH * PF_BN) {
+#pragma unroll
+    for (int d = 0; d < PF_DEPTH; ++d) {
+      const int k = k0 + d * PF_BN;
+      if (k > key_end) break;
+      __syncthreads();                       // every wave is done with the tile in LDS
+      stash(k, k_stages[d], v_stages[d]);
+      __syncthreads();
+      fetch(k + PF_DEPTH * PF_BN, k_stages[d], v_stages[d]);
+      compute(k);
+    }
+  }
   // ---- write: the lane holds columns 4g..4g+3 of each block, output dim 16 db + r
 #pragma unroll
   for (int mb = 0; mb < PF_MB; ++mb) {
@@ -747,7 +785,8 @@ extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, 
       num_requests < 1 || heads > 65535 || min_q_len < 1)
     return DISTIE_BAD_ARGUMENT;
   const int tiles = (tokens + PF_BM - 1) / PF_BM + num_requests;     // an upper bound; spare blocks leave at once
-  attn_prefill_kernel<<<dim3(tiles, heads), PF_THREADS, 0, stream>>>(
+  if (tiles > 65535) return DISTIE_BAD_ARGUMENT;
+  attn_prefill_kernel<<<dim3(heads, tiles), PF_THREADS, 0, stream>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),
       positions, cu_q, block_table, table_width, static_cast<bf16_t*>(out), num_requests, heads, kv_heads, block_size,
       scale, window, min_q_len);
