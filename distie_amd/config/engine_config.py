@@ -41,6 +41,7 @@ class EngineConfig:
     token_budget: int = DEFAULT_TOKEN_BUDGET
     max_model_len: Optional[int] = None     # None = the model's max positions
     use_graphs: bool = True
+    packed_weights: bool = True             # a second copy of the weights in the matrix cores' order, for decode
     step_stats: int = 0
     seed: int = 0
 

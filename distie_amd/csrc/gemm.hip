@@ -236,3 +236,167 @@ extern "C" int distie_gemm_skinny_bf16(const void* x, const void* w, const float
 #undef SKINNY
   return launch_status();
 }
+
+// ---------------------------------------------------------------- skinny on packed weights
+// A second copy of a weight in the order in which the matrix cores take it: tiles of 16 rows x 32 k,
+// the 1 KB of a tile in lane order (lane = 16 g + r holds W[16 nb + r][32 kt + 8 g .. + 7]), tiles
+// ordered [row block nb][k tile kt], rows and k padded with zeros to whole tiles. One load instruction
+// of a wave then reads 1 KB of consecutive bytes (eight whole cache lines) instead of 64 bytes from
+// each of 16 rows, which brought 15-25 % on every shape measured.
+//
+// GATED: the weight stacks a gate and an up projection ([2 I, K]); a row block holds gate rows
+// 8 nb .. + 7 and then up rows 8 nb .. + 7, so that one wave owns both halves of eight outputs, and
+// the kernel writes silu(gate) * up ([M, I]) itself. A gated product is never cut along K.
+#define PK_TILE 512         // elements of a tile
+
+__global__ __launch_bounds__(256) void pack_weight_kernel(const bf16_t* __restrict__ w, bf16_t* __restrict__ out,
+                                                          int N, int K, int row_blocks, int k_tiles, int gated_half) {
+  const int64_t chunk = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;     // 8 elements
+  const int64_t chunks = static_cast<int64_t>(row_blocks) * k_tiles * 64;
+  if (chunk >= chunks) return;
+  const int lane = static_cast<int>(chunk % 64);
+  const int64_t tile = chunk / 64;
+  const int kt = static_cast<int>(tile % k_tiles);
+  const int64_t nb = tile / k_tiles;
+  const int r = lane % 16, g = lane / 16;
+  int64_t n;
+  bool in;
+  if (gated_half > 0) {
+    const int64_t j = 8 * nb + r % 8;
+    n = (r / 8) * static_cast<int64_t>(gated_half) + j;
+    in = j < gated_half;
+  } else {
+    n = 16 * nb + r;
+    in = n < N;
+  }
+  const int k = 32 * kt + 8 * g;
+  uint4 v = {0u, 0u, 0u, 0u};
+  if (in && k < K) v = *reinterpret_cast<const uint4*>(w + n * K + k);       // K is a multiple of 8
+  *reinterpret_cast<uint4*>(out + chunk * 8) = v;
+}
+
+// Elements of the packed copy of a [N, K] weight (gated: N = 2 I).
+extern "C" int64_t distie_packed_elements(int N, int K, int gated) {
+  const int64_t row_blocks = gated ? (N / 2 + 7) / 8 : (N + 15) / 16;
+  return row_blocks * ((K + 31) / 32) * PK_TILE;
+}
+
+extern "C" int distie_pack_weight(const void* w, void* out, int N, int K, int gated, hipStream_t stream) {
+  if (N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
+  const int row_blocks = gated ? (N / 2 + 7) / 8 : (N + 15) / 16;
+  const int k_tiles = (K + 31) / 32;
+  const int64_t chunks = static_cast<int64_t>(row_blocks) * k_tiles * 64;
+  pack_weight_kernel<<<static_cast<unsigned>((chunks + 255) / 256), 256, 0, stream>>>(
+      static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), N, K, row_blocks, k_tiles, gated ? N / 2 : 0);
+  return launch_status();
+}
+
+// The four tiles of one k-step for COUNT k-steps: every load issued before the first product.
+template <int COUNT>
+__device__ __forceinline__ void packed_steps(const bf16_t* wp, const bf16_t* xp, int t_begin, int steps, int& step,
+                                             floatx4& acc) {
+  bf16x8 a[COUNT][4], xb[COUNT][4];
+#pragma unroll
+  for (int u = 0; u < COUNT; ++u) {
+    const int t = t_begin + 4 * step;
+    step = step + 1 == steps ? 0 : step + 1;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      a[u][j] = *reinterpret_cast<const bf16x8*>(wp + static_cast<int64_t>(t + j) * PK_TILE);
+      xb[u][j] = *reinterpret_cast<const bf16x8*>(xp + 32 * (t + j));
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < COUNT; ++u)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][j], xb[u][j], acc, 0, 0, 0);
+}
+
+// One wave per block. blockIdx.x: row block; blockIdx.y: slice of K (tiles_per_slice is a multiple of 4).
+// M <= 16. Not GATED: as gemm_skinny_kernel (slices side by side, bias on slice 0). GATED: y is
+// [M, N / 2], one slice.
+template <typename Y, bool GATED>
+__global__ __launch_bounds__(64) void gemm_packed_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                         const float* __restrict__ bias, Y* __restrict__ y,
+                                                         int M, int N, int K, int tiles_per_slice) {
+  constexpr int UN = 4;
+  const int lane = threadIdx.x;
+  const int r = lane % 16;
+  const int g = lane / 16;
+  const int k_tiles = (K + 31) / 32;
+  const int t_begin = blockIdx.y * tiles_per_slice;
+  const int t_end = min(k_tiles, t_begin + tiles_per_slice);
+  const int t_whole = min(K / 32, t_end);                 // tiles before this one lie inside K for every lane
+
+  const bf16_t* wp = w + static_cast<int64_t>(blockIdx.x) * k_tiles * PK_TILE + lane * 8;
+  const bf16_t* xp = x + static_cast<int64_t>(min(r, M - 1)) * K + 8 * g;      // rows beyond M: results dropped
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+
+  const int steps = max(0, t_whole - t_begin) / 4;
+  int step = steps > 0 ? static_cast<int>(blockIdx.x % steps) : 0;   // staggered start, wraps around
+  int it = 0;
+  for (; it + UN <= steps; it += UN) packed_steps<UN>(wp, xp, t_begin, steps, step, acc);
+  switch (steps - it) {
+    case 3: packed_steps<3>(wp, xp, t_begin, steps, step, acc); break;
+    case 2: packed_steps<2>(wp, xp, t_begin, steps, step, acc); break;
+    case 1: packed_steps<1>(wp, xp, t_begin, steps, step, acc); break;
+    default: break;
+  }
+  // the slice's last tiles; the very last may reach beyond K (the copy holds zeros there, x is not read)
+  for (int t = t_begin + 4 * steps; t < t_end; ++t) {
+    const bf16x8 a = *reinterpret_cast<const bf16x8*>(wp + static_cast<int64_t>(t) * PK_TILE);
+    bf16x8 xb = {};
+    if (32 * t + 8 * g < K) xb = *reinterpret_cast<const bf16x8*>(xp + 32 * t);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, xb, acc, 0, 0, 0);
+  }
+
+  // acc[i] = sum for row 4 g + i of the block and x row r
+  if constexpr (GATED) {
+    const int half = N / 2;
+    float up[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) up[i] = __shfl_xor(acc[i], 32, 64);          // rows 8..15 of the block: up
+    if (g < 2 && r < M) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int64_t n = static_cast<int64_t>(blockIdx.x) * 8 + 4 * g + i;
+        if (n >= half) continue;
+        float gate = acc[i], u = up[i];
+        if (bias != nullptr) { gate += bias[n]; u += bias[half + n]; }
+        y[static_cast<int64_t>(r) * half + n] = from_float<Y>(gate / (1.f + expf(-gate)) * u);
+      }
+    }
+  } else {
+    Y* out = y + static_cast<int64_t>(blockIdx.y) * M * N;
+    const bool with_bias = bias != nullptr && blockIdx.y == 0;
+    if (r < M) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int64_t n = static_cast<int64_t>(blockIdx.x) * 16 + 4 * g + i;
+        if (n < N) out[static_cast<int64_t>(r) * N + n] = from_float<Y>(acc[i] + (with_bias ? bias[n] : 0.f));
+      }
+    }
+  }
+}
+
+// y: as distie_gemm_skinny_bf16 (the same cut along K); gated: [M, N / 2] of y_dtype.
+extern "C" int distie_gemm_packed_bf16(const void* x, const void* w_packed, const float* bias, void* y, int y_dtype,
+                                       int M, int N, int K, int gated, hipStream_t stream) {
+  if (M <= 0) return 0;
+  if (M > 16 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
+  int slices = 1, k_per_slice = (K + SK_KSTEP - 1) / SK_KSTEP * SK_KSTEP;
+  if (!gated) skinny_plan(N, K, &slices, &k_per_slice);
+  if (slices > 1 && y_dtype != DISTIE_F32) return DISTIE_BAD_ARGUMENT;
+  const int row_blocks = gated ? (N / 2 + 7) / 8 : (N + 15) / 16;
+  dim3 grid(row_blocks, slices);
+  const bf16_t* xb = static_cast<const bf16_t*>(x);
+  const bf16_t* wb = static_cast<const bf16_t*>(w_packed);
+  if (gated) {
+    DISTIE_DISPATCH(y_dtype, Y, (gemm_packed_kernel<Y, true><<<grid, 64, 0, stream>>>(
+                                    xb, wb, bias, static_cast<Y*>(y), M, N, K, k_per_slice / 32)));
+  } else {
+    DISTIE_DISPATCH(y_dtype, Y, (gemm_packed_kernel<Y, false><<<grid, 64, 0, stream>>>(
+                                    xb, wb, bias, static_cast<Y*>(y), M, N, K, k_per_slice / 32)));
+  }
+  return launch_status();
+}

@@ -74,7 +74,7 @@ class LLM:
         if ops is None:
             from ..kernels.hip_ops import HipOps
 
-            ops = HipOps(device)
+            ops = HipOps(device, packed_weights=self.engine_config.packed_weights)
         self.ops = ops
         if model is not None:
             self.model_config = load_model_config(model)

@@ -78,6 +78,12 @@ class Model:
         # tied: one buffer (worker/src/inference/qwen2/model.py:302-303)
         self.head = self.embedding if self.tied_head else fetch(s.head.prefix + "weight").contiguous()
 
+    def prepare(self, ops) -> None:
+        """Once after loading, with the kernel surface the model will run on."""
+        for part in self._parts():
+            part.prepare(ops)
+        ops.prepare_linear(self.head)
+
     def cache_requirements(self) -> list:
         return [block.mixer.cache_requirement() for block in self.blocks]
 

@@ -29,6 +29,7 @@ class ModelRunner:
         self.max_model_len = int(max_model_len or model.spec.max_positions)
         self.builder = BatchBuilder(cache, self.max_model_len, ops.device, model.spec.vocab_size)
         self.graphs = None          # set by the engine when captured decode steps are on
+        model.prepare(ops)
 
     def step(self, entries: Sequence[StepEntry], reserve: bool = True) -> Optional[torch.Tensor]:
         """-> float32 [wanted, vocab] in the order of the entries and of their `want`

@@ -77,6 +77,16 @@ class Ops(abc.ABC):
         read (the HIP kernels return partial sums over slices of K for small batches); parts
         hand the result on to those operations and do nothing else with it."""
 
+    def prepare_linear(self, weight: torch.Tensor, gated: bool = False) -> None:
+        """Called once for every weight of a `linear` after it is loaded (`gated`: the weight of a
+        `linear_silu_mul`). An implementation may build what its products need beside the tensor
+        (the HIP kernels keep a second copy in the matrix cores' order for small batches)."""
+
+    def linear_silu_mul(self, x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
+        """silu_mul(linear(x, gate_up_weight)) with gate_up_weight [2I, K] -> act [T, I]; an
+        implementation may fuse the two."""
+        return self.silu_mul(self.linear(x, gate_up_weight))
+
     @abc.abstractmethod
     def linear_f32out(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         """As `linear` without bias, result in float32 (the logits)."""

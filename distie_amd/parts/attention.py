@@ -65,6 +65,10 @@ class Attention(Mixer):
             self.out_bias_t = tensors["o_proj.bias"].float().contiguous()
         self.position.to_device(self.out_weight.device)
 
+    def prepare(self, ops) -> None:
+        ops.prepare_linear(self.qkv_weight)
+        ops.prepare_linear(self.out_weight)
+
     def forward(self, ops, x, ctx, cache, writes_cache: bool):
         qkv = ops.linear(x, self.qkv_weight, self.qkv_bias_t)
         qkv = ops.rope_kv_write(qkv, ctx.meta, cache.group, cache.k, cache.v, self.position.rotary(),

@@ -79,6 +79,10 @@ class Part(abc.ABC):
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         """Take the tensors (by local name, on the device, in the kept dtype)."""
 
+    def prepare(self, ops) -> None:
+        """After `load`, once, with the kernel surface the part will run on: announce the weights
+        of matrix products (`ops.prepare_linear`)."""
+
 
 class Norm(Part):
     @abc.abstractmethod

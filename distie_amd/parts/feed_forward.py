@@ -29,8 +29,12 @@ class SwiGLU(FeedForward):
         self.gate_up_weight = torch.cat([gate.to(dtype), up.to(dtype)], dim=0).contiguous()
         self.down_weight = tensors["down_proj.weight"].contiguous()
 
+    def prepare(self, ops) -> None:
+        ops.prepare_linear(self.gate_up_weight, gated=True)
+        ops.prepare_linear(self.down_weight)
+
     def forward(self, ops, x, ctx):
-        return ops.linear(ops.silu_mul(ops.linear(x, self.gate_up_weight)), self.down_weight)
+        return ops.linear(ops.linear_silu_mul(x, self.gate_up_weight), self.down_weight)
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

@@ -92,6 +92,52 @@ def test_gemm_skinny_bf16(ops, M, N, K):
     close(got, want + b.double(), torch.bfloat16, scale=want.abs().max().item())
 
 
+@pytest.mark.parametrize("M", [1, 3, 8, 16])
+@pytest.mark.parametrize("N,K", [(48, 128), (100, 264), (1536, 1536), (333, 8960), (2050, 72), (16, 8), (7, 40)])
+def test_gemm_packed_bf16(ops, M, N, K):
+    """The same products through the weight's packed copy (what `prepare_linear` leaves): rows and
+    k that do not fill a tile, one slice and several, with and without a bias."""
+    from distie_amd.kernels.hip_ops import PartialSums
+
+    x, w, b = rand(M, K, dtype=torch.bfloat16, seed=1), rand(N, K, dtype=torch.bfloat16, seed=2), rand(N, seed=3)
+    natural = ops.dense(ops.linear(x, w, b)).float()
+    ops.prepare_linear(w)
+    assert w._distie_packed.numel() == -(-N // 16) * -(-K // 32) * 512
+    want = x.double() @ w.double().T
+    got = ops.linear_f32out(x, w)
+    close(got, want, torch.float32, scale=5 * want.abs().max().item())
+    part = ops.linear(x, w, b)
+    assert isinstance(part, PartialSums) == (K >= 768)
+    got = ops.dense(part)
+    assert got.dtype == torch.bfloat16
+    close(got, want + b.double(), torch.bfloat16, scale=want.abs().max().item())
+    # the packed and the natural kernel add the same products in another order: float32 rounding only
+    assert (got.float() - natural).abs().max().item() <= 2 ** -7 * want.abs().max().item()
+
+
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("I,K", [(88, 2048), (8, 32), (172, 64), (250, 96), (4484, 1536), (13, 72)])
+def test_linear_silu_mul_fused(ops, M, I, K):
+    x = rand(M, K, dtype=torch.bfloat16, seed=1)
+    w = rand(2 * I, K, dtype=torch.bfloat16, seed=5, scale=2.0 / K ** 0.5)
+    gu = x.double() @ w.double().T
+    want = gu[:, :I] / (1 + torch.exp(-gu[:, :I])) * gu[:, I:]
+    # unfused, a product that is not cut along K is rounded to bfloat16 before the activation: gate, up
+    # and result each carry a rounding (2^-8 of the value at most), where the fused kernel rounds once
+    unfused = ops.linear_silu_mul(x, w)
+    close(unfused, want, torch.bfloat16, scale=2 * want.abs().max().item())
+    ops.prepare_linear(w, gated=True)
+    assert w._distie_gated.numel() == -(-I // 8) * -(-K // 32) * 512
+    got = ops.linear_silu_mul(x, w)
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (M, I)
+    close(got, want, torch.bfloat16, scale=want.abs().max().item())
+    # more rows than the fused kernel takes: the unfused path, same result
+    big = rand(40, K, dtype=torch.bfloat16, seed=2)
+    gu = big.double() @ w.double().T
+    want = gu[:, :I] / (1 + torch.exp(-gu[:, :I])) * gu[:, I:]
+    close(ops.linear_silu_mul(big, w), want, torch.bfloat16, scale=2 * want.abs().max().item())
+
+
 def test_partial_sums_are_added_by_their_readers(ops):
     """A product over a long K comes back as slices; norm, activation and rotation add them."""
     from distie_amd.kernels.hip_ops import PartialSums
