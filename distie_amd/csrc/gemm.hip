@@ -239,55 +239,52 @@ extern "C" int distie_gemm_skinny_bf16(const void* x, const void* w, const float
 
 // ---------------------------------------------------------------- skinny on packed weights
 // A second copy of a weight in the order in which the matrix cores take it: tiles of 16 rows x 32 k,
-// the 1 KB of a tile in lane order (lane = 16 g + r holds W[16 nb + r][32 kt + 8 g .. + 7]), tiles
-// ordered [row block nb][k tile kt], rows and k padded with zeros to whole tiles. One load instruction
-// of a wave then reads 1 KB of consecutive bytes (eight whole cache lines) instead of 64 bytes from
-// each of 16 rows, which brought 15-25 % on every shape measured.
+// the 1 KB of a tile in lane order (lane = 16 g + r holds row r of the block, k 32 kt + 8 g .. + 7), tiles
+// ordered [row block][k tile], k padded with zeros to whole tiles. One load instruction of a wave then
+// reads 1 KB of consecutive bytes (eight whole cache lines) instead of 64 bytes from each of 16 rows,
+// which brought 15-25 % on every shape measured.
 //
-// GATED: the weight stacks a gate and an up projection ([2 I, K]); a row block holds gate rows
-// 8 nb .. + 7 and then up rows 8 nb .. + 7, so that one wave owns both halves of eight outputs, and
-// the kernel writes silu(gate) * up ([M, I]) itself. A gated product is never cut along K.
+// Which row of W sits at which place of a block is given by a row map (-1: a row of zeros), so that a
+// wave can own the rows its epilogue needs together:
+//  * PLAIN: rows in order.
+//  * GATED: the weight stacks a gate and an up projection ([2 I, K]); block b holds gate rows 8 b .. + 7 and
+//    then up rows 8 b .. + 7, and the kernel writes silu(gate) * up ([M, I]) itself.
+//  * ROTARY: the weight stacks q, k and v heads of size D, all of D rotated (pairs j, j + D / 2). Block
+//    (head, s) of a q or k head holds its rows 8 s .. + 7 and D / 2 + 8 s .. + 7, blocks of v heads hold 16 rows
+//    in order. The kernel adds the bias, turns the pairs by the token's angle, writes q, k, v to the
+//    [M, N] result and k and v into the paged cache.
+// In all of them lanes 0-31 of the accumulator hold rows 0-7 of the block and lanes 32-63 rows 8-15 for
+// the same tokens, so partners meet through one exchange between lane l and lane l ^ 32.
 #define PK_TILE 512         // elements of a tile
+#define PK_PLAIN 0
+#define PK_GATED 1
+#define PK_ROTARY 2
 
-__global__ __launch_bounds__(256) void pack_weight_kernel(const bf16_t* __restrict__ w, bf16_t* __restrict__ out,
-                                                          int N, int K, int row_blocks, int k_tiles, int gated_half) {
+__global__ __launch_bounds__(256) void pack_rows_kernel(const bf16_t* __restrict__ w, bf16_t* __restrict__ out,
+                                                        const int32_t* __restrict__ row_map, int K, int64_t row_blocks,
+                                                        int k_tiles) {
   const int64_t chunk = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;     // 8 elements
-  const int64_t chunks = static_cast<int64_t>(row_blocks) * k_tiles * 64;
-  if (chunk >= chunks) return;
+  if (chunk >= row_blocks * k_tiles * 64) return;
   const int lane = static_cast<int>(chunk % 64);
   const int64_t tile = chunk / 64;
   const int kt = static_cast<int>(tile % k_tiles);
   const int64_t nb = tile / k_tiles;
-  const int r = lane % 16, g = lane / 16;
-  int64_t n;
-  bool in;
-  if (gated_half > 0) {
-    const int64_t j = 8 * nb + r % 8;
-    n = (r / 8) * static_cast<int64_t>(gated_half) + j;
-    in = j < gated_half;
-  } else {
-    n = 16 * nb + r;
-    in = n < N;
-  }
-  const int k = 32 * kt + 8 * g;
+  const int64_t n = row_map[nb * 16 + lane % 16];
+  const int k = 32 * kt + 8 * (lane / 16);
   uint4 v = {0u, 0u, 0u, 0u};
-  if (in && k < K) v = *reinterpret_cast<const uint4*>(w + n * K + k);       // K is a multiple of 8
+  if (n >= 0 && k < K) v = *reinterpret_cast<const uint4*>(w + n * K + k);       // K is a multiple of 8
   *reinterpret_cast<uint4*>(out + chunk * 8) = v;
 }
 
-// Elements of the packed copy of a [N, K] weight (gated: N = 2 I).
-extern "C" int64_t distie_packed_elements(int N, int K, int gated) {
-  const int64_t row_blocks = gated ? (N / 2 + 7) / 8 : (N + 15) / 16;
-  return row_blocks * ((K + 31) / 32) * PK_TILE;
-}
-
-extern "C" int distie_pack_weight(const void* w, void* out, int N, int K, int gated, hipStream_t stream) {
-  if (N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
-  const int row_blocks = gated ? (N / 2 + 7) / 8 : (N + 15) / 16;
+// out: row_blocks * ceil(K / 32) * 512 elements; row_map: int32 [16 * row_blocks] on the device, entries in
+// [-1, N) (the caller's duty).
+extern "C" int distie_pack_rows(const void* w, void* out, const int32_t* row_map, int row_blocks, int K,
+                                hipStream_t stream) {
+  if (row_blocks <= 0 || K <= 0 || K % 8 != 0) return DISTIE_BAD_ARGUMENT;
   const int k_tiles = (K + 31) / 32;
   const int64_t chunks = static_cast<int64_t>(row_blocks) * k_tiles * 64;
-  pack_weight_kernel<<<static_cast<unsigned>((chunks + 255) / 256), 256, 0, stream>>>(
-      static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), N, K, row_blocks, k_tiles, gated ? N / 2 : 0);
+  pack_rows_kernel<<<static_cast<unsigned>((chunks + 255) / 256), 256, 0, stream>>>(
+      static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), row_map, K, row_blocks, k_tiles);
   return launch_status();
 }
 
@@ -312,28 +309,15 @@ __device__ __forceinline__ void packed_steps(const bf16_t* wp, const bf16_t* xp,
     for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][j], xb[u][j], acc, 0, 0, 0);
 }
 
-// One wave per block. blockIdx.x: row block; blockIdx.y: slice of K (tiles_per_slice is a multiple of 4).
-// M <= 16. Not GATED: as gemm_skinny_kernel (slices side by side, bias on slice 0). GATED: y is
-// [M, N / 2], one slice.
-template <typename Y, bool GATED>
-__global__ __launch_bounds__(64) void gemm_packed_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                         const float* __restrict__ bias, Y* __restrict__ y,
-                                                         int M, int N, int K, int tiles_per_slice) {
+// The sums of one row block over the k tiles [t_begin, t_end): acc[i] = row 4 g + i of the block, x row r.
+// wp: the block's first tile + 8 * lane; xp: x row min(r, M - 1) + 8 g.
+__device__ __forceinline__ floatx4 packed_accumulate(const bf16_t* wp, const bf16_t* xp, int t_begin, int t_end, int K,
+                                                     int g, unsigned stagger) {
   constexpr int UN = 4;
-  const int lane = threadIdx.x;
-  const int r = lane % 16;
-  const int g = lane / 16;
-  const int k_tiles = (K + 31) / 32;
-  const int t_begin = blockIdx.y * tiles_per_slice;
-  const int t_end = min(k_tiles, t_begin + tiles_per_slice);
-  const int t_whole = min(K / 32, t_end);                 // tiles before this one lie inside K for every lane
-
-  const bf16_t* wp = w + static_cast<int64_t>(blockIdx.x) * k_tiles * PK_TILE + lane * 8;
-  const bf16_t* xp = x + static_cast<int64_t>(min(r, M - 1)) * K + 8 * g;      // rows beyond M: results dropped
   floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-
+  const int t_whole = min(K / 32, t_end);                 // tiles before this one lie inside K for every lane
   const int steps = max(0, t_whole - t_begin) / 4;
-  int step = steps > 0 ? static_cast<int>(blockIdx.x % steps) : 0;   // staggered start, wraps around
+  int step = steps > 0 ? static_cast<int>(stagger % steps) : 0;      // staggered start, wraps around
   int it = 0;
   for (; it + UN <= steps; it += UN) packed_steps<UN>(wp, xp, t_begin, steps, step, acc);
   switch (steps - it) {
@@ -342,16 +326,72 @@ __global__ __launch_bounds__(64) void gemm_packed_kernel(const bf16_t* __restric
     case 1: packed_steps<1>(wp, xp, t_begin, steps, step, acc); break;
     default: break;
   }
-  // the slice's last tiles; the very last may reach beyond K (the copy holds zeros there, x is not read)
+  // the last tiles; the very last may reach beyond K (the copy holds zeros there, x is not read)
   for (int t = t_begin + 4 * steps; t < t_end; ++t) {
     const bf16x8 a = *reinterpret_cast<const bf16x8*>(wp + static_cast<int64_t>(t) * PK_TILE);
     bf16x8 xb = {};
     if (32 * t + 8 * g < K) xb = *reinterpret_cast<const bf16x8*>(xp + 32 * t);
     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, xb, acc, 0, 0, 0);
   }
+  return acc;
+}
 
-  // acc[i] = sum for row 4 g + i of the block and x row r
-  if constexpr (GATED) {
+struct RotaryOut {
+  const float2* table;        // [M, D / 2] cosine and sine of each token's angles
+  const int32_t* slots;       // [M] place of each token in the cache
+  bf16_t* k_cache;            // [pages, kv_heads, block_size, D]
+  bf16_t* v_cache;            // [pages, kv_heads, D, block_size]
+  int heads, kv_heads, dim, block_size, write;
+};
+
+static __device__ __forceinline__ uint2 pack_bf16x4(const float v[4]) {
+  uint32_t h[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) h[i] = __builtin_bit_cast(uint16_t, static_cast<bf16_t>(v[i]));
+  return uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+}
+
+// blockIdx.x: row block; blockIdx.y: slice of K (PLAIN only; slices side by side in y, bias on slice 0, as
+// gemm_skinny_kernel). The WAVES waves of a workgroup share the slice's tiles and add their sums through
+// LDS; wave 0 writes. M <= 16.
+template <typename Y, int MODE, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gemm_packed_kernel(const bf16_t* __restrict__ x,
+                                                                 const bf16_t* __restrict__ w,
+                                                                 const float* __restrict__ bias, Y* __restrict__ y,
+                                                                 int M, int N, int K, int tiles_per_slice,
+                                                                 RotaryOut rotary) {
+  const int lane = threadIdx.x % 64;
+  const int wave = threadIdx.x / 64;
+  const int r = lane % 16;
+  const int g = lane / 16;
+  const int k_tiles = (K + 31) / 32;
+  const int s_begin = blockIdx.y * tiles_per_slice;
+  const int s_end = min(k_tiles, s_begin + tiles_per_slice);
+  int t_begin = s_begin, t_end = s_end;
+  if constexpr (WAVES > 1) {
+    const int per_wave = ((s_end - s_begin + WAVES - 1) / WAVES + 3) / 4 * 4;
+    t_begin = min(s_end, s_begin + wave * per_wave);
+    t_end = min(s_end, t_begin + per_wave);
+  }
+  const bf16_t* wp = w + static_cast<int64_t>(blockIdx.x) * k_tiles * PK_TILE + lane * 8;
+  const bf16_t* xp = x + static_cast<int64_t>(min(r, M - 1)) * K + 8 * g;      // rows beyond M: results dropped
+  floatx4 acc = packed_accumulate(wp, xp, t_begin, t_end, K, g, blockIdx.x + wave);
+
+  if constexpr (WAVES > 1) {
+    __shared__ float part[WAVES - 1][4][64];
+    if (wave > 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) part[wave - 1][i][lane] = acc[i];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int v = 0; v < WAVES - 1; ++v)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] += part[v][i][lane];
+  }
+
+  if constexpr (MODE == PK_GATED) {
     const int half = N / 2;
     float up[4];
 #pragma unroll
@@ -364,6 +404,54 @@ __global__ __launch_bounds__(64) void gemm_packed_kernel(const bf16_t* __restric
         float gate = acc[i], u = up[i];
         if (bias != nullptr) { gate += bias[n]; u += bias[half + n]; }
         y[static_cast<int64_t>(r) * half + n] = from_float<Y>(gate / (1.f + expf(-gate)) * u);
+      }
+    }
+  } else if constexpr (MODE == PK_ROTARY) {
+    const int dim = rotary.dim;
+    const int half = dim / 2;
+    const int per_head = dim / 16;                                  // blocks of a head
+    const int rotated_blocks = (rotary.heads + rotary.kv_heads) * per_head;
+    const int b = blockIdx.x;
+    const bool turns = b < rotated_blocks;
+    const int head = b / per_head;                                  // among q, k, v heads in this order
+    const int sub = b % per_head;
+    // the first of this lane's four columns within its head
+    const int d0 = turns ? (g / 2) * half + 8 * sub + 4 * (g % 2) : 16 * sub + 4 * g;
+    float own[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) own[i] = acc[i] + (bias != nullptr ? bias[static_cast<int64_t>(head) * dim + d0 + i] : 0.f);
+    float other[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) other[i] = __shfl_xor(own[i], 32, 64);
+    if (r >= M) return;
+    float v[4];
+    if (turns) {
+      const float2* angles = rotary.table + static_cast<int64_t>(r) * half + 8 * sub + 4 * (g % 2);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float2 cs = angles[i];
+        // first half: x1 cos - x2 sin; second half: x2 cos + x1 sin
+        v[i] = g < 2 ? own[i] * cs.x - other[i] * cs.y : own[i] * cs.x + other[i] * cs.y;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = own[i];
+    }
+    const uint2 packed = pack_bf16x4(v);
+    *reinterpret_cast<uint2*>(y + static_cast<int64_t>(r) * N + static_cast<int64_t>(head) * dim + d0) = packed;
+    if (rotary.write && head >= rotary.heads) {
+      const int64_t slot = rotary.slots[r];
+      const int64_t page = slot / rotary.block_size;
+      const int offset = static_cast<int>(slot % rotary.block_size);
+      if (turns) {
+        const int kv_head = head - rotary.heads;
+        *reinterpret_cast<uint2*>(rotary.k_cache + ((page * rotary.kv_heads + kv_head) * rotary.block_size + offset) * dim + d0) =
+            packed;
+      } else {
+        const int kv_head = head - rotary.heads - rotary.kv_heads;
+        bf16_t* at = rotary.v_cache + ((page * rotary.kv_heads + kv_head) * dim + d0) * rotary.block_size + offset;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) at[static_cast<int64_t>(i) * rotary.block_size] = static_cast<bf16_t>(v[i]);
       }
     }
   } else {
@@ -379,6 +467,12 @@ __global__ __launch_bounds__(64) void gemm_packed_kernel(const bf16_t* __restric
   }
 }
 
+// Waves of a workgroup for a product that is not cut into slices: each should still own a few k-steps.
+static int packed_waves(int K) {
+  const int steps = K / SK_KSTEP;
+  return steps >= 24 ? 8 : steps >= 8 ? 4 : steps >= 4 ? 2 : 1;
+}
+
 // y: as distie_gemm_skinny_bf16 (the same cut along K); gated: [M, N / 2] of y_dtype.
 extern "C" int distie_gemm_packed_bf16(const void* x, const void* w_packed, const float* bias, void* y, int y_dtype,
                                        int M, int N, int K, int gated, hipStream_t stream) {
@@ -391,12 +485,44 @@ extern "C" int distie_gemm_packed_bf16(const void* x, const void* w_packed, cons
   dim3 grid(row_blocks, slices);
   const bf16_t* xb = static_cast<const bf16_t*>(x);
   const bf16_t* wb = static_cast<const bf16_t*>(w_packed);
+  const RotaryOut none = {};
   if (gated) {
-    DISTIE_DISPATCH(y_dtype, Y, (gemm_packed_kernel<Y, true><<<grid, 64, 0, stream>>>(
-                                    xb, wb, bias, static_cast<Y*>(y), M, N, K, k_per_slice / 32)));
+    DISTIE_DISPATCH(y_dtype, Y, (gemm_packed_kernel<Y, PK_GATED, 1><<<grid, 64, 0, stream>>>(
+                                    xb, wb, bias, static_cast<Y*>(y), M, N, K, k_per_slice / 32, none)));
   } else {
-    DISTIE_DISPATCH(y_dtype, Y, (gemm_packed_kernel<Y, false><<<grid, 64, 0, stream>>>(
-                                    xb, wb, bias, static_cast<Y*>(y), M, N, K, k_per_slice / 32)));
+    DISTIE_DISPATCH(y_dtype, Y, (gemm_packed_kernel<Y, PK_PLAIN, 1><<<grid, 64, 0, stream>>>(
+                                    xb, wb, bias, static_cast<Y*>(y), M, N, K, k_per_slice / 32, none)));
   }
+  return launch_status();
+}
+
+// The stacked q/k/v product with the rotation and the cache write in its epilogue. w_packed: the ROTARY
+// copy of the [(heads + 2 kv_heads) * dim, K] weight. y: bfloat16 [M, N], rotated. dim a multiple of 16;
+// table: [M, dim / 2] (cos, sin).
+extern "C" int distie_gemm_packed_rotary_bf16(const void* x, const void* w_packed, const float* bias, void* y,
+                                              const void* table, const int32_t* slots, void* k_cache, void* v_cache,
+                                              int M, int K, int heads, int kv_heads, int dim, int block_size,
+                                              int write, hipStream_t stream) {
+  if (M <= 0) return 0;
+  if (M > 16 || K <= 0 || K % 8 != 0 || heads < 1 || kv_heads < 1 || dim < 16 || dim % 16 != 0 || block_size < 1 ||
+      table == nullptr || (write && (slots == nullptr || k_cache == nullptr || v_cache == nullptr)))
+    return DISTIE_BAD_ARGUMENT;
+  const int N = (heads + 2 * kv_heads) * dim;
+  const RotaryOut rotary = {static_cast<const float2*>(table), slots, static_cast<bf16_t*>(k_cache),
+                            static_cast<bf16_t*>(v_cache), heads, kv_heads, dim, block_size, write};
+  const bf16_t* xb = static_cast<const bf16_t*>(x);
+  const bf16_t* wb = static_cast<const bf16_t*>(w_packed);
+  bf16_t* out = static_cast<bf16_t*>(y);
+  const int tiles = (K + 31) / 32;
+  dim3 grid(N / 16, 1);
+#define ROTARY(WAVES) \
+  gemm_packed_kernel<bf16_t, PK_ROTARY, WAVES><<<grid, 64 * WAVES, 0, stream>>>(xb, wb, bias, out, M, N, K, tiles, rotary)
+  switch (packed_waves(K)) {
+    case 8: ROTARY(8); break;
+    case 4: ROTARY(4); break;
+    case 2: ROTARY(2); break;
+    default: ROTARY(1); break;
+  }
+#undef ROTARY
   return launch_status();
 }

@@ -97,10 +97,9 @@ class HipOps(Ops):
         o.distie_gemm_generic.argtypes = [_P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _P]
         o.distie_gemm_skinny_slices.argtypes = [_I, _I, _I]
         o.distie_gemm_skinny_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _P]
-        o.distie_packed_elements.argtypes = [_I, _I, _I]
-        o.distie_packed_elements.restype = _L
-        o.distie_pack_weight.argtypes = [_P, _P, _I, _I, _I, _P]
+        o.distie_pack_rows.argtypes = [_P, _P, _P, _I, _I, _P]
         o.distie_gemm_packed_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
+        o.distie_gemm_packed_rotary_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         o.distie_argmax.argtypes = [_P, _P, _I, _I, _P, _P, _P]
         o.distie_argmax_parts.argtypes = [_I, _I]
         o.distie_sample.argtypes = [_P, _P, _P, _P, _P, _I, _I, _P]
@@ -186,18 +185,60 @@ class HipOps(Ops):
                                            _CODES[x.dtype], self._stream()), "sum_slices")
         return out
 
-    def prepare_linear(self, weight, gated=False):
-        name = "_distie_gated" if gated else "_distie_packed"
-        if not self.packed_weights or weight.dtype != torch.bfloat16 or weight.dim() != 2 or \
-                weight.shape[1] % 8 or (gated and weight.shape[0] % 2) or hasattr(weight, name):
+    # ---- packed copies of weights: tiles of 16 rows x 32 k in the matrix cores' lane order
+    @staticmethod
+    def _row_map(N, gated, rotary):
+        """Which row of the weight sits at each place of the packed copy's row blocks (-1: zeros)."""
+        if gated:
+            inter = N // 2
+            j = torch.arange(-(-inter // 8) * 8, dtype=torch.int64).view(-1, 8)
+            gate = torch.where(j < inter, j, -1)
+            up = torch.where(j < inter, j + inter, -1)
+            return torch.cat([gate, up], dim=1).reshape(-1)
+        if rotary is not None:
+            heads, kv_heads, dim = rotary
+            lo = torch.arange(dim // 2, dtype=torch.int64).view(-1, 8)                 # [dim/16, 8]
+            one = torch.cat([lo, lo + dim // 2], dim=1).reshape(-1)                   # rows of a q or k head
+            turned = (torch.arange(heads + kv_heads, dtype=torch.int64)[:, None] * dim + one[None, :]).reshape(-1)
+            return torch.cat([turned, torch.arange((heads + kv_heads) * dim, N, dtype=torch.int64)])
+        rows = torch.full((-(-N // 16) * 16,), -1, dtype=torch.int64)
+        rows[:N] = torch.arange(N)
+        return rows
+
+    @staticmethod
+    def _packed_elements(N, K, gated):
+        row_blocks = -(-(N // 2) // 8) if gated else -(-N // 16)
+        return row_blocks * -(-K // 32) * 512
+
+    def prepare_linear(self, weight, gated=False, rotary=None):
+        if not self.packed_weights or weight.dtype != torch.bfloat16 or weight.dim() != 2 or weight.shape[1] % 8:
+            return
+        N, K = weight.shape
+        name = "_distie_packed"
+        if gated:
+            if N % 2:
+                return
+            name = "_distie_gated"
+        elif rotary is not None:
+            heads, kv_heads, dim = rotary
+            if dim % 16 or N != (heads + 2 * kv_heads) * dim:
+                rotary = None                 # the fused kernel does not take it: the plain copy serves
+            else:
+                name = "_distie_rotary"
+        if hasattr(weight, name):
             return
         self._own(weight)
-        N, K = weight.shape
-        packed = torch.empty(self._ops.distie_packed_elements(N, K, int(gated)), dtype=torch.bfloat16,
-                             device=self.device)
-        _check(self._ops.distie_pack_weight(weight.data_ptr(), packed.data_ptr(), N, K, int(gated), self._stream()),
-               "pack_weight")
-        setattr(weight, name, packed)      # lives and dies with the weight
+        row_map = self._row_map(N, gated, rotary)
+        if row_map.numel() % 16 or int(row_map.max()) >= N or int(row_map.min()) < -1 or \
+                row_map.numel() // 16 * -(-K // 32) * 512 != self._packed_elements(N, K, gated):
+            raise KernelError("prepare_linear: bad row map")
+        row_map = row_map.to(device=self.device, dtype=torch.int32)
+        packed = torch.empty(self._packed_elements(N, K, gated), dtype=torch.bfloat16, device=self.device)
+        _check(self._ops.distie_pack_rows(weight.data_ptr(), packed.data_ptr(), row_map.data_ptr(),
+                                          row_map.numel() // 16, K, self._stream()), "pack_rows")
+        torch.cuda.current_stream(self.device).synchronize()      # row_map is freed on return
+        # the copy lives and dies with the weight
+        setattr(weight, name, (packed, tuple(rotary)) if name == "_distie_rotary" else packed)
 
     def linear_silu_mul(self, x, gate_up_weight):
         packed = getattr(gate_up_weight, "_distie_gated", None)
@@ -209,12 +250,57 @@ class HipOps(Ops):
         N = gate_up_weight.shape[0]
         if gate_up_weight.shape[1] != K:
             raise KernelError(f"linear: x is [{M}, {K}], weight is {list(gate_up_weight.shape)}")
-        if packed.numel() != self._ops.distie_packed_elements(N, K, 1):
+        if packed.numel() != self._packed_elements(N, K, True):
             raise KernelError("linear_silu_mul: the packed copy does not belong to this weight")
         out = torch.empty((M, N // 2), dtype=x.dtype, device=self.device)
         _check(self._ops.distie_gemm_packed_bf16(x.data_ptr(), packed.data_ptr(), None, out.data_ptr(), _code(out),
                                                  M, N, K, 1, self._stream()), "gemm_packed_bf16")
         return out
+
+    def linear_rope_kv_write(self, x, weight, bias, meta, group, k_cache, v_cache, inv_freq, num_heads, num_kv_heads,
+                             head_dim, write):
+        held = getattr(weight, "_distie_rotary", None)
+        x = self.dense(x)
+        fused = held is not None and held[1] == (num_heads, num_kv_heads, head_dim) and \
+            x.dtype == torch.bfloat16 and x.shape[0] <= self.SKINNY_MAX_ROWS and \
+            inv_freq is not None and 2 * inv_freq.shape[0] == head_dim and k_cache.dtype == torch.bfloat16
+        if not fused:
+            return self.rope_kv_write(self.linear(x, weight, bias), meta, group, k_cache, v_cache, inv_freq,
+                                      num_heads, num_kv_heads, head_dim, write)
+        packed = held[0]
+        slots = meta.groups[group].slots
+        self._own(x, bias, k_cache, v_cache, inv_freq, slots)
+        M, K = x.shape
+        N = weight.shape[0]
+        if weight.shape[1] != K or N != (num_heads + 2 * num_kv_heads) * head_dim:
+            raise KernelError(f"linear: x is [{M}, {K}], weight is {list(weight.shape)}")
+        if bias is not None and (bias.dtype != torch.float32 or bias.shape[0] != N):
+            raise KernelError("linear: bias must be float32 [N]")
+        if packed.numel() != self._packed_elements(N, K, False):
+            raise KernelError("linear_rope_kv_write: the packed copy does not belong to this weight")
+        self._check_cache(k_cache, v_cache, num_kv_heads, meta.block_size, head_dim)
+        if M != meta.num_tokens or slots.shape[0] != M:
+            raise KernelError("linear_rope_kv_write: rows do not match the batch")
+        table = self._rope_table(meta, inv_freq)
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=self.device)
+        _check(self._ops.distie_gemm_packed_rotary_bf16(
+            x.data_ptr(), packed.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(),
+            table.data_ptr(), slots.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), M, K, num_heads,
+            num_kv_heads, head_dim, meta.block_size, 1 if write else 0, self._stream()), "gemm_packed_rotary_bf16")
+        return out
+
+    def _rope_table(self, meta, inv_freq):
+        """Cosines and sines of the step's positions, float32 [T, pairs, 2]: computed by the first layer
+        that asks, used by all."""
+        pairs = inv_freq.shape[0]
+        key = ("rope", inv_freq.data_ptr(), pairs)
+        table = meta.scratch.get(key)
+        if table is None:
+            table = torch.empty((meta.num_tokens, pairs, 2), dtype=torch.float32, device=self.device)
+            _check(self._ops.distie_rope_table(meta.positions.data_ptr(), inv_freq.data_ptr(), table.data_ptr(),
+                                               meta.num_tokens, pairs, self._stream()), "rope_table")
+            meta.scratch[key] = table
+        return table
 
     def _linear(self, x, weight, bias, out_dtype, partial_ok=False):
         x = self.dense(x)
@@ -234,7 +320,7 @@ class HipOps(Ops):
                 out = torch.empty((slices, M, N), dtype=torch.float32, device=self.device)
             packed = getattr(weight, "_distie_packed", None)
             if packed is not None:
-                if packed.numel() != self._ops.distie_packed_elements(N, K, 0):
+                if packed.numel() != self._packed_elements(N, K, False):
                     raise KernelError("linear: the packed copy does not belong to this weight")
                 _check(self._ops.distie_gemm_packed_bf16(
                     x.data_ptr(), packed.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(),
@@ -289,16 +375,7 @@ class HipOps(Ops):
             raise KernelError("rope_kv_write: qkv rows do not match the batch")
         pairs = 0 if inv_freq is None else inv_freq.shape[0]
         slots = meta.groups[group].slots
-        table = None
-        if pairs:
-            # cosines and sines of the step's positions: computed by the first layer that asks, used by all
-            key = ("rope", inv_freq.data_ptr(), pairs)
-            table = meta.scratch.get(key)
-            if table is None:
-                table = torch.empty((T, pairs, 2), dtype=torch.float32, device=self.device)
-                _check(self._ops.distie_rope_table(meta.positions.data_ptr(), inv_freq.data_ptr(), table.data_ptr(),
-                                                   T, pairs, self._stream()), "rope_table")
-                meta.scratch[key] = table
+        table = self._rope_table(meta, inv_freq) if pairs else None
         _check(self._ops.distie_rope_kv_write(
             source.data_ptr(), _code(source), slices, out.data_ptr(), _code(out),
             table.data_ptr() if table is not None else None, meta.positions.data_ptr(),

@@ -77,10 +77,21 @@ class Ops(abc.ABC):
         read (the HIP kernels return partial sums over slices of K for small batches); parts
         hand the result on to those operations and do nothing else with it."""
 
-    def prepare_linear(self, weight: torch.Tensor, gated: bool = False) -> None:
+    def prepare_linear(self, weight: torch.Tensor, gated: bool = False, rotary=None) -> None:
         """Called once for every weight of a `linear` after it is loaded (`gated`: the weight of a
-        `linear_silu_mul`). An implementation may build what its products need beside the tensor
-        (the HIP kernels keep a second copy in the matrix cores' order for small batches)."""
+        `linear_silu_mul`; `rotary = (num_heads, num_kv_heads, head_dim)`: the stacked q/k/v weight
+        of a `linear_rope_kv_write`). An implementation may build what its products need beside
+        the tensor (the HIP kernels keep a second copy in the matrix cores' order for small
+        batches)."""
+
+    def linear_rope_kv_write(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                             meta: BatchMeta, group: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                             inv_freq: Optional[torch.Tensor], num_heads: int, num_kv_heads: int,
+                             head_dim: int, write: bool) -> torch.Tensor:
+        """rope_kv_write(linear(x, weight, bias), ...) for the stacked q/k/v weight; an
+        implementation may fuse the two."""
+        return self.rope_kv_write(self.linear(x, weight, bias), meta, group, k_cache, v_cache, inv_freq,
+                                  num_heads, num_kv_heads, head_dim, write)
 
     def linear_silu_mul(self, x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
         """silu_mul(linear(x, gate_up_weight)) with gate_up_weight [2I, K] -> act [T, I]; an

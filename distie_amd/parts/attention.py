@@ -66,13 +66,13 @@ class Attention(Mixer):
         self.position.to_device(self.out_weight.device)
 
     def prepare(self, ops) -> None:
-        ops.prepare_linear(self.qkv_weight)
+        ops.prepare_linear(self.qkv_weight, rotary=(self.num_heads, self.num_kv_heads, self.head_dim))
         ops.prepare_linear(self.out_weight)
 
     def forward(self, ops, x, ctx, cache, writes_cache: bool):
-        qkv = ops.linear(x, self.qkv_weight, self.qkv_bias_t)
-        qkv = ops.rope_kv_write(qkv, ctx.meta, cache.group, cache.k, cache.v, self.position.rotary(),
-                                self.num_heads, self.num_kv_heads, self.head_dim, writes_cache)
+        qkv = ops.linear_rope_kv_write(x, self.qkv_weight, self.qkv_bias_t, ctx.meta, cache.group, cache.k, cache.v,
+                                       self.position.rotary(), self.num_heads, self.num_kv_heads, self.head_dim,
+                                       writes_cache)
         mixed = ops.paged_attention(qkv, ctx.meta, cache.group, cache.k, cache.v, self.num_heads,
                                     self.num_kv_heads, self.head_dim, self.scale, self.window)
         return ops.linear(mixed, self.out_weight, self.out_bias_t)

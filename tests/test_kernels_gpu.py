@@ -138,6 +138,56 @@ def test_linear_silu_mul_fused(ops, M, I, K):
     close(ops.linear_silu_mul(big, w), want, torch.bfloat16, scale=2 * want.abs().max().item())
 
 
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("heads,kv_heads,dim,K,P", [(3, 1, 32, 2048, 4), (12, 2, 128, 1536, 16), (4, 4, 16, 72, 16),
+                                                    (5, 5, 48, 240, 8), (2, 1, 80, 520, 16), (7, 1, 256, 136, 32)])
+@pytest.mark.parametrize("with_bias,write", [(True, True), (False, True), (True, False)])
+def test_linear_rope_kv_write_fused(ops, M, heads, kv_heads, dim, K, P, with_bias, write):
+    """The q/k/v product with rotation and cache write in its epilogue, against product, rotation
+    and write one after the other in plain torch."""
+    N = (heads + 2 * kv_heads) * dim
+    x = rand(M, K, dtype=torch.bfloat16, seed=1)
+    w = rand(N, K, dtype=torch.bfloat16, seed=6, scale=1.0 / K ** 0.5)
+    b = rand(N, seed=7) if with_bias else None
+    pages = 2 * M + 2
+    g = torch.Generator().manual_seed(M * 131 + dim)
+    slots = torch.randperm(pages * P, generator=g)[:M].tolist()
+    positions = torch.randint(0, 5000, (M,), generator=g).tolist()
+    meta = make_meta(positions, list(range(M)), list(range(M + 1)), [p + 1 for p in positions],
+                     [[0] * 8] * M, slots, P)
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, dim, 2, dtype=torch.float32) / dim))).cuda()
+    k1 = rand(pages, kv_heads, P, dim, dtype=torch.bfloat16, seed=8)
+    v1 = rand(pages, kv_heads, dim, P, dtype=torch.bfloat16, seed=9)
+    k2, v2 = k1.clone(), v1.clone()
+    dense = x.double() @ w.double().T + (b.double() if with_bias else 0.0)
+    want = TorchOps("cuda").rope_kv_write(dense.float().clone(), meta, 0, k2, v2, inv_freq, heads, kv_heads, dim, write)
+    ops.prepare_linear(w, rotary=(heads, kv_heads, dim))
+    assert hasattr(w, "_distie_rotary")
+    got = ops.linear_rope_kv_write(x, w, b, meta, 0, k1, v1, inv_freq, heads, kv_heads, dim, write)
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (M, N)
+    scale = want.abs().max().item()
+    close(got, want, torch.bfloat16, scale=scale)
+    # the cache: the new tokens' places hold what the result holds, every other place is untouched
+    close(k1, k2, torch.bfloat16, scale=scale)
+    close(v1, v2, torch.bfloat16, scale=scale)
+    untouched = torch.ones(pages * P, dtype=torch.bool)
+    if write:
+        untouched[slots] = False
+    keep = untouched.view(pages, P).cuda()
+    assert torch.equal(k1.permute(0, 2, 1, 3)[keep], k2.permute(0, 2, 1, 3)[keep])
+    assert torch.equal(v1.permute(0, 3, 1, 2)[keep], v2.permute(0, 3, 1, 2)[keep])
+    if write:
+        view = got.view(M, heads + 2 * kv_heads, dim)
+        at = torch.tensor(slots).cuda()
+        assert torch.equal(k1[at // P, :, at % P], view[:, heads:heads + kv_heads])
+        assert torch.equal(v1[at // P, :, :, at % P], view[:, heads + kv_heads:])
+    # unfused (no packed copy), the same within rounding
+    w2 = w.clone()
+    k3, v3 = k2.clone(), v2.clone()
+    unfused = ops.linear_rope_kv_write(x, w2, b, meta, 0, k3, v3, inv_freq, heads, kv_heads, dim, write)
+    close(unfused, want, torch.bfloat16, scale=2 * scale)
+
+
 def test_partial_sums_are_added_by_their_readers(ops):
     """A product over a long K comes back as slices; norm, activation and rotation add them."""
     from distie_amd.kernels.hip_ops import PartialSums
