@@ -87,9 +87,11 @@ __global__ void rmsnorm_kernel(float* __restrict__ residual, const D* __restrict
 template <typename D, typename W>
 static int rmsnorm_launch_out(float* residual, const D* delta, int slices, const W* weight, void* out,
                               int out_dtype, int rows, int width, float eps, hipStream_t stream) {
-  // with slices to add, a thread's work is a chain of loads: spread a row over more threads
-  int threads = width >= 2048 ? 512 : (width >= 512 ? 256 : 64);
-  if (slices > 1) threads = width >= 1024 ? 1024 : (width >= 512 ? 512 : threads);
+  // a thread's work is a chain of loads: about two elements a thread, so that a row stays in registers
+  // between the two passes
+  int threads = (width / 2 + 63) / 64 * 64;
+  threads = threads < 64 ? 64 : (threads > 1024 ? 1024 : threads);
+  (void)slices;
   DISTIE_DISPATCH(out_dtype, O,
                   rmsnorm_kernel<D, W, O><<<rows, threads, 0, stream>>>(
                       residual, delta, slices, static_cast<int64_t>(rows) * width, weight, static_cast<O*>(out), width, eps));

@@ -326,12 +326,21 @@ __device__ __forceinline__ floatx4 packed_accumulate(const bf16_t* wp, const bf1
     case 1: packed_steps<1>(wp, xp, t_begin, steps, step, acc); break;
     default: break;
   }
-  // the last tiles; the very last may reach beyond K (the copy holds zeros there, x is not read)
-  for (int t = t_begin + 4 * steps; t < t_end; ++t) {
-    const bf16x8 a = *reinterpret_cast<const bf16x8*>(wp + static_cast<int64_t>(t) * PK_TILE);
-    bf16x8 xb = {};
-    if (32 * t + 8 * g < K) xb = *reinterpret_cast<const bf16x8*>(xp + 32 * t);
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, xb, acc, 0, 0, 0);
+  // the last tiles, at most three whole ones and one that reaches beyond K (the copy holds zeros there, x
+  // is not read): loaded together
+  const int t_rest = t_begin + 4 * steps;
+  if (t_rest < t_end) {
+    bf16x8 a[4], xb[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int t = t_rest + j;
+      a[j] = bf16x8{};
+      xb[j] = bf16x8{};
+      if (t < t_end) a[j] = *reinterpret_cast<const bf16x8*>(wp + static_cast<int64_t>(t) * PK_TILE);
+      if (t < t_end && 32 * t + 8 * g < K) xb[j] = *reinterpret_cast<const bf16x8*>(xp + 32 * t);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], xb[j], acc, 0, 0, 0);
   }
   return acc;
 }
@@ -467,13 +476,15 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_packed_kernel(const bf16_t* _
   }
 }
 
-// Waves of a workgroup for a product that is not cut into slices: each should still own a few k-steps.
+// Waves of a workgroup: each should own about four k-steps (one trip to memory).
 static int packed_waves(int K) {
   const int steps = K / SK_KSTEP;
-  return steps >= 24 ? 8 : steps >= 8 ? 4 : steps >= 4 ? 2 : 1;
+  return steps >= 48 ? 16 : steps >= 24 ? 8 : steps >= 8 ? 4 : steps >= 4 ? 2 : 1;
 }
 
-// y: as distie_gemm_skinny_bf16 (the same cut along K); gated: [M, N / 2] of y_dtype.
+// y: as distie_gemm_skinny_bf16 (the same cut along K: slices go to other workgroups, hence to other
+// compute units, which a product with few rows of W needs to pull its bytes fast enough);
+// gated: [M, N / 2] of y_dtype, never cut.
 extern "C" int distie_gemm_packed_bf16(const void* x, const void* w_packed, const float* bias, void* y, int y_dtype,
                                        int M, int N, int K, int gated, hipStream_t stream) {
   if (M <= 0) return 0;
@@ -518,6 +529,7 @@ extern "C" int distie_gemm_packed_rotary_bf16(const void* x, const void* w_packe
 #define ROTARY(WAVES) \
   gemm_packed_kernel<bf16_t, PK_ROTARY, WAVES><<<grid, 64 * WAVES, 0, stream>>>(xb, wb, bias, out, M, N, K, tiles, rotary)
   switch (packed_waves(K)) {
+    case 16: ROTARY(16); break;
     case 8: ROTARY(8); break;
     case 4: ROTARY(4); break;
     case 2: ROTARY(2); break;

@@ -313,15 +313,16 @@ class HipOps(Ops):
             raise KernelError("linear: bias must be float32 [N]")
         both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
         if both_bf16 and M <= self.SKINNY_MAX_ROWS and K % 8 == 0:
-            slices = self._ops.distie_gemm_skinny_slices(M, N, K)
-            if slices == 1:
-                out = torch.empty((M, N), dtype=out_dtype, device=self.device)
-            else:
-                out = torch.empty((slices, M, N), dtype=torch.float32, device=self.device)
             packed = getattr(weight, "_distie_packed", None)
             if packed is not None:
                 if packed.numel() != self._packed_elements(N, K, False):
                     raise KernelError("linear: the packed copy does not belong to this weight")
+            slices = self._ops.distie_gemm_skinny_slices(M, N, K)       # the same cut for both kernels
+            if slices == 1:
+                out = torch.empty((M, N), dtype=out_dtype, device=self.device)
+            else:
+                out = torch.empty((slices, M, N), dtype=torch.float32, device=self.device)
+            if packed is not None:
                 _check(self._ops.distie_gemm_packed_bf16(
                     x.data_ptr(), packed.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(),
                     _code(out), M, N, K, 0, self._stream()), "gemm_packed_bf16")
