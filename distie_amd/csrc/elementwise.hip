@@ -84,17 +84,106 @@ __global__ void rmsnorm_kernel(float* __restrict__ residual, const D* __restrict
   for (int i = threadIdx.x; i < width; i += blockDim.x) y[i] = from_float<O>(x[i] * scale * to_float(weight[i]));
 }
 
+// The same for rows of whole float4s and float32 (or no) delta: a thread owns NV groups of four
+// consecutive elements, every load of the row (residual, all slices, weights) is in flight before the
+// first sum, and nothing is read twice.
+static __device__ __forceinline__ float4 load_weights4(const float* w) { return *reinterpret_cast<const float4*>(w); }
+static __device__ __forceinline__ float4 load_weights4(const bf16_t* w) {
+  const uint2 raw = *reinterpret_cast<const uint2*>(w);
+  return float4{__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u), __uint_as_float(raw.y << 16),
+                __uint_as_float(raw.y & 0xffff0000u)};
+}
+static __device__ __forceinline__ void store4(float* p, const float4& v) { *reinterpret_cast<float4*>(p) = v; }
+static __device__ __forceinline__ void store4(bf16_t* p, const float4& v) {
+  const uint32_t a = __builtin_bit_cast(uint16_t, static_cast<bf16_t>(v.x));
+  const uint32_t b = __builtin_bit_cast(uint16_t, static_cast<bf16_t>(v.y));
+  const uint32_t c = __builtin_bit_cast(uint16_t, static_cast<bf16_t>(v.z));
+  const uint32_t d = __builtin_bit_cast(uint16_t, static_cast<bf16_t>(v.w));
+  *reinterpret_cast<uint2*>(p) = uint2{a | (b << 16), c | (d << 16)};
+}
+
+template <typename W, typename O, int NV>
+__global__ __launch_bounds__(1024) void rmsnorm_vec_kernel(float* __restrict__ residual, const float* __restrict__ delta,
+                                                           int slices, int64_t slice_stride,
+                                                           const W* __restrict__ weight, O* __restrict__ out, int width,
+                                                           float eps) {
+  __shared__ float scratch[16];
+  constexpr int GROUP = 8;                     // slices loaded together
+  const int64_t row = blockIdx.x;
+  const int quads = width / 4;
+  float4 v[NV], wq[NV];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < NV; ++e) {
+    const int q = threadIdx.x + e * blockDim.x;
+    const bool in = q < quads;
+    const int64_t at = row * width + 4 * static_cast<int64_t>(in ? q : 0);
+    const float4 x4 = *reinterpret_cast<const float4*>(residual + at);
+    wq[e] = load_weights4(weight + 4 * (in ? q : 0));
+    float4 sum = {0.f, 0.f, 0.f, 0.f};
+    if (delta != nullptr) {
+      const int last = slices - 1;
+      for (int s0 = 0; s0 < slices; s0 += GROUP) {
+        float4 part[GROUP];
+#pragma unroll
+        for (int u = 0; u < GROUP; ++u)
+          part[u] = *reinterpret_cast<const float4*>(delta + min(s0 + u, last) * slice_stride + at);
+#pragma unroll
+        for (int u = 0; u < GROUP; ++u) {
+          if (s0 + u <= last) {
+            sum.x += part[u].x;
+            sum.y += part[u].y;
+            sum.z += part[u].z;
+            sum.w += part[u].w;
+          }
+        }
+      }
+    }
+    v[e] = float4{x4.x + sum.x, x4.y + sum.y, x4.z + sum.z, x4.w + sum.w};
+    if (!in) v[e] = float4{0.f, 0.f, 0.f, 0.f};
+    if (in && delta != nullptr) *reinterpret_cast<float4*>(residual + at) = v[e];
+    ss += v[e].x * v[e].x + v[e].y * v[e].y + v[e].z * v[e].z + v[e].w * v[e].w;
+  }
+  const float scale = rsqrtf(block_sum(ss, scratch) / static_cast<float>(width) + eps);
+#pragma unroll
+  for (int e = 0; e < NV; ++e) {
+    const int q = threadIdx.x + e * blockDim.x;
+    if (q >= quads) continue;
+    store4(out + row * width + 4 * static_cast<int64_t>(q),
+           float4{v[e].x * scale * wq[e].x, v[e].y * scale * wq[e].y, v[e].z * scale * wq[e].z, v[e].w * scale * wq[e].w});
+  }
+}
+
+static inline bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
 template <typename D, typename W>
 static int rmsnorm_launch_out(float* residual, const D* delta, int slices, const W* weight, void* out,
                               int out_dtype, int rows, int width, float eps, hipStream_t stream) {
+  const int64_t slice_stride = static_cast<int64_t>(rows) * width;
+  if constexpr (sizeof(D) == 4) {
+    if (width % 4 == 0 && width <= 8192 && aligned16(residual) && aligned16(delta) && aligned16(weight) &&
+        aligned16(out)) {
+      const int quads = width / 4;
+      int threads = (quads + 63) / 64 * 64;
+      const int nv = threads > 1024 ? 2 : 1;
+      if (nv == 2) threads = ((quads + 1) / 2 + 63) / 64 * 64;
+      if (nv == 1) {
+        DISTIE_DISPATCH(out_dtype, O, (rmsnorm_vec_kernel<W, O, 1><<<rows, threads, 0, stream>>>(
+                                          residual, delta, slices, slice_stride, weight, static_cast<O*>(out), width, eps)));
+      } else {
+        DISTIE_DISPATCH(out_dtype, O, (rmsnorm_vec_kernel<W, O, 2><<<rows, threads, 0, stream>>>(
+                                          residual, delta, slices, slice_stride, weight, static_cast<O*>(out), width, eps)));
+      }
+      return launch_status();
+    }
+  }
   // a thread's work is a chain of loads: about two elements a thread, so that a row stays in registers
   // between the two passes
   int threads = (width / 2 + 63) / 64 * 64;
   threads = threads < 64 ? 64 : (threads > 1024 ? 1024 : threads);
-  (void)slices;
   DISTIE_DISPATCH(out_dtype, O,
                   rmsnorm_kernel<D, W, O><<<rows, threads, 0, stream>>>(
-                      residual, delta, slices, static_cast<int64_t>(rows) * width, weight, static_cast<O*>(out), width, eps));
+                      residual, delta, slices, slice_stride, weight, static_cast<O*>(out), width, eps));
   return launch_status();
 }
 

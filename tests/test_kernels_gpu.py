@@ -43,7 +43,7 @@ def test_embed(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width", [40, 1000, 3000])
+@pytest.mark.parametrize("width", [40, 1000, 1002, 3000, 5000, 8200])
 def test_rmsnorm_and_fused_add(ops, dtype, width):
     x = rand(7, width, seed=1, scale=3.0)
     w = rand(width, dtype=dtype, seed=2)
@@ -59,6 +59,24 @@ def test_rmsnorm_and_fused_add(ops, dtype, width):
     assert torch.allclose(res.double(), s, atol=1e-6)
     want = s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + eps) * w.double()
     close(got, want, dtype, scale=want.abs().max().item())
+
+
+@pytest.mark.parametrize("width,slices", [(1536, 14), (1536, 4), (96, 9), (4100, 3), (250, 5), (8192, 17)])
+def test_add_rmsnorm_adds_slices_in_order(ops, width, slices):
+    from distie_amd.kernels.hip_ops import PartialSums
+
+    rows = 5
+    res = rand(rows, width, seed=1, scale=2.0)
+    part = rand(slices, rows, width, seed=2)
+    w = rand(width, dtype=torch.bfloat16, seed=3)
+    total = part[0].clone()
+    for s in range(1, slices):
+        total += part[s]                       # float32, in order, as the kernel
+    want_res = res + total
+    want = want_res.double() * torch.rsqrt(want_res.double().pow(2).mean(-1, keepdim=True) + 1e-6) * w.double()
+    got = ops.add_rmsnorm(res, PartialSums(part, torch.bfloat16), w, 1e-6, torch.bfloat16)
+    assert torch.equal(res, want_res)
+    close(got, want, torch.bfloat16, scale=want.abs().max().item())
 
 
 @pytest.mark.parametrize("xd,wd", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
