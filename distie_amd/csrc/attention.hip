@@ -183,7 +183,7 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ kv_len, const int32_t* __restrict__ cu_q,
     const int32_t* __restrict__ block_table, int table_width, float* __restrict__ part_o,
     float* __restrict__ part_ml, int heads, int kv_heads, int block_size, float scale, int window, int split_len,
-    int max_splits) {
+    int max_splits, int dense_rows) {
   const int lane = threadIdx.x;
   const int r = lane % 16;
   const int g = lane / 16;
@@ -191,14 +191,21 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
   const float scale_log2 = scale * 1.4426950408889634f;
   const int request = blockIdx.z;
   const int kh = blockIdx.y;
-  const int token = cu_q[request];
-  if (cu_q[request + 1] - token != 1) return;        // a portion of a prompt: the tiled kernel's
+  const int32_t* table = block_table + static_cast<int64_t>(request) * table_width;
+  // The pages of the run's first chunk are asked for before it is known whether the run holds a key at all
+  // (the entry is inside the table either way): one trip to memory less on the way to the keys.
+  const int run_begin = static_cast<int>(blockIdx.x) * split_len;
+  int pages[DC_BLOCKS];
+#pragma unroll
+  for (int b = 0; b < DC_BLOCKS; ++b) pages[b] = table[min((run_begin + 16 * b) / block_size, table_width - 1)];
+  // dense_rows: every request brings one token, so request i's token is row i
+  const int token = dense_rows ? request : cu_q[request];
+  if (!dense_rows && cu_q[request + 1] - token != 1) return;        // a portion of a prompt: the tiled kernel's
   const int q_pos = kv_len[request] - 1;              // the new token is the last one cached
   const int first = window > 0 ? max(0, q_pos - window + 1) : 0;
-  const int key_begin = max(first, static_cast<int>(blockIdx.x) * split_len);
-  const int key_end = min(q_pos, static_cast<int>(blockIdx.x + 1) * split_len - 1);
+  const int key_begin = max(first, run_begin);
+  const int key_end = min(q_pos, run_begin + split_len - 1);
   if (key_begin > key_end) return;
-  const int32_t* table = block_table + static_cast<int64_t>(request) * table_width;
 
   // ---- the query of this lane's column (head kh * G + 16 mb + r; columns past the group repeat the last)
   bf16x8 q_reg[MB][DK32 > 0 ? DK32 : 1];
@@ -221,7 +228,7 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
     for (int db = 0; db < DB16; ++db) o_acc[mb][db] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int chunk = key_begin / DC_KEYS * DC_KEYS; chunk <= key_end; chunk += DC_KEYS) {
+  for (int chunk = run_begin; chunk <= key_end; chunk += DC_KEYS) {       // split_len is a multiple of DC_KEYS
     // ---- every load of the chunk first
     bool live[DC_BLOCKS];
     bf16x8 k_reg[DC_BLOCKS][DK32 > 0 ? DK32 : 1];
@@ -237,7 +244,7 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
 #pragma unroll
       for (int db = 0; db < DB16; ++db) v_reg[b][db] = uint2{0u, 0u};
       if (!live[b]) continue;
-      const int page = table[key0 / block_size];
+      const int page = pages[b];
       const int64_t page_base = (static_cast<int64_t>(page) * kv_heads + kh) * block_size * D;
       const int offset = key0 % block_size;
       const bf16_t* k_row = k_cache + page_base + static_cast<int64_t>(offset + r) * D;
@@ -255,6 +262,12 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
         const uint2 raw = *reinterpret_cast<const uint2*>(v_col + static_cast<int64_t>(16 * db + r) * block_size);
         v_reg[b][db] = uint2{raw.x & keep_lo, raw.y & keep_hi};
       }
+    }
+    // the next chunk's pages, while this chunk's keys and values are on their way
+    if (chunk + DC_KEYS <= key_end) {
+#pragma unroll
+      for (int b = 0; b < DC_BLOCKS; ++b)
+        pages[b] = table[min((chunk + DC_KEYS + 16 * b) / block_size, table_width - 1)];
     }
     // ---- scores
     floatx4 s[MB][DC_BLOCKS];
@@ -361,16 +374,23 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
 
 // Combines the partial results of the runs of keys of one (request, head): grid (heads, requests), four waves.
 // All threads first find the maximum and the weight of every run; then each wave adds a quarter of the runs
-// (in order, four loads in flight at a time) for the output dims its lanes own, and the four sums are added
-// in order through LDS.
+// (in order) for the output dims its lanes own, and the four sums are added in order through LDS.
+// FAST (at most RD_FAST_RUNS runs fit the buffers): every partial result the block may need is asked for at
+// once, before the request's length says which runs exist (their places are inside the buffers either way,
+// and what a run that does not exist left there is dropped by a select, never multiplied): one trip to
+// memory instead of three.
 constexpr int RD_WAVES = 4;
 constexpr int RD_THREADS = RD_WAVES * DISTIE_WAVE;
 constexpr int RD_MAX_RUNS = 1024;
+constexpr int RD_FAST_PER_WAVE = 16;
+constexpr int RD_FAST_RUNS = RD_FAST_PER_WAVE * RD_WAVES;
 
+template <bool FAST>
 __global__ __launch_bounds__(RD_THREADS) void attn_reduce_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int32_t* __restrict__ kv_len,
-    const int32_t* __restrict__ cu_q, bf16_t* __restrict__ out, int heads, int window, int split_len, int max_splits) {
-  __shared__ float weight_s[RD_MAX_RUNS];
+    const int32_t* __restrict__ cu_q, bf16_t* __restrict__ out, int heads, int window, int split_len, int max_splits,
+    int dense_rows) {
+  __shared__ float weight_s[FAST ? RD_FAST_RUNS : RD_MAX_RUNS];
   __shared__ float sum_s[RD_WAVES][D];
   __shared__ float scratch[32];
   const int tid = threadIdx.x;
@@ -378,13 +398,67 @@ __global__ __launch_bounds__(RD_THREADS) void attn_reduce_kernel(
   const int lane = tid % DISTIE_WAVE;
   const int request = blockIdx.y;
   const int head = blockIdx.x;
-  const int token = cu_q[request];
-  if (cu_q[request + 1] - token != 1) return;
+  const int64_t base0 = (static_cast<int64_t>(request) * heads + head) * max_splits;
+
+  float early[FAST ? RD_FAST_PER_WAVE : 1][DIMS_PER_LANE];
+  float2 early_ml = {0.f, 0.f};
+  if constexpr (FAST) {
+#pragma unroll
+    for (int u = 0; u < RD_FAST_PER_WAVE; ++u) {
+      const int j = min(wave + RD_WAVES * u, max_splits - 1);
+#pragma unroll
+      for (int i = 0; i < DIMS_PER_LANE; ++i) {
+        const int d = lane + i * DISTIE_WAVE;
+        early[u][i] = d < D ? part_o[(base0 + j) * D + d] : 0.f;
+      }
+    }
+    early_ml = *reinterpret_cast<const float2*>(part_ml + 2 * (base0 + min(tid, max_splits - 1)));
+  }
+
+  const int token = dense_rows ? request : cu_q[request];
+  if (!dense_rows && cu_q[request + 1] - token != 1) return;
   const int q_pos = kv_len[request] - 1;
   const int first = window > 0 ? max(0, q_pos - window + 1) : 0;
   const int s_first = first / split_len;
   const int runs = q_pos / split_len - s_first + 1;
-  const int64_t base = (static_cast<int64_t>(request) * heads + head) * max_splits + s_first;
+  const int64_t base = base0 + s_first;
+  bf16_t* o = out + (static_cast<int64_t>(token) * heads + head) * D;
+
+  if constexpr (FAST) {
+    // run j (counted from the buffers' start) exists iff s_first <= j < s_first + runs
+    const bool mine = tid >= s_first && tid < s_first + runs;
+    float m = mine ? early_ml.x : -INFINITY;
+    m = wave_max(m);
+    if (lane == 0) scratch[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3]));
+    const float w = mine ? fast_exp2(early_ml.x - m) : 0.f;
+    if (tid < RD_FAST_RUNS) weight_s[tid] = w;
+    const float l = block_sum(mine ? w * early_ml.y : 0.f, scratch + 16);     // has the barrier that publishes the weights
+#pragma unroll
+    for (int i = 0; i < DIMS_PER_LANE; ++i) {
+      const int d = lane + i * DISTIE_WAVE;
+      if (d >= D) continue;
+      float a = 0.f;
+#pragma unroll
+      for (int u = 0; u < RD_FAST_PER_WAVE; ++u) {
+        const int j = wave + RD_WAVES * u;
+        const bool exists = j >= s_first && j < s_first + runs;
+        a = exists ? fmaf(weight_s[j], early[u][i], a) : a;
+      }
+      sum_s[wave][d] = a;
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    const float inv = 1.f / l;
+#pragma unroll
+    for (int i = 0; i < DIMS_PER_LANE; ++i) {
+      const int d = lane + i * DISTIE_WAVE;
+      if (d < D) o[d] = static_cast<bf16_t>((((sum_s[0][d] + sum_s[1][d]) + sum_s[2][d]) + sum_s[3][d]) * inv);
+    }
+    return;
+  }
+
   // the maximum over all runs (in units of log 2), then every run's weight
   float m = -INFINITY;
   for (int j = tid; j < runs; j += RD_THREADS) m = fmaxf(m, part_ml[2 * (base + j)]);
@@ -419,7 +493,6 @@ __global__ __launch_bounds__(RD_THREADS) void attn_reduce_kernel(
   }
   __syncthreads();
   if (wave != 0) return;
-  bf16_t* o = out + (static_cast<int64_t>(token) * heads + head) * D;
   const float inv = 1.f / l;
 #pragma unroll
   for (int i = 0; i < DIMS_PER_LANE; ++i) {
@@ -440,7 +513,8 @@ extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, c
                                             const int32_t* kv_len, const int32_t* cu_q, const int32_t* block_table,
                                             int table_width, void* out, float* part_o, float* part_ml,
                                             int num_requests, int heads, int kv_heads, int block_size, float scale,
-                                            int window, int split_len, int max_splits, hipStream_t stream) {
+                                            int window, int split_len, int max_splits, int dense_rows,
+                                            hipStream_t stream) {
   if (num_requests <= 0) return 0;
   const int group = kv_heads > 0 ? heads / kv_heads : 0;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size % 16 != 0 || table_width < 1 || window < 0 ||
@@ -454,7 +528,7 @@ extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, c
 #define DECODE_LAUNCH(MB)                                                                                             \
   attn_decode_kernel<MB><<<grid, DISTIE_WAVE, 0, stream>>>(q, q_stride, kc, vc, kv_len, cu_q, block_table, table_width, \
                                                            part_o, part_ml, heads, kv_heads, block_size, scale, window, \
-                                                           split_len, max_splits)
+                                                           split_len, max_splits, dense_rows)
   if (group <= 16) {
     DECODE_LAUNCH(1);
   } else if (group <= 32) {
@@ -465,8 +539,13 @@ extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, c
 #undef DECODE_LAUNCH
   int status = launch_status();
   if (status != 0) return status;
-  attn_reduce_kernel<<<dim3(heads, num_requests), RD_THREADS, 0, stream>>>(
-      part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, split_len, max_splits);
+  if (max_splits <= RD_FAST_RUNS) {
+    attn_reduce_kernel<true><<<dim3(heads, num_requests), RD_THREADS, 0, stream>>>(
+        part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, split_len, max_splits, dense_rows);
+  } else {
+    attn_reduce_kernel<false><<<dim3(heads, num_requests), RD_THREADS, 0, stream>>>(
+        part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, split_len, max_splits, dense_rows);
+  }
   return launch_status();
 }
 

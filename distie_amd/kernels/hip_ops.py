@@ -123,7 +123,7 @@ class HipOps(Ops):
             lib.distie_attention_prefill_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I,
                                                           _F, _I, _I, _P]
             lib.distie_attention_decode_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I,
-                                                         _I, _F, _I, _I, _I, _P]
+                                                         _I, _F, _I, _I, _I, _I, _P]
             if lib.distie_attention_head_dim() != head_dim:
                 raise KernelError("attention library was built for another head size")
             self._attn[head_dim] = lib
@@ -417,7 +417,8 @@ class HipOps(Ops):
                     qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), meta.kv_len.data_ptr(),
                     meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], out.data_ptr(), part_o.data_ptr(),
                     part_ml.data_ptr(), meta.num_requests, num_heads, num_kv_heads, meta.block_size, float(scale),
-                    int(window or 0), split_len, max_splits, self._stream()), "attention_decode_bf16")
+                    int(window or 0), split_len, max_splits, 1 if meta.all_decode else 0, self._stream()),
+                    "attention_decode_bf16")
             if singles < meta.num_requests:
                 # portions of prompts (and single tokens too, if the decode kernel did not take them)
                 _check(lib.distie_attention_prefill_bf16(
