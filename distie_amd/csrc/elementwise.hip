@@ -102,8 +102,8 @@ static __device__ __forceinline__ void store4(bf16_t* p, const float4& v) {
   *reinterpret_cast<uint2*>(p) = uint2{a | (b << 16), c | (d << 16)};
 }
 
-template <typename W, typename O, int NV>
-__global__ __launch_bounds__(1024) void rmsnorm_vec_kernel(float* __restrict__ residual, const float* __restrict__ delta,
+template <typename D, typename W, typename O, int NV>
+__global__ __launch_bounds__(1024) void rmsnorm_vec_kernel(float* __restrict__ residual, const D* __restrict__ delta,
                                                            int slices, int64_t slice_stride,
                                                            const W* __restrict__ weight, O* __restrict__ out, int width,
                                                            float eps) {
@@ -127,7 +127,7 @@ __global__ __launch_bounds__(1024) void rmsnorm_vec_kernel(float* __restrict__ r
         float4 part[GROUP];
 #pragma unroll
         for (int u = 0; u < GROUP; ++u)
-          part[u] = *reinterpret_cast<const float4*>(delta + min(s0 + u, last) * slice_stride + at);
+          part[u] = load_weights4(delta + min(s0 + u, last) * slice_stride + at);
 #pragma unroll
         for (int u = 0; u < GROUP; ++u) {
           if (s0 + u <= last) {
@@ -160,7 +160,7 @@ template <typename D, typename W>
 static int rmsnorm_launch_out(float* residual, const D* delta, int slices, const W* weight, void* out,
                               int out_dtype, int rows, int width, float eps, hipStream_t stream) {
   const int64_t slice_stride = static_cast<int64_t>(rows) * width;
-  if constexpr (sizeof(D) == 4) {
+  {
     if (width % 4 == 0 && width <= 8192 && aligned16(residual) && aligned16(delta) && aligned16(weight) &&
         aligned16(out)) {
       const int quads = width / 4;
@@ -168,10 +168,10 @@ static int rmsnorm_launch_out(float* residual, const D* delta, int slices, const
       const int nv = threads > 1024 ? 2 : 1;
       if (nv == 2) threads = ((quads + 1) / 2 + 63) / 64 * 64;
       if (nv == 1) {
-        DISTIE_DISPATCH(out_dtype, O, (rmsnorm_vec_kernel<W, O, 1><<<rows, threads, 0, stream>>>(
+        DISTIE_DISPATCH(out_dtype, O, (rmsnorm_vec_kernel<D, W, O, 1><<<rows, threads, 0, stream>>>(
                                           residual, delta, slices, slice_stride, weight, static_cast<O*>(out), width, eps)));
       } else {
-        DISTIE_DISPATCH(out_dtype, O, (rmsnorm_vec_kernel<W, O, 2><<<rows, threads, 0, stream>>>(
+        DISTIE_DISPATCH(out_dtype, O, (rmsnorm_vec_kernel<D, W, O, 2><<<rows, threads, 0, stream>>>(
                                           residual, delta, slices, slice_stride, weight, static_cast<O*>(out), width, eps)));
       }
       return launch_status();
@@ -286,6 +286,87 @@ __global__ void rope_kv_write_kernel(const I* in, int slices, int64_t slice_stri
   }
 }
 
+// The same for a finished bfloat16 product (one slice), a bfloat16 cache, the whole head rotated and a head
+// size that is a multiple of 16: a thread turns eight pairs at a time with 16-byte loads and stores.
+static __device__ __forceinline__ void unpack8(const uint4& raw, float v[8]) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    v[2 * e] = __uint_as_float(w[e] << 16);
+    v[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+  }
+}
+static __device__ __forceinline__ uint4 pack8(const float v[8]) {
+  uint32_t w[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    w[e] = static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<bf16_t>(v[2 * e]))) |
+           (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<bf16_t>(v[2 * e + 1]))) << 16);
+  return uint4{w[0], w[1], w[2], w[3]};
+}
+
+__global__ void rope_kv_write_bf16_kernel(const bf16_t* in, bf16_t* out, const float2* __restrict__ table,
+                                          const int32_t* __restrict__ slots, bf16_t* __restrict__ k_cache,
+                                          bf16_t* __restrict__ v_cache, int heads, int kv_heads, int dim,
+                                          int block_size, int write) {
+  const int64_t t = blockIdx.x;
+  const int64_t width = static_cast<int64_t>(heads + 2 * kv_heads) * dim;
+  const bf16_t* src = in + t * width;
+  bf16_t* row = out + t * width;
+  const int64_t slot = write ? slots[t] : 0;
+  const int64_t page = slot / block_size;
+  const int offset = static_cast<int>(slot % block_size);
+  const int half = dim / 2;
+  const int per_head = half / 8;
+  const int rotated_heads = heads + kv_heads;
+  for (int i = threadIdx.x; i < rotated_heads * per_head; i += blockDim.x) {
+    const int head = i / per_head;
+    const int j0 = 8 * (i % per_head);
+    const int64_t lo = static_cast<int64_t>(head) * dim + j0;
+    const uint4 raw0 = *reinterpret_cast<const uint4*>(src + lo);
+    const uint4 raw1 = *reinterpret_cast<const uint4*>(src + lo + half);
+    const float4* angles = reinterpret_cast<const float4*>(table + t * half + j0);      // (cos, sin) x 8
+    float4 cs[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) cs[e] = angles[e];
+    float x0[8], x1[8], a[8], b[8];
+    unpack8(raw0, x0);
+    unpack8(raw1, x1);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      a[2 * e] = x0[2 * e] * cs[e].x - x1[2 * e] * cs[e].y;
+      b[2 * e] = x1[2 * e] * cs[e].x + x0[2 * e] * cs[e].y;
+      a[2 * e + 1] = x0[2 * e + 1] * cs[e].z - x1[2 * e + 1] * cs[e].w;
+      b[2 * e + 1] = x1[2 * e + 1] * cs[e].z + x0[2 * e + 1] * cs[e].w;
+    }
+    const uint4 pa = pack8(a), pb = pack8(b);
+    *reinterpret_cast<uint4*>(row + lo) = pa;
+    *reinterpret_cast<uint4*>(row + lo + half) = pb;
+    if (write && head >= heads) {
+      bf16_t* at = k_cache + ((page * kv_heads + (head - heads)) * block_size + offset) * dim + j0;
+      *reinterpret_cast<uint4*>(at) = pa;
+      *reinterpret_cast<uint4*>(at + half) = pb;
+    }
+  }
+  // v: copied (nothing to do in place), and written into the cache with the key index innermost
+  const int v_items = kv_heads * (dim / 8);
+  for (int i = threadIdx.x; i < v_items; i += blockDim.x) {
+    const int head = i / (dim / 8);
+    const int d0 = 8 * (i % (dim / 8));
+    const int64_t at = static_cast<int64_t>(rotated_heads + head) * dim + d0;
+    const uint4 raw = *reinterpret_cast<const uint4*>(src + at);
+    if (row != src) *reinterpret_cast<uint4*>(row + at) = raw;
+    if (!write) continue;
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+    uint16_t* dst = reinterpret_cast<uint16_t*>(v_cache) + ((page * kv_heads + head) * dim + d0) * block_size + offset;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      dst[static_cast<int64_t>(2 * e) * block_size] = static_cast<uint16_t>(w[e] & 0xffffu);
+      dst[static_cast<int64_t>(2 * e + 1) * block_size] = static_cast<uint16_t>(w[e] >> 16);
+    }
+  }
+}
+
 extern "C" int distie_rope_kv_write(const void* in, int in_dtype, int slices, void* out, int dtype, const void* table,
                                     const int32_t* positions, const int32_t* slots, void* k_cache, void* v_cache,
                                     int cache_dtype, const float* inv_freq, int pairs, int tokens, int heads,
@@ -295,6 +376,17 @@ extern "C" int distie_rope_kv_write(const void* in, int in_dtype, int slices, vo
     return DISTIE_BAD_ARGUMENT;
   if (pairs > 0 && inv_freq == nullptr) return DISTIE_BAD_ARGUMENT;
   if (in == out && (slices != 1 || in_dtype != dtype)) return DISTIE_BAD_ARGUMENT;
+  if (slices == 1 && in_dtype == DISTIE_BF16 && dtype == DISTIE_BF16 && cache_dtype == DISTIE_BF16 && dim % 16 == 0 &&
+      2 * pairs == dim && table != nullptr && reinterpret_cast<uintptr_t>(in) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(out) % 16 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(table) % 16 == 0) {
+    const int items = (heads + kv_heads) * (dim / 16) + kv_heads * (dim / 8);
+    const int threads = items >= 256 ? 256 : (items >= 128 ? 128 : 64);
+    rope_kv_write_bf16_kernel<<<tokens, threads, 0, stream>>>(
+        static_cast<const bf16_t*>(in), static_cast<bf16_t*>(out), static_cast<const float2*>(table), slots,
+        static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), heads, kv_heads, dim, block_size, write);
+    return launch_status();
+  }
   const int work = (heads + kv_heads) * dim / 2;
   int threads = work >= 512 ? 256 : (work >= 128 ? 128 : 64);
   if (slices > 1 && work >= 512) threads = work >= 1024 ? 1024 : 512;

@@ -507,6 +507,249 @@ extern "C" int distie_gemm_packed_bf16(const void* x, const void* w_packed, cons
   return launch_status();
 }
 
+// ---------------------------------------------------------------- packed weights, 17 to 64 rows of x
+// A workgroup of four waves owns four row blocks (one a wave) and one slice of K. Per k-step of 128 the
+// weights go straight into registers, four k-steps ahead; the x tile ([16 MB rows, 128 k], the same for
+// all four waves) is fetched four k-steps ahead as well, into registers, and put into LDS (two stages)
+// right before it is used, so that x is read from the L2 once per workgroup and not once per wave.
+// Epilogues as in gemm_packed_kernel, for every block of 16 rows of x.
+constexpr int WD_STAGES = 4;
+constexpr int WD_XROW = SK_KSTEP + 8;          // elements of an x row in LDS: 16 bytes of padding against bank conflicts
+
+template <typename Y, int MODE, int MB>
+__global__ __launch_bounds__(256, 2) void gemm_packed_wide_kernel(const bf16_t* __restrict__ x,
+                                                               const bf16_t* __restrict__ w,
+                                                               const float* __restrict__ bias, Y* __restrict__ y,
+                                                               int M, int N, int K, int row_blocks, int tiles_per_slice,
+                                                               RotaryOut rotary) {
+  __shared__ __attribute__((aligned(16))) bf16_t xs[2][MB * 16][WD_XROW];
+  const int tid = threadIdx.x;
+  const int lane = tid % 64;
+  const int wave = tid / 64;
+  const int r = lane % 16;
+  const int g = lane / 16;
+  const int k_tiles = (K + 31) / 32;
+  const int s_begin = blockIdx.y * tiles_per_slice;
+  const int s_end = min(k_tiles, s_begin + tiles_per_slice);
+  const int steps = (s_end - s_begin + 3) / 4;
+  const int block = blockIdx.x * 4 + wave;
+  const bool active = block < row_blocks;                       // a wave without a row block still carries x
+  const bf16_t* wp = w + static_cast<int64_t>(min(block, row_blocks - 1)) * k_tiles * PK_TILE + lane * 8;
+  // this thread's part of an x tile: rows 16 p + tid / 16 (p < MB), k 8 (tid % 16) .. + 7 of the step
+  const int x_row = tid / 16;
+  const int x_chunk = tid % 16;
+  const bf16_t* xsrc[MB];
+#pragma unroll
+  for (int p = 0; p < MB; ++p) xsrc[p] = x + static_cast<int64_t>(min(16 * p + x_row, M - 1)) * K;
+
+  bf16x8 a[WD_STAGES][4];
+  uint4 xr[WD_STAGES][MB];
+  floatx4 acc[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) acc[b] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // Loads are unconditional and nothing touches their results before the k-step that uses them: a load
+  // under a branch, or a select right behind it, would make the wave wait for every load in flight.
+  // Addresses are clamped into the buffers instead. A weight tile past the slice's end is read from the
+  // slice's last tile (the same rows, so whatever it holds reaches no output it would not reach anyway) and
+  // meets zeros in x: x past the slice or past K is replaced by zeros when it is put into LDS.
+  auto x_inside = [&](int step) {
+    const int t0 = s_begin + 4 * step;
+    return 32 * t0 + 8 * x_chunk < K && t0 + x_chunk / 4 < s_end;
+  };
+  auto fetch = [&](int step, int slot) {
+    const int t0 = s_begin + 4 * step;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      a[slot][j] = *reinterpret_cast<const bf16x8*>(wp + static_cast<int64_t>(min(t0 + j, s_end - 1)) * PK_TILE);
+    const int k = x_inside(step) ? 32 * t0 + 8 * x_chunk : 0;
+#pragma unroll
+    for (int p = 0; p < MB; ++p) xr[slot][p] = *reinterpret_cast<const uint4*>(xsrc[p] + k);
+  };
+
+#pragma unroll
+  for (int slot = 0; slot < WD_STAGES; ++slot)
+    if (slot < steps) fetch(slot, slot);
+
+  // One k-step: x of this step into LDS, barrier, products. Stage `slot % 2` was last read two k-steps ago;
+  // every wave has passed the barrier of the k-step in between, so all of them are done with it.
+  auto k_step = [&](int step, int slot) {
+    const int stage = slot % 2;
+    const bool inside = x_inside(step);
+#pragma unroll
+    for (int p = 0; p < MB; ++p)
+      *reinterpret_cast<uint4*>(&xs[stage][16 * p + x_row][8 * x_chunk]) = inside ? xr[slot][p] : uint4{0u, 0u, 0u, 0u};
+    __syncthreads();
+    if (active) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+          const bf16x8 xb = *reinterpret_cast<const bf16x8*>(&xs[stage][16 * b + r][32 * j + 8 * g]);
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[slot][j], xb, acc[b], 0, 0, 0);
+        }
+    }
+  };
+  int s = 0;
+  // the steady state has no branch between the loads and their use, so the waits the compiler places let
+  // the loads of the three k-steps ahead stay in flight
+  for (; s + 2 * WD_STAGES <= steps; s += WD_STAGES) {
+#pragma unroll
+    for (int slot = 0; slot < WD_STAGES; ++slot) {
+      k_step(s + slot, slot);
+      fetch(s + slot + WD_STAGES, slot);
+    }
+  }
+  for (; s < steps; s += WD_STAGES) {
+#pragma unroll
+    for (int slot = 0; slot < WD_STAGES; ++slot) {
+      if (s + slot >= steps) break;
+      k_step(s + slot, slot);
+      if (s + slot + WD_STAGES < steps) fetch(s + slot + WD_STAGES, slot);
+    }
+  }
+  if (!active) return;
+
+  // acc[b][i] = sum for row 4 g + i of the block and x row 16 b + r
+#pragma unroll
+  for (int b = 0; b < MB; ++b) {
+    const int m = 16 * b + r;
+    if constexpr (MODE == PK_GATED) {
+      const int half = N / 2;
+      float up[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) up[i] = __shfl_xor(acc[b][i], 32, 64);
+      if (g < 2 && m < M) {
+        float v[4];
+        const int64_t n0 = static_cast<int64_t>(block) * 8 + 4 * g;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float gate = acc[b][i], u = up[i];
+          if (bias != nullptr && n0 + i < half) { gate += bias[n0 + i]; u += bias[half + n0 + i]; }
+          v[i] = gate / (1.f + expf(-gate)) * u;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n0 + i < half) y[static_cast<int64_t>(m) * half + n0 + i] = from_float<Y>(v[i]);
+      }
+    } else if constexpr (MODE == PK_ROTARY) {
+      const int dim = rotary.dim;
+      const int half = dim / 2;
+      const int per_head = dim / 16;
+      const int rotated_blocks = (rotary.heads + rotary.kv_heads) * per_head;
+      const bool turns = block < rotated_blocks;
+      const int head = block / per_head;
+      const int sub = block % per_head;
+      const int d0 = turns ? (g / 2) * half + 8 * sub + 4 * (g % 2) : 16 * sub + 4 * g;
+      float own[4], other[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        own[i] = acc[b][i] + (bias != nullptr ? bias[static_cast<int64_t>(head) * dim + d0 + i] : 0.f);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) other[i] = __shfl_xor(own[i], 32, 64);
+      if (m >= M) continue;
+      float v[4];
+      if (turns) {
+        const float2* angles = rotary.table + static_cast<int64_t>(m) * half + 8 * sub + 4 * (g % 2);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float2 cs = angles[i];
+          v[i] = g < 2 ? own[i] * cs.x - other[i] * cs.y : own[i] * cs.x + other[i] * cs.y;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = own[i];
+      }
+      const uint2 packed = pack_bf16x4(v);
+      *reinterpret_cast<uint2*>(y + static_cast<int64_t>(m) * N + static_cast<int64_t>(head) * dim + d0) = packed;
+      if (rotary.write && head >= rotary.heads) {
+        const int64_t slot = rotary.slots[m];
+        const int64_t page = slot / rotary.block_size;
+        const int offset = static_cast<int>(slot % rotary.block_size);
+        if (turns) {
+          const int kv_head = head - rotary.heads;
+          *reinterpret_cast<uint2*>(rotary.k_cache +
+                                    ((page * rotary.kv_heads + kv_head) * rotary.block_size + offset) * dim + d0) = packed;
+        } else {
+          const int kv_head = head - rotary.heads - rotary.kv_heads;
+          bf16_t* at = rotary.v_cache + ((page * rotary.kv_heads + kv_head) * dim + d0) * rotary.block_size + offset;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) at[static_cast<int64_t>(i) * rotary.block_size] = static_cast<bf16_t>(v[i]);
+        }
+      }
+    } else {
+      Y* out = y + static_cast<int64_t>(blockIdx.y) * M * N;
+      const bool with_bias = bias != nullptr && blockIdx.y == 0;
+      if (m < M) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int64_t n = static_cast<int64_t>(block) * 16 + 4 * g + i;
+          if (n < N) out[static_cast<int64_t>(m) * N + n] = from_float<Y>(acc[b][i] + (with_bias ? bias[n] : 0.f));
+        }
+      }
+    }
+  }
+}
+
+// Slices of K for the wide kernel: enough workgroups for the chip, slices of whole k-steps, at least two
+// k-steps long.
+static void wide_plan(int row_blocks, int K, int* slices, int* tiles_per_slice) {
+  const int groups = (row_blocks + 3) / 4;
+  const int steps = (K + SK_KSTEP - 1) / SK_KSTEP;
+  int want = 1;
+  while (want < 64 && groups * want < 256 && steps / (want * 2) >= 2) want *= 2;
+  int per = (steps + want - 1) / want;
+  *tiles_per_slice = 4 * per;
+  *slices = (steps + per - 1) / per;
+}
+
+extern "C" int distie_gemm_packed_wide_slices(int N, int K) {
+  int slices, per;
+  wide_plan((N + 15) / 16, K, &slices, &per);
+  return slices;
+}
+
+// 17 to 64 rows of x. mode 0: y [M, N] of y_dtype, or float32 [slices, M, N] when the plan cuts K
+// (distie_gemm_packed_wide_slices); 1 (gated): [M, N / 2]; 2 (rotary): as distie_gemm_packed_rotary_bf16.
+static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bias, void* y, int y_dtype, int M, int N,
+                              int K, int mode, const RotaryOut& rotary, hipStream_t stream) {
+  const int row_blocks = mode == PK_GATED ? (N / 2 + 7) / 8 : (N + 15) / 16;
+  int slices = 1, tiles_per_slice = 4 * ((K + SK_KSTEP - 1) / SK_KSTEP);
+  if (mode == PK_PLAIN) wide_plan(row_blocks, K, &slices, &tiles_per_slice);
+  if (slices > 1 && y_dtype != DISTIE_F32) return DISTIE_BAD_ARGUMENT;
+  dim3 grid((row_blocks + 3) / 4, slices);
+  const int mb = (M + 15) / 16;
+#define WIDE(MODE, MB)                                                                                   \
+  DISTIE_DISPATCH(y_dtype, Y, (gemm_packed_wide_kernel<Y, MODE, MB><<<grid, 256, 0, stream>>>(           \
+                                  x, w, bias, static_cast<Y*>(y), M, N, K, row_blocks, tiles_per_slice, rotary)))
+#define WIDE_MB(MODE)                    \
+  switch (mb) {                          \
+    case 1: WIDE(MODE, 1); break;        \
+    case 2: WIDE(MODE, 2); break;        \
+    case 3: WIDE(MODE, 3); break;        \
+    default: WIDE(MODE, 4); break;       \
+  }
+  if (mode == PK_GATED) {
+    WIDE_MB(PK_GATED);
+  } else if (mode == PK_ROTARY) {
+    WIDE_MB(PK_ROTARY);
+  } else {
+    WIDE_MB(PK_PLAIN);
+  }
+#undef WIDE_MB
+#undef WIDE
+  return launch_status();
+}
+
+extern "C" int distie_gemm_packed_wide_bf16(const void* x, const void* w_packed, const float* bias, void* y,
+                                            int y_dtype, int M, int N, int K, int gated, hipStream_t stream) {
+  if (M <= 0) return 0;
+  if (M > 64 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
+  const RotaryOut none = {};
+  return packed_wide_launch(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w_packed), bias, y, y_dtype, M, N,
+                            K, gated ? PK_GATED : PK_PLAIN, none, stream);
+}
+
 // The stacked q/k/v product with the rotation and the cache write in its epilogue. w_packed: the ROTARY
 // copy of the [(heads + 2 kv_heads) * dim, K] weight. y: bfloat16 [M, N], rotated. dim a multiple of 16;
 // table: [M, dim / 2] (cos, sin).
@@ -515,7 +758,7 @@ extern "C" int distie_gemm_packed_rotary_bf16(const void* x, const void* w_packe
                                               int M, int K, int heads, int kv_heads, int dim, int block_size,
                                               int write, hipStream_t stream) {
   if (M <= 0) return 0;
-  if (M > 16 || K <= 0 || K % 8 != 0 || heads < 1 || kv_heads < 1 || dim < 16 || dim % 16 != 0 || block_size < 1 ||
+  if (M > 64 || K <= 0 || K % 8 != 0 || heads < 1 || kv_heads < 1 || dim < 16 || dim % 16 != 0 || block_size < 1 ||
       table == nullptr || (write && (slots == nullptr || k_cache == nullptr || v_cache == nullptr)))
     return DISTIE_BAD_ARGUMENT;
   const int N = (heads + 2 * kv_heads) * dim;
@@ -524,6 +767,7 @@ extern "C" int distie_gemm_packed_rotary_bf16(const void* x, const void* w_packe
   const bf16_t* xb = static_cast<const bf16_t*>(x);
   const bf16_t* wb = static_cast<const bf16_t*>(w_packed);
   bf16_t* out = static_cast<bf16_t*>(y);
+  if (M > 16) return packed_wide_launch(xb, wb, bias, y, DISTIE_BF16, M, N, K, PK_ROTARY, rotary, stream);
   const int tiles = (K + 31) / 32;
   dim3 grid(N / 16, 1);
 #define ROTARY(WAVES) \

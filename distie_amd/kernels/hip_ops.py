@@ -67,6 +67,7 @@ class PartialSums:
 
 class HipOps(Ops):
     SKINNY_MAX_ROWS = 16       # above this the library's tiles are faster than streaming with x from memory
+    PACKED_MAX_ROWS = 64       # ... unless the weight has a packed copy: then up to here x goes through LDS
 
     def __init__(self, device="cuda:0", packed_weights: bool = True) -> None:
         """`packed_weights`: keep a second copy of every bfloat16 weight in the order in which the
@@ -99,6 +100,8 @@ class HipOps(Ops):
         o.distie_gemm_skinny_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _P]
         o.distie_pack_rows.argtypes = [_P, _P, _P, _I, _I, _P]
         o.distie_gemm_packed_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
+        o.distie_gemm_packed_wide_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
+        o.distie_gemm_packed_wide_slices.argtypes = [_I, _I]
         o.distie_gemm_packed_rotary_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         o.distie_argmax.argtypes = [_P, _P, _I, _I, _P, _P, _P]
         o.distie_argmax_parts.argtypes = [_I, _I]
@@ -243,7 +246,7 @@ class HipOps(Ops):
     def linear_silu_mul(self, x, gate_up_weight):
         packed = getattr(gate_up_weight, "_distie_gated", None)
         x = self.dense(x)
-        if packed is None or x.dtype != torch.bfloat16 or x.shape[0] > self.SKINNY_MAX_ROWS:
+        if packed is None or x.dtype != torch.bfloat16 or x.shape[0] > self.PACKED_MAX_ROWS:
             return self.silu_mul(self.linear(x, gate_up_weight))
         self._own(x)
         M, K = x.shape
@@ -253,8 +256,9 @@ class HipOps(Ops):
         if packed.numel() != self._packed_elements(N, K, True):
             raise KernelError("linear_silu_mul: the packed copy does not belong to this weight")
         out = torch.empty((M, N // 2), dtype=x.dtype, device=self.device)
-        _check(self._ops.distie_gemm_packed_bf16(x.data_ptr(), packed.data_ptr(), None, out.data_ptr(), _code(out),
-                                                 M, N, K, 1, self._stream()), "gemm_packed_bf16")
+        kernel = self._ops.distie_gemm_packed_bf16 if M <= self.SKINNY_MAX_ROWS else self._ops.distie_gemm_packed_wide_bf16
+        _check(kernel(x.data_ptr(), packed.data_ptr(), None, out.data_ptr(), _code(out), M, N, K, 1, self._stream()),
+               "gemm_packed_bf16")
         return out
 
     def linear_rope_kv_write(self, x, weight, bias, meta, group, k_cache, v_cache, inv_freq, num_heads, num_kv_heads,
@@ -262,7 +266,7 @@ class HipOps(Ops):
         held = getattr(weight, "_distie_rotary", None)
         x = self.dense(x)
         fused = held is not None and held[1] == (num_heads, num_kv_heads, head_dim) and \
-            x.dtype == torch.bfloat16 and x.shape[0] <= self.SKINNY_MAX_ROWS and \
+            x.dtype == torch.bfloat16 and x.shape[0] <= self.PACKED_MAX_ROWS and \
             inv_freq is not None and 2 * inv_freq.shape[0] == head_dim and k_cache.dtype == torch.bfloat16
         if not fused:
             return self.rope_kv_write(self.linear(x, weight, bias), meta, group, k_cache, v_cache, inv_freq,
@@ -312,8 +316,22 @@ class HipOps(Ops):
         if bias is not None and (bias.dtype != torch.float32 or bias.shape[0] != N):
             raise KernelError("linear: bias must be float32 [N]")
         both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+        packed = getattr(weight, "_distie_packed", None) if both_bf16 else None
+        if packed is not None and self.SKINNY_MAX_ROWS < M <= self.PACKED_MAX_ROWS and K % 8 == 0:
+            if packed.numel() != self._packed_elements(N, K, False):
+                raise KernelError("linear: the packed copy does not belong to this weight")
+            slices = self._ops.distie_gemm_packed_wide_slices(N, K)
+            if slices == 1:
+                out = torch.empty((M, N), dtype=out_dtype, device=self.device)
+            else:
+                out = torch.empty((slices, M, N), dtype=torch.float32, device=self.device)
+            _check(self._ops.distie_gemm_packed_wide_bf16(
+                x.data_ptr(), packed.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(),
+                _code(out), M, N, K, 0, self._stream()), "gemm_packed_wide_bf16")
+            if slices == 1:
+                return out
+            return PartialSums(out, out_dtype) if partial_ok else self.dense(PartialSums(out, out_dtype))
         if both_bf16 and M <= self.SKINNY_MAX_ROWS and K % 8 == 0:
-            packed = getattr(weight, "_distie_packed", None)
             if packed is not None:
                 if packed.numel() != self._packed_elements(N, K, False):
                     raise KernelError("linear: the packed copy does not belong to this weight")
