@@ -106,6 +106,8 @@ def main() -> int:
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     parser.add_argument("--no-points", action="store_true", help="skip batch 1 and batch 64")
+    parser.add_argument("--no-tune", action="store_true",
+                        help="leave the choice of the library's product kernels (prefill) to the library's defaults")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: --gpus {args.gpus} is not supported (this engine has no multi-GPU path)")
@@ -123,7 +125,7 @@ def main() -> int:
     tokens_per_request = CONTEXT + args.warmup + args.steps + 2 * max_batch + 8
     pages = max_batch * -(-tokens_per_request // BLOCK_SIZE) + 8
     llm = LLM(config=shape, random_weights=True, seed=0, dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=pages,
-              max_seqs=max_batch, token_budget=TOKEN_BUDGET, use_graphs=True)
+              max_seqs=max_batch, token_budget=TOKEN_BUDGET, use_graphs=True, tune_products=not args.no_tune)
     vocab = shape["vocab_size"]
     elem = 2 if args.dtype == "bf16" else 4
 
@@ -157,7 +159,7 @@ def main() -> int:
             "intermediate": shape["intermediate_size"], "vocab": vocab, "tied_head": True,
             "global_batch": args.batch, "seq_len": CONTEXT, "context_limit": shape["max_position_embeddings"],
             "block_size": BLOCK_SIZE, "token_budget": TOKEN_BUDGET, "prefill_tokens": PREFILL_TOKENS,
-            "captured_decode": True, "parallelism": "single GPU",
+            "captured_decode": True, "tuned_products": not args.no_tune, "parallelism": "single GPU",
         },
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -106,9 +106,30 @@ class LLM:
             from .graphs import DecodeGraphs
 
             self.runner.graphs = DecodeGraphs(self.runner, ec.max_seqs)
+        if ec.tune_products and hasattr(ops, "tune_library_products"):
+            self._tune_products()
         _log.info("engine ready: %s dtype=%s pages=%d x %d tokens, %d cache groups, %.1f MiB cache",
                   spec.architecture, ec.dtype, ec.pages(), ec.block_size, len(self.cache.groups),
                   self.cache.bytes() / 2 ** 20)
+
+    def _tune_products(self) -> None:
+        """One step with as many tokens as a full portion of a prompt has, while the library is
+        allowed to time its candidate kernels for every product shape it meets; afterwards it
+        uses what it found for these shapes and its defaults for all others."""
+        tokens = min(self.engine_config.token_budget, self.max_model_len,
+                     self.cache.block_size * self.cache.num_blocks)
+        if tokens < 1:
+            return
+        started = time.perf_counter()
+        self.ops.tune_library_products(True)
+        try:
+            ids = [i % self.model.spec.vocab_size for i in range(tokens)]
+            self.step([StepEntry("__tune__", ids, [tokens - 1])])
+            torch.cuda.synchronize()
+        finally:
+            self.finish("__tune__")
+            self.ops.tune_library_products(False)
+        _log.info("library products tuned for portions of %d tokens in %.1f s", tokens, time.perf_counter() - started)
 
     # ------------------------------------------------------------ the step function
     def step(self, entries: Seq[StepEntry]) -> Optional[torch.Tensor]:

@@ -107,6 +107,22 @@ class HipOps(Ops):
         o.distie_argmax_parts.argtypes = [_I, _I]
         o.distie_sample.argtypes = [_P, _P, _P, _P, _P, _I, _I, _P]
 
+    def tune_library_products(self, on: bool) -> None:
+        """While on, the library times its candidate kernels for every new shape of a large product and
+        keeps the fastest; afterwards it uses what it found (its own choice for shapes it has not
+        seen). Products of up to `PACKED_MAX_ROWS` rows do not go to the library at all."""
+        import os
+        import tempfile
+
+        import torch.cuda.tunable as tunable
+
+        if on:
+            # the library insists on a results file: keep it out of the working directory
+            folder = tempfile.mkdtemp(prefix=f"distie_tune_{os.getuid()}_")
+            tunable.set_filename(os.path.join(folder, "results.csv"))
+        tunable.enable(True)
+        tunable.tuning_enable(bool(on))
+
     def graphs_supported(self) -> bool:
         """Every kernel launches on torch's current stream and keeps its scratch at fixed
         addresses, so a step can be captured into a HIP graph."""

@@ -49,6 +49,21 @@ def test_prompt_then_last_32_one_by_one(setup, ops):
     check_logits(replay_cut(runner, "a", ids, [88]), weights, cfg, ids, dtype, folder)
 
 
+def test_without_packed_weights(setup):
+    """The products on the stored layout (no second copy of the weights), rotation and activation as
+    kernels of their own: the same requests, the same bounds."""
+    from distie_amd.kernels.hip_ops import HipOps
+
+    cfg, block, folder, weights, dtype = setup
+    plain_ops = HipOps("cuda:0", packed_weights=False)
+    runner = build_runner(folder, plain_ops, dtype, block_size=block)
+    ids = random_ids(cfg, 120, 2)
+    check_logits(replay_cut(runner, "a", ids, [40, 20, 17, 11]), weights, cfg, ids, dtype, folder)
+    tensors = [t for b in runner.model.blocks for part in (b.mixer, b.feed_forward) for t in vars(part).values()
+               if isinstance(t, torch.Tensor)] + [runner.model.head]
+    assert not any(hasattr(t, name) for t in tensors for name in ("_distie_packed", "_distie_gated", "_distie_rotary"))
+
+
 @pytest.mark.parametrize("cuts", [[2, 3, 5, 7, 2, 11, 4, 33, 2, 2, 19], [64, 2, 2, 2, 30], [1, 1, 2, 70, 9]])
 def test_portions(setup, ops, cuts):
     cfg, block, folder, weights, dtype = setup

@@ -132,3 +132,27 @@ def test_generation_through_the_entry_point_and_the_command_line(tmp_path):
     assert done.returncode == 0, done.stderr
     report = json.loads((tmp_path / "report.json").read_text())
     assert [r["token_ids"] for r in report] == want
+
+
+def test_tuned_library_products(tmp_path):
+    """`tune_products`: the engine starts with one full portion while the library times its kernels for
+    the large products; results stay within the bounds, with whatever kernels it picked."""
+    import torch.cuda.tunable as tunable
+
+    from distie_amd import LLM
+    from distie_amd.engine.batch import StepEntry
+    from engine_util import check_logits
+
+    cfg = plain.TINY_C
+    folder, weights = make_model_dir(tmp_path, cfg, seed=5, dtype=torch.bfloat16)
+    try:
+        llm = LLM(folder, dtype="bf16", block_size=16, num_blocks=40, token_budget=200, tune_products=True)
+        assert tunable.is_enabled() and not tunable.tuning_is_enabled()
+        ids = random_ids(cfg, 150, 4)
+        logits = llm.step([StepEntry("a", ids, list(range(len(ids))))]).float().cpu()
+        llm.finish("a")
+        check_logits(logits, weights, cfg, ids, torch.bfloat16, folder)
+        llm.cache.check()
+    finally:
+        tunable.tuning_enable(False)
+        tunable.enable(False)
