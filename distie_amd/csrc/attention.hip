@@ -228,7 +228,14 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
     for (int db = 0; db < DB16; ++db) o_acc[mb][db] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int chunk = run_begin; chunk <= key_end; chunk += DC_KEYS) {       // split_len is a multiple of DC_KEYS
+  // every chunk of the walk holds at least one visible key (the running maximum is then finite): under a
+  // window the walk starts at the chunk of the first visible key, whose pages are asked for now
+  const int chunk_begin = max(run_begin, key_begin / DC_KEYS * DC_KEYS);      // split_len is a multiple of DC_KEYS
+  if (chunk_begin != run_begin) {
+#pragma unroll
+    for (int b = 0; b < DC_BLOCKS; ++b) pages[b] = table[min((chunk_begin + 16 * b) / block_size, table_width - 1)];
+  }
+  for (int chunk = chunk_begin; chunk <= key_end; chunk += DC_KEYS) {
     // ---- every load of the chunk first
     bool live[DC_BLOCKS];
     bf16x8 k_reg[DC_BLOCKS][DK32 > 0 ? DK32 : 1];
@@ -574,8 +581,9 @@ constexpr int PF_V_PER_THREAD = (PF_V_CHUNKS + PF_THREADS - 1) / PF_THREADS;
 __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_kernel(
     const bf16_t* __restrict__ qkv, int64_t q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ positions, const int32_t* __restrict__ cu_q,
-    const int32_t* __restrict__ block_table, int table_width, bf16_t* __restrict__ out, int num_requests, int heads,
-    int kv_heads, int block_size, float scale, int window, int min_q_len) {
+    const int32_t* __restrict__ block_table, int table_width, bf16_t* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int tokens, int num_requests, int heads, int kv_heads, int block_size, float scale,
+    int window, int min_q_len) {
   __shared__ __attribute__((aligned(16))) bf16_t k_lds[PF_BN * PF_K_STRIDE];
   __shared__ __attribute__((aligned(16))) bf16_t v_lds[D * PF_V_STRIDE];
   const int tid = threadIdx.x;
@@ -816,15 +824,22 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
       }
   };
 
+  // With gridDim.z = 2 the key tiles of these tokens are cut in two halves, one workgroup each, which write
+  // unnormalised partial results that attn_prefill_merge_kernel combines: the last tokens of a long
+  // portion walk over many key tiles one after the other, and this halves the longest walk.
   // PF_DEPTH tiles of loads are in flight (tiles past the last key load the start of the cache and are not used)
-  const int tile0 = key_begin / PF_BN * PF_BN;
+  const int all_tile0 = key_begin / PF_BN * PF_BN;
+  const int all_tiles = (key_end - all_tile0) / PF_BN + 1;
+  const int per_split = (all_tiles + gridDim.z - 1) / gridDim.z;
+  const int tile0 = all_tile0 + static_cast<int>(blockIdx.z) * per_split * PF_BN;
+  const int loop_end = min(key_end, tile0 + per_split * PF_BN - 1);            // last key of this workgroup's walk
 #pragma unroll
   for (int d = 0; d < PF_DEPTH; ++d) fetch(tile0 + d * PF_BN, k_stages[d], v_stages[d]);
-  for (int k0 = tile0; k0 <= key_end; k0 += PF_DEPTH * PF_BN) {
+  for (int k0 = tile0; k0 <= loop_end; k0 += PF_DEPTH * PF_BN) {
 #pragma unroll
     for (int d = 0; d < PF_DEPTH; ++d) {
       const int k = k0 + d * PF_BN;
-      if (k > key_end) break;
+      if (k > loop_end) break;
       __syncthreads();                       // every wave is done with the tile in LDS
       stash(k, k_stages[d], v_stages[d]);
       __syncthreads();
@@ -844,12 +859,57 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
     for (int i = 0; i < 4; ++i) {
       const int col = 16 * mb + 4 * g + i;
       const float l_col = __shfl(l_run[mb], 4 * g + i, DISTIE_WAVE);
+      const float m_col = __shfl(m_run[mb], 4 * g + i, DISTIE_WAVE);
       if (col >= wave_cols) continue;
-      bf16_t* o = out + (static_cast<int64_t>(token0 + wave_col0 + col) * heads + head) * D;
-      const float inv = 1.f / l_col;
+      const int64_t row = static_cast<int64_t>(token0 + wave_col0 + col) * heads + head;
+      if (gridDim.z == 1) {
+        bf16_t* o = out + row * D;
+        const float inv = 1.f / l_col;
 #pragma unroll
-      for (int db = 0; db < DB16; ++db) o[16 * db + r] = static_cast<bf16_t>(o_acc[mb][db][i] * inv);
+        for (int db = 0; db < DB16; ++db) o[16 * db + r] = static_cast<bf16_t>(o_acc[mb][db][i] * inv);
+      } else {
+        // a half without a key for this column leaves l = 0, and the merge does not read its sums
+        const int64_t at = static_cast<int64_t>(blockIdx.z) * tokens * heads + row;
+        float* po = part_o + at * D;
+#pragma unroll
+        for (int db = 0; db < DB16; ++db) po[16 * db + r] = o_acc[mb][db][i];
+        if (r == 0) {
+          part_ml[2 * at] = m_col;
+          part_ml[2 * at + 1] = l_col;
+        }
+      }
     }
+}
+
+// Combines the two halves of attn_prefill_kernel with gridDim.z = 2: one block per token; tokens of requests
+// that the kernel skipped (fewer than min_q_len tokens) are skipped here as well.
+__global__ void attn_prefill_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                          const int32_t* __restrict__ token_request, const int32_t* __restrict__ cu_q,
+                                          bf16_t* __restrict__ out, int tokens, int heads, int min_q_len) {
+  const int64_t token = blockIdx.x;
+  const int request = token_request[token];
+  if (cu_q[request + 1] - cu_q[request] < min_q_len) return;
+  const int64_t half = static_cast<int64_t>(tokens) * heads;
+  for (int i = threadIdx.x; i < heads * (D / 4); i += blockDim.x) {
+    const int head = i / (D / 4);
+    const int d = 4 * (i % (D / 4));
+    const int64_t row = token * heads + head;
+    const float2 ml0 = *reinterpret_cast<const float2*>(part_ml + 2 * row);
+    const float2 ml1 = *reinterpret_cast<const float2*>(part_ml + 2 * (half + row));
+    float4 o0 = {0.f, 0.f, 0.f, 0.f}, o1 = {0.f, 0.f, 0.f, 0.f};
+    if (ml0.y > 0.f) o0 = *reinterpret_cast<const float4*>(part_o + row * D + d);
+    if (ml1.y > 0.f) o1 = *reinterpret_cast<const float4*>(part_o + (half + row) * D + d);
+    const float m = fmaxf(ml0.y > 0.f ? ml0.x : -INFINITY, ml1.y > 0.f ? ml1.x : -INFINITY);
+    const float w0 = ml0.y > 0.f ? fast_exp2(ml0.x - m) : 0.f;
+    const float w1 = ml1.y > 0.f ? fast_exp2(ml1.x - m) : 0.f;
+    const float inv = 1.f / (w0 * ml0.y + w1 * ml1.y);
+    const float v[4] = {(w0 * o0.x + w1 * o1.x) * inv, (w0 * o0.y + w1 * o1.y) * inv, (w0 * o0.z + w1 * o1.z) * inv,
+                        (w0 * o0.w + w1 * o1.w) * inv};
+    uint32_t h[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) h[e] = __builtin_bit_cast(uint16_t, static_cast<bf16_t>(v[e]));
+    *reinterpret_cast<uint2*>(out + row * D + d) = uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+  }
 }
 
 // Portions of prompts (and whole mixed steps). bfloat16 only; block_size must be a multiple of 16. Requests that
@@ -858,16 +918,26 @@ extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, 
                                              const int32_t* positions, const int32_t* cu_q, const int32_t* block_table,
                                              int table_width, void* out, int tokens, int num_requests, int heads,
                                              int kv_heads, int block_size, float scale, int window, int min_q_len,
+                                             const int32_t* token_request, float* part_o, float* part_ml,
                                              hipStream_t stream) {
+  // part_o (float32 [2, tokens, heads, D]) and part_ml (float32 [2, tokens, heads, 2]) given: the keys are walked
+  // in two halves (worth it for long portions); both null: in one.
   if (tokens <= 0) return 0;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size % 16 != 0 || table_width < 1 || window < 0 ||
-      num_requests < 1 || heads > 65535 || min_q_len < 1)
+      num_requests < 1 || heads > 65535 || min_q_len < 1 || (part_o == nullptr) != (part_ml == nullptr) ||
+      (part_o != nullptr && token_request == nullptr))
     return DISTIE_BAD_ARGUMENT;
   const int tiles = (tokens + PF_BM - 1) / PF_BM + num_requests;     // an upper bound; spare blocks leave at once
   if (tiles > 65535) return DISTIE_BAD_ARGUMENT;
-  attn_prefill_kernel<<<dim3(heads, tiles), PF_THREADS, 0, stream>>>(
+  const int splits = part_o != nullptr ? 2 : 1;
+  attn_prefill_kernel<<<dim3(heads, tiles, splits), PF_THREADS, 0, stream>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),
-      positions, cu_q, block_table, table_width, static_cast<bf16_t*>(out), num_requests, heads, kv_heads, block_size,
-      scale, window, min_q_len);
+      positions, cu_q, block_table, table_width, static_cast<bf16_t*>(out), part_o, part_ml, tokens, num_requests, heads,
+      kv_heads, block_size, scale, window, min_q_len);
+  int status = launch_status();
+  if (status != 0 || splits == 1) return status;
+  const int work = heads * (D / 4);
+  attn_prefill_merge_kernel<<<tokens, work >= 512 ? 512 : (work >= 256 ? 256 : 64), 0, stream>>>(
+      part_o, part_ml, token_request, cu_q, static_cast<bf16_t*>(out), tokens, heads, min_q_len);
   return launch_status();
 }

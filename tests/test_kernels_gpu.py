@@ -365,11 +365,35 @@ def test_paged_attention_long_portions(ops, dtype, heads, kv_heads, dim, P, wind
     close(got, want, dtype, scale=want.abs().max().item())
 
 
+@pytest.mark.parametrize("heads,kv_heads,dim,P,window", [(4, 2, 16, 16, None), (12, 2, 128, 16, None), (3, 1, 48, 16, 700),
+                                                         (2, 1, 256, 32, 100), (6, 2, 64, 64, None)])
+def test_paged_attention_keys_walked_in_two_halves(ops, heads, kv_heads, dim, P, window, monkeypatch):
+    """From 1,024 visible keys on, the tiled kernel cuts the walk over the keys in two and merges: a long
+    portion without a past, one that starts in the middle of a tile after a long past, a short one, a
+    two-token one, and single tokens (which the decode kernel takes, or the tiled kernel too)."""
+    dtype = torch.bfloat16
+    lens, q_lens = [1300, 1500, 90, 777, 40, 1100], [1300, 100, 90, 1, 2, 1]
+    meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, lens, q_lens, dtype, seed=5)
+    assert meta.max_kv >= ops.PREFILL_SPLIT_KEYS
+    want = TorchOps("cuda").paged_attention(qkv.double(), meta, 0, k.double(), v.double(), heads, kv_heads, dim,
+                                            dim ** -0.5, window)
+    got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
+    close(got, want, dtype, scale=want.abs().max().item())
+    meta.host_cu_q = None                      # the tiled kernel takes the single tokens too
+    got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
+    close(got, want, dtype, scale=want.abs().max().item())
+    # in one walk, the same within rounding
+    monkeypatch.setattr(type(ops), "PREFILL_SPLIT_KEYS", 1 << 30)
+    whole = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
+    close(whole, want, dtype, scale=want.abs().max().item())
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,kv_heads,dim,P,window", ATTENTION_SHAPES)
 def test_paged_attention_decode_step(ops, dtype, heads, kv_heads, dim, P, window):
-    """Every request brings one token (the split-key kernel in bfloat16), contexts from 1 to 700."""
-    lens = [1, 2, 16, 17, 64, 65, 129, 300, 700]
+    """Every request brings one token (the split-key kernel in bfloat16), contexts from 1 to 1,100 (the last:
+    under a window of 100 its first visible key lies in the second half of a run of 64)."""
+    lens = [1, 2, 16, 17, 64, 65, 129, 300, 700, 1100]
     meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, lens, [1] * len(lens), dtype)
     assert meta.all_decode
     want = TorchOps("cuda").paged_attention(qkv.double(), meta, 0, k.double(), v.double(), heads, kv_heads, dim,
