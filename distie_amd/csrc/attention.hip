@@ -824,7 +824,7 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
       }
   };
 
-  // With gridDim.z = 2 the key tiles of these tokens are cut in two halves, one workgroup each, which write
+  // With gridDim.z > 1 the key tiles of these tokens are cut in that many parts, one workgroup each, which write
   // unnormalised partial results that attn_prefill_merge_kernel combines: the last tokens of a long
   // portion walk over many key tiles one after the other, and this halves the longest walk.
   // PF_DEPTH tiles of loads are in flight (tiles past the last key load the start of the cache and are not used)
@@ -881,30 +881,48 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
     }
 }
 
-// Combines the two halves of attn_prefill_kernel with gridDim.z = 2: one block per token; tokens of requests
-// that the kernel skipped (fewer than min_q_len tokens) are skipped here as well.
+// Combines the `splits` parts of attn_prefill_kernel with gridDim.z > 1, in order: one block per token; tokens
+// of requests that the kernel skipped (fewer than min_q_len tokens) are skipped here as well.
+constexpr int PF_MAX_SPLITS = 8;
+
 __global__ void attn_prefill_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                           const int32_t* __restrict__ token_request, const int32_t* __restrict__ cu_q,
-                                          bf16_t* __restrict__ out, int tokens, int heads, int min_q_len) {
+                                          bf16_t* __restrict__ out, int tokens, int heads, int min_q_len, int splits) {
   const int64_t token = blockIdx.x;
   const int request = token_request[token];
   if (cu_q[request + 1] - cu_q[request] < min_q_len) return;
-  const int64_t half = static_cast<int64_t>(tokens) * heads;
+  const int64_t part = static_cast<int64_t>(tokens) * heads;
   for (int i = threadIdx.x; i < heads * (D / 4); i += blockDim.x) {
     const int head = i / (D / 4);
     const int d = 4 * (i % (D / 4));
     const int64_t row = token * heads + head;
-    const float2 ml0 = *reinterpret_cast<const float2*>(part_ml + 2 * row);
-    const float2 ml1 = *reinterpret_cast<const float2*>(part_ml + 2 * (half + row));
-    float4 o0 = {0.f, 0.f, 0.f, 0.f}, o1 = {0.f, 0.f, 0.f, 0.f};
-    if (ml0.y > 0.f) o0 = *reinterpret_cast<const float4*>(part_o + row * D + d);
-    if (ml1.y > 0.f) o1 = *reinterpret_cast<const float4*>(part_o + (half + row) * D + d);
-    const float m = fmaxf(ml0.y > 0.f ? ml0.x : -INFINITY, ml1.y > 0.f ? ml1.x : -INFINITY);
-    const float w0 = ml0.y > 0.f ? fast_exp2(ml0.x - m) : 0.f;
-    const float w1 = ml1.y > 0.f ? fast_exp2(ml1.x - m) : 0.f;
-    const float inv = 1.f / (w0 * ml0.y + w1 * ml1.y);
-    const float v[4] = {(w0 * o0.x + w1 * o1.x) * inv, (w0 * o0.y + w1 * o1.y) * inv, (w0 * o0.z + w1 * o1.z) * inv,
-                        (w0 * o0.w + w1 * o1.w) * inv};
+    float2 ml[PF_MAX_SPLITS];
+    float4 o[PF_MAX_SPLITS];
+    float m = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < PF_MAX_SPLITS; ++s) {
+      ml[s] = float2{-INFINITY, 0.f};
+      o[s] = float4{0.f, 0.f, 0.f, 0.f};
+      if (s < splits) ml[s] = *reinterpret_cast<const float2*>(part_ml + 2 * (s * part + row));
+      // a part without a key for this token has l = 0; what it left in part_o is not read
+      if (s < splits && ml[s].y > 0.f) {
+        o[s] = *reinterpret_cast<const float4*>(part_o + (s * part + row) * D + d);
+        m = fmaxf(m, ml[s].x);
+      }
+    }
+    float l = 0.f;
+    float4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < PF_MAX_SPLITS; ++s) {
+      const float w = ml[s].y > 0.f ? fast_exp2(ml[s].x - m) : 0.f;
+      l += w * ml[s].y;
+      sum.x += w * o[s].x;
+      sum.y += w * o[s].y;
+      sum.z += w * o[s].z;
+      sum.w += w * o[s].w;
+    }
+    const float inv = 1.f / l;
+    const float v[4] = {sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv};
     uint32_t h[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) h[e] = __builtin_bit_cast(uint16_t, static_cast<bf16_t>(v[e]));
@@ -919,17 +937,16 @@ extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, 
                                              int table_width, void* out, int tokens, int num_requests, int heads,
                                              int kv_heads, int block_size, float scale, int window, int min_q_len,
                                              const int32_t* token_request, float* part_o, float* part_ml,
-                                             hipStream_t stream) {
-  // part_o (float32 [2, tokens, heads, D]) and part_ml (float32 [2, tokens, heads, 2]) given: the keys are walked
-  // in two halves (worth it for long portions); both null: in one.
+                                             int splits, hipStream_t stream) {
+  // splits > 1: the keys are walked in that many parts side by side (worth it for long portions), with
+  // part_o (float32 [splits, tokens, heads, D]) and part_ml (float32 [splits, tokens, heads, 2]) in between.
   if (tokens <= 0) return 0;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size % 16 != 0 || table_width < 1 || window < 0 ||
-      num_requests < 1 || heads > 65535 || min_q_len < 1 || (part_o == nullptr) != (part_ml == nullptr) ||
-      (part_o != nullptr && token_request == nullptr))
+      num_requests < 1 || heads > 65535 || min_q_len < 1 || splits < 1 || splits > PF_MAX_SPLITS ||
+      (splits > 1 && (part_o == nullptr || part_ml == nullptr || token_request == nullptr)))
     return DISTIE_BAD_ARGUMENT;
   const int tiles = (tokens + PF_BM - 1) / PF_BM + num_requests;     // an upper bound; spare blocks leave at once
   if (tiles > 65535) return DISTIE_BAD_ARGUMENT;
-  const int splits = part_o != nullptr ? 2 : 1;
   attn_prefill_kernel<<<dim3(heads, tiles, splits), PF_THREADS, 0, stream>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),
       positions, cu_q, block_table, table_width, static_cast<bf16_t*>(out), part_o, part_ml, tokens, num_requests, heads,
@@ -938,6 +955,6 @@ extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, 
   if (status != 0 || splits == 1) return status;
   const int work = heads * (D / 4);
   attn_prefill_merge_kernel<<<tokens, work >= 512 ? 512 : (work >= 256 ? 256 : 64), 0, stream>>>(
-      part_o, part_ml, token_request, cu_q, static_cast<bf16_t*>(out), tokens, heads, min_q_len);
+      part_o, part_ml, token_request, cu_q, static_cast<bf16_t*>(out), tokens, heads, min_q_len, splits);
   return launch_status();
 }

@@ -67,7 +67,8 @@ class PartialSums:
 
 class HipOps(Ops):
     SKINNY_MAX_ROWS = 16       # above this the library's tiles are faster than streaming with x from memory
-    PREFILL_SPLIT_KEYS = 1024  # portions that see at least this many keys walk over them in two halves
+    PREFILL_SPLIT_KEYS = 1024  # from this many visible keys on, a portion's walk over the keys is cut in two parts
+    PREFILL_MAX_SPLITS = 4     # (three from four times as many, four from six times; measured: 2 beat 3 at 2,048)
     PACKED_MAX_ROWS = 64       # ... unless the weight has a packed copy: then up to here x goes through LDS
 
     def __init__(self, device="cuda:0", packed_weights: bool = True) -> None:
@@ -141,7 +142,7 @@ class HipOps(Ops):
             lib.distie_attention_generic.argtypes = [_P, _I, _L, _P, _P, _I, _P, _P, _P, _I, _P,
                                                      _I, _I, _I, _I, _F, _I, _P]
             lib.distie_attention_prefill_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I,
-                                                          _F, _I, _I, _P, _P, _P, _P]
+                                                          _F, _I, _I, _P, _P, _P, _I, _P]
             lib.distie_attention_decode_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I,
                                                          _I, _F, _I, _I, _I, _I, _P]
             if lib.distie_attention_head_dim() != head_dim:
@@ -456,18 +457,21 @@ class HipOps(Ops):
                     "attention_decode_bf16")
             if singles < meta.num_requests or not split_decode:
                 # portions of prompts (and single tokens too, if the decode kernel did not take them). Long
-                # walks over the keys are cut in two halves that run side by side.
-                halves = meta.max_kv >= self.PREFILL_SPLIT_KEYS
+                # walks over the keys are cut into parts that run side by side.
+                parts = 1
+                if meta.max_kv >= self.PREFILL_SPLIT_KEYS:
+                    parts = max(2, min(self.PREFILL_MAX_SPLITS, 1 + meta.max_kv // (2 * self.PREFILL_SPLIT_KEYS)))
                 part_o = part_ml = None
-                if halves:
-                    part_o = torch.empty((2, T, num_heads, head_dim), dtype=torch.float32, device=self.device)
-                    part_ml = torch.empty((2, T, num_heads, 2), dtype=torch.float32, device=self.device)
+                if parts > 1:
+                    part_o = torch.empty((parts, T, num_heads, head_dim), dtype=torch.float32, device=self.device)
+                    part_ml = torch.empty((parts, T, num_heads, 2), dtype=torch.float32, device=self.device)
                 _check(lib.distie_attention_prefill_bf16(
                     qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), meta.positions.data_ptr(),
                     meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], out.data_ptr(), T, meta.num_requests,
                     num_heads, num_kv_heads, meta.block_size, float(scale), int(window or 0),
                     2 if split_decode else 1, meta.token_request.data_ptr(),
-                    part_o.data_ptr() if halves else None, part_ml.data_ptr() if halves else None, self._stream()),
+                    part_o.data_ptr() if parts > 1 else None, part_ml.data_ptr() if parts > 1 else None, parts,
+                    self._stream()),
                     "attention_prefill_bf16")
             return out
         _check(lib.distie_attention_generic(
