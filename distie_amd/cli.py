@@ -32,6 +32,11 @@ def _engine_options(parser: argparse.ArgumentParser) -> None:
     parser.add_argument("--token-budget", type=int, default=None)
     parser.add_argument("--no-decode-graphs", action="store_true")
     parser.add_argument("--step-stats", type=int, default=None, help="log a time breakdown every N steps")
+    parser.add_argument("--no-packed-weights", action="store_true",
+                        help="no second copy of the weights in the matrix cores' order (half the weight memory, "
+                             "slower decode)")
+    parser.add_argument("--tune-products", action="store_true",
+                        help="at start, let the library time its kernels for the products of a full portion")
 
 
 def _build(args):
@@ -41,7 +46,8 @@ def _build(args):
     engine = EngineConfig.from_env(
         dtype=args.dtype, block_size=args.block_size, num_blocks=args.num_blocks, max_seqs=args.max_seqs,
         token_budget=args.token_budget, use_graphs=False if args.no_decode_graphs else None,
-        step_stats=args.step_stats, seed=args.seed)
+        step_stats=args.step_stats, seed=args.seed, packed_weights=False if args.no_packed_weights else None,
+        tune_products=True if args.tune_products else None)
     config = json.loads(args.config_json.read_text()) if args.config_json else None
     if args.model is None and config is None:
         raise SystemExit("give --model DIR, or --config-json FILE with --random-weights")

@@ -42,6 +42,7 @@ class EngineConfig:
     max_model_len: Optional[int] = None     # None = the model's max positions
     use_graphs: bool = True
     packed_weights: bool = True             # a second copy of the weights in the matrix cores' order, for decode
+    lookahead: bool = True                  # launch the next decode step before this step's tokens reach the host
     tune_products: bool = False             # at start, let the library time its kernels for a full portion's products
     step_stats: int = 0
     seed: int = 0

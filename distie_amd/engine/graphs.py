@@ -73,20 +73,20 @@ class DecodeGraphs:
     def captured(self) -> List[int]:
         return sorted(size for size, b in self._made.items() if b.graph is not None)
 
-    def try_run(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def try_run(self, entries: Sequence[StepEntry], feed: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Logits [wanted, vocab] if this step went through a graph, None if it must run the
         ordinary way (not a pure decode step, too many rows, or graphs have failed)."""
         if self.failed or len(entries) > self.max_batch or any(len(e.tokens) != 1 for e in entries):
             return None
         try:
-            return self._run(entries)
+            return self._run(entries, feed)
         except Exception:  # noqa: BLE001 - the ordinary path rewrites the same slots
             _log.exception("captured decode step failed; all steps run uncaptured from now on")
             self.failed = True
             self._made.clear()
             return None
 
-    def _run(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def _run(self, entries: Sequence[StepEntry], feed: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         runner = self.runner
         size = bucket_for(self.buckets, len(entries))
         bucket = self._made.get(size)
@@ -96,6 +96,8 @@ class DecodeGraphs:
         runner.builder.fill(bucket.host_np, entries, pad_requests=size - len(entries), want_all=True)
         bucket.dev.copy_(bucket.host, non_blocking=True)
         bucket.copied.record()
+        if feed is not None:
+            bucket.dev[:len(entries)].copy_(feed)        # the token ids lead the packed buffer
         if bucket.graph is None:
             self._capture(bucket)
         else:

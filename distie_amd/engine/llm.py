@@ -28,7 +28,7 @@ from ..weights import load_into, random_into
 from .batch import StepEntry
 from .model import Model
 from .runner import ModelRunner
-from .scheduler import Emission, Scheduler, Sequence, StepPlan
+from .scheduler import Emission, Scheduler, Sequence, SeqState, StepPlan
 from .stats import StepStats
 
 _log = logging.getLogger(__name__)
@@ -100,6 +100,10 @@ class LLM:
         self.stats = StepStats(ec.step_stats) if ec.step_stats else None
         self.eos_ids = tuple(spec.eos_token_ids)
         self._counter = itertools.count()
+        self._ahead = None            # (plan, logits) of a step that is launched and not yet completed
+        self._picked = None           # pinned host buffer for the sampled ids
+        self._ahead_failed = None     # (plan, error) of a step planned ahead whose launch raised
+        self.steps_ahead = 0          # steps launched before the tokens of the step before were known
         self._outputs: Dict[Hashable, RequestOutput] = {}
         self._started: Dict[Hashable, float] = {}
         if ec.use_graphs and hasattr(ops, "graphs_supported") and ops.graphs_supported():
@@ -167,36 +171,58 @@ class LLM:
         return self.scheduler.has_work()
 
     def run_step(self) -> List[Emission]:
-        """One turn of the loop: schedule, step, sample, complete."""
+        """One turn of the loop: schedule, step, sample, complete.
+
+        With `lookahead`, a step of decoding requests is followed at once by the next one, planned
+        before the host has seen this step's tokens (`Scheduler.schedule_ahead`) and fed with them
+        on the device; the host then waits for this step's tokens while the next step runs, and the
+        next turn starts with that step already launched."""
         t0 = time.perf_counter()
-        plan = self.scheduler.schedule()
-        if not plan.items:
-            if self.scheduler.num_waiting and not self.scheduler.num_running:
-                raise RuntimeError("the scheduler cannot place the waiting requests: cache too small")
-            return []
+        plan, logits = None, None
+        if self._ahead is not None:
+            plan, logits = self._ahead
+            self._ahead = None
+            if not any(it.seq.state is SeqState.RUNNING for it in plan.items):
+                plan, logits = None, None        # every request of it has ended meanwhile: nothing to take from it
+        launched = plan is not None
+        if plan is None:
+            plan = self.scheduler.schedule()
+            if not plan.items:
+                if self.scheduler.num_waiting and not self.scheduler.num_running:
+                    raise RuntimeError("the scheduler cannot place the waiting requests: cache too small")
+                return []
         t1 = time.perf_counter()
-        entries = [StepEntry(it.seq.request_id, it.token_ids, [len(it.token_ids) - 1] if it.samples else [])
-                   for it in plan.items]
         try:
-            logits = self.runner.step(entries, reserve=False)
+            if not launched:
+                logits = self.runner.step(self._entries(plan), reserve=False)
             t2 = time.perf_counter()
             sampling = [it for it in plan.items if it.samples]
             picks: List[Optional[int]] = [None] * len(plan.items)
             if sampling:
                 seeds = [it.seq.params.seed if it.seq.params.seed is not None else self.engine_config.seed
                          for it in sampling]
-                tokens = self.sampler.sample(
+                chosen = self.sampler.sample_device(
                     logits, [it.seq.params.temperature for it in sampling], seeds,
                     [len(it.seq.output_ids) for it in sampling])
-                chosen = iter(tokens)
-                picks = [next(chosen) if it.samples else None for it in plan.items]
+                fetch = self._to_host(chosen)
+                if self.engine_config.lookahead:
+                    self._launch_ahead(plan, chosen)
+                tokens = iter(fetch())
+                picks = [next(tokens) if it.samples else None for it in plan.items]
         except Exception as exc:  # noqa: BLE001 - every request of the step learns of it
             _log.exception("step failed; its %d requests end with the error", len(plan.items))
+            self._ahead = None
             for seq in self.scheduler.fail(plan, exc):
                 out = self._outputs[seq.request_id]
                 out.finished, out.finish_reason, out.error = True, "error", repr(exc)
             return []
         emissions = self.scheduler.complete(plan, picks)
+        if self._ahead_failed is not None:
+            failed_plan, exc = self._ahead_failed
+            self._ahead_failed = None
+            for seq in self.scheduler.fail(failed_plan, exc):
+                out = self._outputs[seq.request_id]
+                out.finished, out.finish_reason, out.error = True, "error", repr(exc)
         now = time.perf_counter()
         for e in emissions:
             out = self._outputs[e.seq.request_id]
@@ -213,6 +239,50 @@ class LLM:
             self.stats.record("decode" if plan.is_decode else "prefill", len(plan.items), plan.num_tokens,
                               sched=(t1 - t0) * 1e3, gpu=(t2 - t1) * 1e3, emit=(now - t2) * 1e3)
         return emissions
+
+    @staticmethod
+    def _entries(plan: StepPlan) -> List[StepEntry]:
+        return [StepEntry(it.seq.request_id, it.token_ids, [len(it.token_ids) - 1] if it.samples else [])
+                for it in plan.items]
+
+    def _to_host(self, chosen: torch.Tensor):
+        """Start the copy of the sampled ids to the host; the returned function waits for it."""
+        if chosen.device.type != "cuda":
+            return chosen.tolist
+        n = chosen.shape[0]
+        if self._picked is None or self._picked.shape[0] < n:
+            self._picked = torch.empty(max(n, self.engine_config.max_seqs), dtype=torch.int32, pin_memory=True)
+        self._picked[:n].copy_(chosen, non_blocking=True)
+        arrived = torch.cuda.Event()
+        arrived.record()
+
+        def fetch():
+            arrived.synchronize()
+            return self._picked[:n].tolist()
+        return fetch
+
+    def _launch_ahead(self, plan: StepPlan, chosen: torch.Tensor) -> None:
+        """Launch the step after `plan`, if it can be planned without `plan`'s tokens: they are taken
+        from `chosen` (row i of the sampled rows of `plan`) on the device."""
+        ahead = self.scheduler.schedule_ahead(plan)
+        if ahead is None:
+            return
+        try:
+            sampled_row = {}
+            for i, it in enumerate(plan.items):
+                if it.samples:
+                    sampled_row[i] = len(sampled_row)
+            rows = [sampled_row[i] for i in ahead.feeds]
+            feed = chosen
+            if rows != list(range(chosen.shape[0])):
+                index = torch.tensor(rows, dtype=torch.int32, device=chosen.device)
+                feed = self.ops.gather_rows(chosen.view(-1, 1), index).view(-1)
+            self._ahead = (ahead, self.runner.step(self._entries(ahead), reserve=False, feed=feed))
+            self.steps_ahead += 1
+        except Exception as exc:  # noqa: BLE001 - its requests learn of it once the running step is completed
+            _log.exception("the step planned ahead failed; its %d requests end with the error", len(ahead.items))
+            self._ahead = None
+            self._ahead_failed = (ahead, exc)
 
     def stream(self, prompts: Seq[Seq[int]], params=None) -> Iterator[Emission]:
         """Yield (request, token, finished) as tokens are produced."""

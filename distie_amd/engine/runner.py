@@ -31,9 +31,16 @@ class ModelRunner:
         self.graphs = None          # set by the engine when captured decode steps are on
         model.prepare(ops)
 
-    def step(self, entries: Sequence[StepEntry], reserve: bool = True) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], reserve: bool = True,
+             feed: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """-> float32 [wanted, vocab] in the order of the entries and of their `want`
-        (None if nothing is wanted). A request not yet known to the cache is added."""
+        (None if nothing is wanted). A request not yet known to the cache is added.
+
+        `feed` (int32 [len(entries)], on the device): every entry brings one token, and the token of
+        entry i is feed[i], which need not have reached the host (the entries' own tokens are
+        placeholders)."""
+        if feed is not None and (any(len(e.tokens) != 1 for e in entries) or feed.shape[0] != len(entries)):
+            raise ValueError("a fed step takes one token for each entry")
         if not entries:
             raise ValueError("empty step")
         for entry in entries:
@@ -51,12 +58,14 @@ class ModelRunner:
                 raise
         logits, ran = None, False
         if self.graphs is not None:
-            logits = self.graphs.try_run(entries)   # a view of the bucket's buffer: use it before the next step
+            logits = self.graphs.try_run(entries, feed)   # a view of the bucket's buffer: use it before the next step
             ran = logits is not None
             if ran and logits.shape[0] == 0:
                 logits = None
         if not ran:
             ids, meta, want_rows = self.builder.build(entries)
+            if feed is not None:
+                ids.copy_(feed)
             logits = self.model.forward(self.ops, ids, meta, self.cache, self.act_dtype, want_rows)
         for entry in entries:
             self.cache.commit(entry.request_id, len(entry.tokens))

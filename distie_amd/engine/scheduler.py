@@ -87,6 +87,9 @@ class ScheduledSeq:
 @dataclass(frozen=True)
 class StepPlan:
     items: tuple
+    # For a step planned ahead (`Scheduler.schedule_ahead`): item i continues the request of item
+    # `feeds[i]` of the step before, whose sampled token is not known to the host yet.
+    feeds: Optional[tuple] = None
 
     @property
     def num_tokens(self) -> int:
@@ -200,6 +203,41 @@ class Scheduler:
             items.append(self._item(seq, n))
             budget -= n
         return StepPlan(items=tuple(items))
+
+    PENDING = 0        # stands in a planned-ahead item for the token that the step before is still sampling
+
+    def schedule_ahead(self, plan: StepPlan) -> Optional[StepPlan]:
+        """The step after `plan` (launched, not yet completed), planned before `plan`'s tokens are known, so that it can be launched
+        while the host still waits for them; None where that is not plain. It is plain when
+        every request of `plan` decodes from here on (each item samples), every running request is
+        in it, nothing waits to be admitted, and the next page of every request is there: then the
+        next step holds the same requests with one token each, except those that reach their
+        length with the pending token. A request that turns out to have ended with the pending
+        token (end of sequence, abort) has a row of the next step computed for nothing;
+        `complete` skips it."""
+        self._reap_aborted()
+        if self._waiting or not plan.items or len(plan.items) != len(self._running):
+            return None
+        if any(not item.samples or item.seq.state is not SeqState.RUNNING for item in plan.items):
+            return None
+        rows = []
+        for i, item in enumerate(plan.items):
+            # called after `plan` was launched and before it is completed: its token is the pending one
+            if len(item.seq.output_ids) + 1 >= item.seq.max_new_tokens:
+                continue                                  # ends with the pending token, whatever it is
+            rows.append((i, item))
+        if not rows or len(rows) > self.token_budget:
+            return None
+        items = []
+        for _, item in rows:
+            if not self.cache.can_reserve(item.seq.request_id, 1):
+                # pages run out: the plain schedule decides who gives way. What was taken so far stays
+                # with requests that need it for their next token anyway.
+                return None
+            self.cache.reserve(item.seq.request_id, 1)
+            items.append(ScheduledSeq(seq=item.seq, token_ids=[self.PENDING],
+                                      past_len=item.past_len + len(item.token_ids), samples=True))
+        return StepPlan(items=tuple(items), feeds=tuple(i for i, _ in rows))
 
     def _item(self, seq: Sequence, n: int) -> ScheduledSeq:
         begin = seq.num_computed

@@ -52,10 +52,15 @@ class Sampler:
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float], seeds: Sequence[int],
                counters: Sequence[int]) -> List[int]:
         """logits float32 [R, V] -> R token ids (one device-to-host copy)."""
+        return self.sample_device(logits, temperatures, seeds, counters).tolist()
+
+    def sample_device(self, logits: torch.Tensor, temperatures: Sequence[float], seeds: Sequence[int],
+                      counters: Sequence[int]) -> torch.Tensor:
+        """As `sample`, but the ids stay on the device (int32 [R]): nothing waits for them."""
         if logits.shape[0] != len(temperatures):
             raise ValueError("one temperature per row of logits")
         if all(t <= 0 for t in temperatures):
-            return self.ops.argmax(logits).tolist()
+            return self.ops.argmax(logits)
         dev = self.ops.device
         # int64 two's complement carries the unsigned 64-bit seed unchanged
         wrap = lambda v: ((int(v) & _MASK) ^ (1 << 63)) - (1 << 63)
@@ -64,4 +69,4 @@ class Sampler:
             torch.tensor(list(temperatures), dtype=torch.float32, device=dev),
             torch.tensor([wrap(s) for s in seeds], dtype=torch.int64, device=dev),
             torch.tensor([wrap(c) for c in counters], dtype=torch.int64, device=dev))
-        return picks.tolist()
+        return picks

@@ -142,3 +142,51 @@ def test_trace_free_running_and_forced(tiny):
     with pytest.raises(ValueError):
         llm.trace(prompt, 3, forced_ids=[1])
     assert llm.cache.free_pages() == [64, 64]
+
+
+def test_steps_planned_ahead_change_nothing(tiny):
+    """Decoding steps are launched before the tokens of the step before have reached the host: the
+    same tokens as step by step, with requests that end at different lengths, one that stops at an
+    end-of-sequence token (its row of the step after is computed for nothing), sampling with a
+    temperature, and a pool so tight that planning ahead has to give way to preemption."""
+    cfg, folder, weights = tiny
+    prompts = [random_ids(cfg, n, 70 + n) for n in (3, 12, 7, 20)]
+    stop = plain_greedy(weights, cfg, prompts[1], 9)[5]
+    params = [SamplingParams(max_new_tokens=9), SamplingParams(max_new_tokens=14, eos_id=stop),
+              SamplingParams(max_new_tokens=2), SamplingParams(max_new_tokens=11, temperature=0.8, seed=3)]
+    for options in ({}, {"num_blocks": 7}, {"token_budget": 5}):
+        plain_loop = engine(folder, lookahead=False, **options)
+        want = plain_loop.generate(prompts, params)
+        assert plain_loop.steps_ahead == 0
+        ahead = engine(folder, **options)
+        got = ahead.generate(prompts, params)
+        assert ahead.steps_ahead > 0
+        assert [o.token_ids for o in got] == [o.token_ids for o in want]
+        assert [o.finish_reason for o in got] == [o.finish_reason for o in want]
+        assert got[1].finish_reason == "stop" and got[0].finish_reason == "length"
+        ahead.cache.check()
+        pages = options.get("num_blocks", 64)
+        assert ahead.cache.free_pages() == [pages, pages] and ahead.cache.slots.num_free == ahead.cache.num_slots
+        # the engine is as good as new: a second round gives the same
+        again = ahead.generate(prompts, params)
+        assert [o.token_ids for o in again] == [o.token_ids for o in want]
+
+
+def test_abort_and_arrival_while_a_step_is_ahead(tiny):
+    cfg, folder, weights = tiny
+    llm = engine(folder)
+    a = llm.add_request(random_ids(cfg, 6, 1), SamplingParams(max_new_tokens=30))
+    b = llm.add_request(random_ids(cfg, 4, 2), SamplingParams(max_new_tokens=8))
+    for _ in range(3):
+        llm.run_step()
+    assert llm._ahead is not None            # a step is in flight beyond the tokens the host has seen
+    llm.abort(a)
+    late_prompt = random_ids(cfg, 5, 3)
+    c = llm.add_request(late_prompt, SamplingParams(max_new_tokens=6))
+    while llm.has_work():
+        llm.run_step()
+    assert llm._outputs[a].finish_reason == "abort"
+    assert llm._outputs[b].token_ids == plain_greedy(weights, cfg, random_ids(cfg, 4, 2), 8)
+    assert llm._outputs[c].token_ids == plain_greedy(weights, cfg, late_prompt, 6)
+    llm.cache.check()
+    assert llm.cache.free_pages() == [64, 64] and llm.cache.slots.num_free == llm.cache.num_slots

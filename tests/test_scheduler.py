@@ -235,3 +235,50 @@ def test_windowed_group_lets_long_requests_decode_in_few_pages():
         cache.check()
     full, windowed = cache.free_pages()
     assert full == 8 - 5 and windowed >= 8 - 2      # 20 cached: 5 pages in full, at most 2 in the window group
+
+
+def test_the_step_after_is_planned_ahead_only_when_that_is_plain():
+    sched, cache = make(8, block=4)
+    a, b, c = seq("a", 3, max_new=2), seq("b", 2, max_new=5), seq("c", 9, max_new=5)
+    sched.submit(a)
+    sched.submit(b)
+    plan = sched.schedule()
+    for item in plan.items:
+        cache.commit(item.seq.request_id, len(item.token_ids))
+    # both decode from here on, nothing waits: the next step can be planned before the tokens are known
+    ahead = sched.schedule_ahead(plan)
+    assert names(ahead) == ["a", "b"] and ahead.feeds == (0, 1)
+    assert [(i.token_ids, i.past_len, i.samples) for i in ahead.items] == [([sched.PENDING], 3, True), ([sched.PENDING], 2, True)]
+    sched.complete(plan, [7, 8])
+    for item in ahead.items:
+        cache.commit(item.seq.request_id, 1)
+    # a reaches its length with the token that is pending now: it is not in the step after
+    after = sched.schedule_ahead(ahead)
+    assert names(after) == ["b"] and after.feeds == (1,)
+    out = sched.complete(ahead, [5, 6])
+    assert [(e.seq.request_id, e.finished) for e in out] == [("a", True), ("b", False)]
+    cache.commit("b", 1)
+    # b ends with an end-of-sequence token: its row of the step after was computed for nothing
+    again = sched.schedule_ahead(after)
+    assert names(again) == ["b"]
+    out = sched.complete(after, [EOS])
+    assert out[0].finished and b.finish_reason == "stop"
+    assert sched.complete(again, [4]) == [] and b.output_ids == [8, 6, EOS]
+    cache.check()
+    assert cache.free_pages() == [8]
+    # a request that waits, a prompt still in portions, or a page that is not there: no planning ahead
+    sched.submit(seq("d", 2))
+    plan = sched.schedule()
+    for item in plan.items:
+        cache.commit(item.seq.request_id, len(item.token_ids))
+    sched.submit(c)
+    assert sched.schedule_ahead(plan) is None
+    sched.complete(plan, [1])
+    small, cache2 = make(2, block=4, budget=4)
+    small.submit(seq("e", 4, max_new=3))
+    small.submit(seq("f", 4, max_new=3))
+    plan = small.schedule()
+    for item in plan.items:
+        cache2.commit(item.seq.request_id, len(item.token_ids))
+    assert names(plan) == ["e"] and small.schedule_ahead(plan) is None          # f waits
+    small.complete(plan, [1])
