@@ -78,6 +78,9 @@ class ModelSpec:
     final_norm: PartSpec
     head: PartSpec
     eos_token_ids: Sequence[int] = ()
+    # A position encoding that acts on the embeddings (learned or computed absolute positions); encodings
+    # that act inside a mixer (rotation) are named in that mixer's params instead.
+    position: Optional[PartSpec] = None
 
 
 def read_config_json(model_dir) -> dict:

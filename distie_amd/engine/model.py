@@ -31,6 +31,7 @@ class Model:
             feed_forward_norm = build_part("norm", layer.feed_forward_norm)
             self.blocks.append(build_part("block", layer.block, mixer, feed_forward, mixer_norm, feed_forward_norm))
         self.final_norm = build_part("norm", spec.final_norm)
+        self.position = build_part("position", spec.position) if spec.position is not None else None
         self.tied_head = bool(spec.head.get("tied", False))
         self.embedding: Optional[torch.Tensor] = None
         self.head: Optional[torch.Tensor] = None
@@ -46,6 +47,8 @@ class Model:
             for part in (block.mixer_norm, block.mixer, block.feed_forward_norm, block.feed_forward, block):
                 yield part
         yield self.final_norm
+        if self.position is not None:
+            yield self.position
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         """Checkpoint name -> shape, in a fixed order (embedding, layers, final norm, head)."""
@@ -103,6 +106,8 @@ class Model:
         """ids int32 [T] -> float32 logits [R, vocab] at `want_rows` (int32 [R]); None if no
         row is wanted (the step then only fills the cache)."""
         stream = ResidualStream(ops.embed(ids, self.embedding))
+        if self.position is not None:
+            self.position.on_embedding(ops, stream.hidden, meta)
         ctx = StepContext(meta, act_dtype)
         for call in self.spec.order:
             view = cache.layer(call.cache_layer)

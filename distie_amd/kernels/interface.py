@@ -77,6 +77,11 @@ class Ops(abc.ABC):
         read (the HIP kernels return partial sums over slices of K for small batches); parts
         hand the result on to those operations and do nothing else with it."""
 
+    def dense(self, x):
+        """The plain tensor of a result that `linear` returned in a form of its own; any other
+        tensor as it is. For parts that compute on a product's values themselves."""
+        return x
+
     def prepare_linear(self, weight: torch.Tensor, gated: bool = False, rotary=None) -> None:
         """Called once for every weight of a `linear` after it is loaded (`gated`: the weight of a
         `linear_silu_mul`; `rotary = (num_heads, num_kv_heads, head_dim)`: the stacked q/k/v weight

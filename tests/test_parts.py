@@ -308,3 +308,160 @@ def test_toy_architecture_with_a_state_mixer_is_registered_built_and_stepped(ops
     # a new request in a used slot starts from a zero state
     got = runner.step([StepEntry("c", b, list(range(9)))]).cpu()
     assert (got - want_b).abs().max() < 1e-4
+
+
+# ---------------------------------------------------------------------------------------------
+# a second toy architecture: positions learned and added to the embeddings (attention without rotation),
+# and in one layer a routed feed-forward (the best of three experts of different widths, scaled by its
+# router weight) beside a dense one in the other: chosen layer by layer by the configuration
+# ---------------------------------------------------------------------------------------------
+from distie_amd.parts import FeedForward, PositionEncoding   # noqa: E402
+
+
+class LearnedPositions(PositionEncoding):
+    def __init__(self, spec):
+        super().__init__(spec)
+        self.shape = (int(spec.params["max_positions"]), int(spec.params["hidden_size"]))
+        self.table = None
+
+    def param_specs(self):
+        return {"weight": ParamSpec(self.shape)}
+
+    def load(self, tensors):
+        self.table = tensors["weight"].float()
+
+    def on_embedding(self, ops, hidden, meta):
+        hidden += self.table[meta.positions.long()]
+
+
+class BestOfExperts(FeedForward):
+    def __init__(self, spec):
+        super().__init__(spec)
+        self.hidden = int(spec.params["hidden_size"])
+        self.widths = [int(w) for w in spec.params["expert_sizes"]]
+        self.router = None
+        self.gate_up, self.down = [], []
+
+    def param_specs(self):
+        specs = {"router.weight": ParamSpec((len(self.widths), self.hidden))}
+        for e, width in enumerate(self.widths):
+            specs[f"experts.{e}.gate_proj.weight"] = ParamSpec((width, self.hidden))
+            specs[f"experts.{e}.up_proj.weight"] = ParamSpec((width, self.hidden))
+            specs[f"experts.{e}.down_proj.weight"] = ParamSpec((self.hidden, width))
+        return specs
+
+    def load(self, tensors):
+        self.router = tensors["router.weight"].contiguous()
+        for e in range(len(self.widths)):
+            self.gate_up.append(torch.cat([tensors[f"experts.{e}.gate_proj.weight"],
+                                           tensors[f"experts.{e}.up_proj.weight"]]).contiguous())
+            self.down.append(tensors[f"experts.{e}.down_proj.weight"].contiguous())
+
+    def prepare(self, ops):
+        for gate_up, down in zip(self.gate_up, self.down):
+            ops.prepare_linear(gate_up, gated=True)
+            ops.prepare_linear(down)
+
+    def forward(self, ops, x, ctx):
+        weights = torch.softmax(ops.dense(ops.linear(x, self.router)).float(), dim=-1)      # router in float32
+        best = weights.argmax(-1)
+        out = torch.zeros(x.shape[0], self.hidden, dtype=torch.float32, device=x.device)
+        for e in range(len(self.widths)):
+            rows = (best == e).nonzero().view(-1).to(torch.int32)
+            if rows.numel() == 0:
+                continue
+            mine = ops.gather_rows(x, rows)
+            y = ops.dense(ops.linear(ops.linear_silu_mul(mine, self.gate_up[e]), self.down[e])).float()
+            out[rows.long()] = y * weights[rows.long(), e][:, None]
+        return out.to(x.dtype)
+
+
+class RoutedToyConfig:
+    def __init__(self, data):
+        self.hidden, self.vocab, self.heads = data["hidden"], data["vocab"], data["heads"]
+        self.expert_sizes, self.max_positions = data["expert_sizes"], data["max_positions"]
+
+    @classmethod
+    def from_dict(cls, data):
+        return cls(data)
+
+    def model_spec(self):
+        h = self.hidden
+        norm = lambda p: PartSpec("rmsnorm", p, {"size": h, "eps": 1e-6})
+        attention = lambda p: PartSpec("attention", p, {"hidden_size": h, "num_heads": self.heads, "num_kv_heads": self.heads,
+                                                        "head_dim": h // self.heads, "qkv_bias": False})     # no position inside
+        feed_forward = [PartSpec("swiglu", "l0.ffn.", {"hidden_size": h, "intermediate_size": 3 * h}),
+                        PartSpec("test_best_of_experts", "l1.moe.", {"hidden_size": h, "expert_sizes": self.expert_sizes})]
+        layers = [LayerSpec(PartSpec("prenorm_residual"), attention(f"l{l}.attn."), feed_forward[l], norm(f"l{l}.n1."),
+                            norm(f"l{l}.n2.")) for l in range(2)]
+        return ModelSpec("RoutedToyForCausalLM", self.vocab, h, self.max_positions, PartSpec("token_embedding", "emb."),
+                         layers, (LayerCall(0), LayerCall(1)), norm("final."), PartSpec("lm_head", "head.", {"tied": False}),
+                         position=PartSpec("test_learned_positions", "pos.", {"max_positions": self.max_positions,
+                                                                              "hidden_size": h}))
+
+
+def routed_toy_plain(weights, cfg, ids, first_position=0):
+    """-> (logits, smallest gap between the two best router weights): float64, whole sequence, no cache."""
+    w = {k: v.double() for k, v in weights.items()}
+    n, h, heads = len(ids), cfg.hidden, cfg.heads
+    x = w["emb.weight"][torch.tensor(ids)] + w["pos.weight"][first_position:first_position + n]
+    rms = lambda t, p: plain.rms_norm(t, w[p + "weight"], 1e-6)
+
+    def attention(t, p):
+        q, k, v = ((t @ w[p + f"{name}_proj.weight"].T).view(n, heads, h // heads) for name in "qkv")
+        return plain.attention(q, k, v).reshape(n, h) @ w[p + "o_proj.weight"].T
+
+    swiglu = lambda t, p: plain.swiglu(t, w[p + "gate_proj.weight"], w[p + "up_proj.weight"], w[p + "down_proj.weight"])
+    x = x + attention(rms(x, "l0.n1."), "l0.attn.")
+    x = x + swiglu(rms(x, "l0.n2."), "l0.ffn.")
+    x = x + attention(rms(x, "l1.n1."), "l1.attn.")
+    t = rms(x, "l1.n2.")
+    route = torch.softmax(t @ w["l1.moe.router.weight"].T, -1)
+    top = route.topk(2, dim=-1).values
+    y = torch.stack([swiglu(t[i:i + 1], f"l1.moe.experts.{int(route[i].argmax())}.")[0] * route[i].max() for i in range(n)])
+    x = x + y
+    return rms(x, "final.") @ w["head.weight"].T, float((top[:, 0] - top[:, 1]).min())
+
+
+def test_toy_architecture_with_learned_positions_and_a_routed_feed_forward(ops):
+    register_part("position", "test_learned_positions", LearnedPositions)
+    register_part("feed_forward", "test_best_of_experts", BestOfExperts)
+    register_architecture("RoutedToyForCausalLM", RoutedToyConfig)
+    from distie_amd.config import config_from_dict
+
+    cfg = config_from_dict({"architectures": ["RoutedToyForCausalLM"], "hidden": 48, "vocab": 90, "heads": 3,
+                            "expert_sizes": [40, 72, 24], "max_positions": 64})
+    model = Model(cfg.model_spec())
+    specs = model.param_specs()
+    assert {"pos.weight", "l1.moe.router.weight", "l1.moe.experts.2.down_proj.weight", "l0.ffn.up_proj.weight",
+            "head.weight"} <= set(specs)
+    gen = torch.Generator().manual_seed(8)
+    weights = {n: (torch.ones(s.shape) if s.init == "ones" else torch.randn(s.shape, generator=gen) * 0.25)
+               for n, s in specs.items()}
+    weights["l1.moe.router.weight"] *= 6.0          # decided choices: rounding must not flip an expert
+    model.load_tensors(lambda name: weights[name].to(ops.device))
+    cache = CacheManager(model.cache_requirements(), 4, 32, 4, device=ops.device, dtype=torch.float32)
+    runner = ModelRunner(model, cache, ops, torch.float32, 64)
+    a = torch.randint(0, 90, (29,), generator=gen).tolist()
+    b = torch.randint(0, 90, (11,), generator=gen).tolist()
+    (want_a, gap_a), (want_b, gap_b) = routed_toy_plain(weights, cfg, a), routed_toy_plain(weights, cfg, b)
+    assert min(gap_a, gap_b) > 1e-3
+    # the pin of the plain side: positions are absolute here, so a shift of all positions does change the result
+    assert (routed_toy_plain(weights, cfg, a[:5], first_position=3)[0] - want_a[:5]).abs().max() > 1e-3
+    got = runner.step([StepEntry("a", a, list(range(29)))]).cpu()
+    assert (got - want_a.float()).abs().max() < 1e-4
+    runner.finish("a")
+    rows = {"a": [], "b": []}
+    seqs = {"a": a, "b": b}
+    for step in [[("a", 0, 6)], [("a", 6, 8), ("b", 0, 4)], [("a", 8, 27), ("b", 4, 5)], [("b", 5, 11), ("a", 27, 28)],
+                 [("a", 28, 29)]]:
+        logits = runner.step([StepEntry(r, seqs[r][lo:hi], list(range(hi - lo))) for r, lo, hi in step]).cpu()
+        at = 0
+        for r, lo, hi in step:
+            rows[r].append(logits[at:at + hi - lo])
+            at += hi - lo
+    assert (torch.cat(rows["a"]) - want_a.float()).abs().max() < 1e-4
+    assert (torch.cat(rows["b"]) - want_b.float()).abs().max() < 1e-4
+    runner.finish("a")
+    runner.finish("b")
+    cache.check()
