@@ -442,7 +442,7 @@ class HipOps(Ops):
             if split_decode:
                 # requests that bring one token: keys are cut into runs, one wave each, so that the chip is
                 # filled even when few requests decode
-                runs = max(1, min(64, 4096 // (singles * num_kv_heads)))
+                runs = max(1, min(64, 1024 // (singles * num_kv_heads)))
                 split_len = max(64, -(-(-(-meta.max_kv // runs)) // 64) * 64)
                 max_splits = -(-meta.max_kv // split_len)
                 part_o = torch.empty((meta.num_requests, num_heads, max_splits, head_dim), dtype=torch.float32,
