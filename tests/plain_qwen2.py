@@ -74,11 +74,16 @@ def rope_inv_freq(head_dim: int, theta: float, dtype=torch.float32) -> torch.Ten
     return 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=dtype) / head_dim))
 
 
-def rope_cos_sin(positions: torch.Tensor, head_dim: int, theta: float, dtype=torch.float32):
-    """cos/sin of concat(ang, ang), ang = pos * inv_freq: worker/src/inference/qwen2/model.py:101-105."""
-    freqs = positions.to(dtype)[:, None] * rope_inv_freq(head_dim, theta, dtype)[None, :]
+def rope_cos_sin(positions: torch.Tensor, head_dim: int, theta: float, dtype=torch.float32,
+                 angle_dtype=torch.float32):
+    """cos/sin of concat(ang, ang), ang = pos * inv_freq: worker/src/inference/qwen2/model.py:101-105.
+    Frequencies, angles and the trigonometry are float32 whatever `dtype` is (`.float()` at :98 and
+    :103), and only the results take the dtype of the activations (:105): at position 2,000 a
+    float32 angle is off by up to 1e-4 rad, which is part of what the reference computes.
+    (`angle_dtype=float64` is for tests of the formula itself.)"""
+    freqs = positions.to(angle_dtype)[:, None] * rope_inv_freq(head_dim, theta, angle_dtype)[None, :]
     emb = torch.cat((freqs, freqs), dim=-1)
-    return emb.cos(), emb.sin()
+    return emb.cos().to(dtype), emb.sin().to(dtype)
 
 
 def rotate_half(x: torch.Tensor) -> torch.Tensor:
@@ -134,7 +139,7 @@ def swiglu(x, w_gate, w_up, w_down) -> torch.Tensor:
     return (silu(x @ w_gate.T) * (x @ w_up.T)) @ w_down.T
 
 
-def self_attention(x, w: dict, prefix: str, positions, cfg: dict, window) -> torch.Tensor:
+def self_attention(x, w: dict, prefix: str, positions, cfg: dict, window, angle_dtype=torch.float32) -> torch.Tensor:
     """q/k/v with bias, rope on q and k, attention, o without bias:
     worker/src/inference/qwen2/model.py:149-152, 214-225."""
     t = x.shape[0]
@@ -144,25 +149,26 @@ def self_attention(x, w: dict, prefix: str, positions, cfg: dict, window) -> tor
     q = (x @ w[prefix + "q_proj.weight"].T + w[prefix + "q_proj.bias"]).view(t, h, d)
     k = (x @ w[prefix + "k_proj.weight"].T + w[prefix + "k_proj.bias"]).view(t, kh, d)
     v = (x @ w[prefix + "v_proj.weight"].T + w[prefix + "v_proj.bias"]).view(t, kh, d)
-    cos, sin = rope_cos_sin(positions, d, rope_theta_of(cfg), x.dtype)
+    cos, sin = rope_cos_sin(positions, d, rope_theta_of(cfg), x.dtype, angle_dtype)
     q = apply_rope(q, cos, sin)
     k = apply_rope(k, cos, sin)
     mixed = attention(q, k, v, window)
     return mixed.reshape(t, h * d) @ w[prefix + "o_proj.weight"].T
 
 
-def decoder_layer(x, w: dict, index: int, positions, cfg: dict, window) -> torch.Tensor:
+def decoder_layer(x, w: dict, index: int, positions, cfg: dict, window, angle_dtype=torch.float32) -> torch.Tensor:
     """h += attn(norm(h)); h += mlp(norm(h)): worker/src/inference/qwen2/model.py:247-249."""
     p = f"model.layers.{index}."
     eps = float(cfg["rms_norm_eps"])
     x = x + self_attention(rms_norm(x, w[p + "input_layernorm.weight"], eps), w, p + "self_attn.",
-                           positions, cfg, window)
+                           positions, cfg, window, angle_dtype)
     normed = rms_norm(x, w[p + "post_attention_layernorm.weight"], eps)
     return x + swiglu(normed, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                       w[p + "mlp.down_proj.weight"])
 
 
-def forward(w: dict, cfg: dict, ids, dtype=torch.float32, first_position: int = 0) -> torch.Tensor:
+def forward(w: dict, cfg: dict, ids, dtype=torch.float32, first_position: int = 0,
+            angle_dtype=torch.float32) -> torch.Tensor:
     """Token ids [T] -> logits [T, vocab] of one whole sequence:
     worker/src/inference/qwen2/model.py:305-314 (tied head: :302-303)."""
     w = {k: v.to(dtype) for k, v in w.items()}
@@ -170,7 +176,7 @@ def forward(w: dict, cfg: dict, ids, dtype=torch.float32, first_position: int = 
     x = w["model.embed_tokens.weight"][ids]
     positions = torch.arange(first_position, first_position + ids.shape[0])
     for index, window in enumerate(layer_windows(cfg)):
-        x = decoder_layer(x, w, index, positions, cfg, window)
+        x = decoder_layer(x, w, index, positions, cfg, window, angle_dtype)
     x = rms_norm(x, w["model.norm.weight"], float(cfg["rms_norm_eps"]))
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
     return x @ head.T

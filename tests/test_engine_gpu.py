@@ -121,3 +121,19 @@ def test_long_decoding(setup, ops):
     runner = build_runner(folder, ops, dtype, block_size=block, num_blocks=-(-n // block))
     ids = random_ids(cfg, n, 4)
     check_logits(replay_cut(runner, "a", ids, [5]), weights, cfg, ids, dtype, folder)
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_long_context_in_portions_then_decoding(tmp_path, ops, dtype_name):
+    """2,300 tokens: portions whose walks over the keys are cut in parts (from 1,024 keys on), a window
+    layer whose pages are given back on the way, then single tokens over many runs of keys."""
+    dtype = DTYPES[dtype_name]
+    cfg = dict(plain.TINY_C, max_position_embeddings=4096, sliding_window=700)
+    folder, weights = make_model_dir(tmp_path, cfg, seed=13, dtype=dtype)
+    runner = build_runner(folder, ops, dtype, block_size=16, num_blocks=160, max_model_len=4096)
+    ids = random_ids(cfg, 2310, 6)
+    got = replay_cut(runner, "a", ids, [1500, 700, 100, 2])
+    check_logits(got, weights, cfg, ids, dtype, folder)
+    runner.cache.check()
+    free = runner.cache.free_pages()
+    assert free[0] == 160 and free[1] == 160

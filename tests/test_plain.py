@@ -49,13 +49,13 @@ def test_inv_freq_values():
 def test_rope_pairing_and_sign():
     # D = 2: the pair is (0, 1); a unit vector on the first axis turns to (cos p, sin p).
     pos = torch.tensor([0, 1, 3])
-    cos, sin = plain.rope_cos_sin(pos, 2, 10000.0, torch.float64)
+    cos, sin = plain.rope_cos_sin(pos, 2, 10000.0, torch.float64, torch.float64)
     x = torch.tensor([1.0, 0.0], dtype=torch.float64).expand(3, 1, 2)
     y = plain.apply_rope(x, cos, sin)
     for t, p in enumerate([0.0, 1.0, 3.0]):
         assert torch.allclose(y[t, 0], torch.tensor([math.cos(p), math.sin(p)], dtype=torch.float64))
     # D = 4: element j pairs with j + D/2, not with j + 1.
-    cos, sin = plain.rope_cos_sin(torch.tensor([2]), 4, 100.0, torch.float64)
+    cos, sin = plain.rope_cos_sin(torch.tensor([2]), 4, 100.0, torch.float64, torch.float64)
     x = torch.tensor([[[1.0, 0.0, 0.0, 0.0]]], dtype=torch.float64)
     y = plain.apply_rope(x, cos, sin)[0, 0]
     assert torch.allclose(y, torch.tensor([math.cos(2.0), 0.0, math.sin(2.0), 0.0], dtype=torch.float64))
@@ -69,17 +69,31 @@ def test_rope_identity_at_zero_norms_and_relative_scores():
     d = 16
     q = torch.randn(6, 2, d, dtype=torch.float64)
     k = torch.randn(6, 2, d, dtype=torch.float64)
-    cos0, sin0 = plain.rope_cos_sin(torch.zeros(6, dtype=torch.long), d, 1e4, torch.float64)
+    cos0, sin0 = plain.rope_cos_sin(torch.zeros(6, dtype=torch.long), d, 1e4, torch.float64, torch.float64)
     assert torch.allclose(plain.apply_rope(q, cos0, sin0), q)
     pos = torch.tensor([0, 3, 4, 9, 20, 21])
-    cos, sin = plain.rope_cos_sin(pos, d, 1e4, torch.float64)
+    cos, sin = plain.rope_cos_sin(pos, d, 1e4, torch.float64, torch.float64)
     rq = plain.apply_rope(q, cos, sin)
     pair = lambda x: x[..., : d // 2] ** 2 + x[..., d // 2:] ** 2
     assert torch.allclose(pair(rq), pair(q))
-    cos2, sin2 = plain.rope_cos_sin(pos + 37, d, 1e4, torch.float64)
+    cos2, sin2 = plain.rope_cos_sin(pos + 37, d, 1e4, torch.float64, torch.float64)
     s1 = torch.einsum("qhd,khd->hqk", rq, plain.apply_rope(k, cos, sin))
     s2 = torch.einsum("qhd,khd->hqk", plain.apply_rope(q, cos2, sin2), plain.apply_rope(k, cos2, sin2))
     assert torch.allclose(s1, s2, atol=1e-9)
+
+
+def test_rope_angles_are_float32_as_in_the_reference():
+    """worker/src/inference/qwen2/model.py:98-105 computes frequencies, angles and trigonometry in
+    float32: far from position 0 that is visibly not the exact angle, and it is what the model uses."""
+    pos = torch.tensor([0, 1, 2000, 4000])
+    cos32, sin32 = plain.rope_cos_sin(pos, 64, 1e6, torch.float64)
+    cos64, sin64 = plain.rope_cos_sin(pos, 64, 1e6, torch.float64, torch.float64)
+    assert cos32.dtype == torch.float64
+    assert torch.equal(cos32[0], cos64[0]) and (cos32[1] - cos64[1]).abs().max() < 1e-6
+    far = (sin32[2:] - sin64[2:]).abs().max().item()
+    assert 1e-6 < far < 5e-4
+    freqs = pos.to(torch.float32)[:, None] * plain.rope_inv_freq(64, 1e6, torch.float32)[None, :]
+    assert torch.equal(cos32[:, :32], freqs.cos().double())
 
 
 def test_attention_is_library_causal_attention_when_heads_are_not_grouped():
@@ -150,10 +164,13 @@ def test_swiglu_reductions():
 def test_shift_of_all_positions_changes_nothing(cfg):
     w = plain.random_weights(cfg, 1, std=0.3, norm_jitter=0.2)
     ids = torch.randint(0, cfg["vocab_size"], (30,), generator=torch.Generator().manual_seed(2))
-    a = plain.forward(w, cfg, ids, torch.float64)
-    b = plain.forward(w, cfg, ids, torch.float64, first_position=41)
+    # with exact angles only distances count; with the reference's float32 angles (the default) nearly
+    a = plain.forward(w, cfg, ids, torch.float64, angle_dtype=torch.float64)
+    b = plain.forward(w, cfg, ids, torch.float64, first_position=41, angle_dtype=torch.float64)
     assert torch.allclose(a, b, atol=1e-8)
     assert a.shape == (30, cfg["vocab_size"])
+    c = plain.forward(w, cfg, ids, torch.float64, first_position=41)
+    assert torch.allclose(a, c, atol=1e-3) and not torch.allclose(a, c, atol=1e-9)
 
 
 def test_logits_are_causal_and_windows_follow_the_config():
