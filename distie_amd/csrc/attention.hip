@@ -573,10 +573,9 @@ constexpr int PF_BM = PF_WAVES * PF_WAVE_COLS;          // query tokens per work
 constexpr int PF_DEPTH = 2;                             // key tiles whose loads are in flight
 constexpr int PF_K_STRIDE = D + 8;                      // elements; the padding spreads rows over the banks
 constexpr int PF_V_STRIDE = PF_BN + 8;
-constexpr int PF_K_CHUNKS = PF_BN * D / 8;              // 16-byte pieces of a K tile
-constexpr int PF_V_CHUNKS = D * PF_BN / 8;
-constexpr int PF_K_PER_THREAD = (PF_K_CHUNKS + PF_THREADS - 1) / PF_THREADS;
-constexpr int PF_V_PER_THREAD = (PF_V_CHUNKS + PF_THREADS - 1) / PF_THREADS;
+constexpr int PF_BLOCK_CHUNKS = 2 * D;                  // 16-byte pieces of 16 keys of K, and of V^T: [16, D] or [D, 16]
+constexpr int PF_PASSES = (PF_BLOCK_CHUNKS + DISTIE_WAVE - 1) / DISTIE_WAVE;   // pieces a lane carries per block
+static_assert(PF_WAVES * 16 == PF_BN, "each wave brings one block of 16 keys of a tile");
 
 __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_kernel(
     const bf16_t* __restrict__ qkv, int64_t q_stride, const bf16_t* __restrict__ k_cache,
@@ -643,83 +642,53 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
     for (int db = 0; db < DB16; ++db) o_acc[mb][db] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // ---- staging of one tile in registers: 16-byte pieces of K rows and of V^T rows
-  // PF_DEPTH tiles are in flight: a tile's trip from memory is longer than the work on a tile
-  uint4 k_stages[PF_DEPTH][PF_K_PER_THREAD], v_stages[PF_DEPTH][PF_V_PER_THREAD];
-  // Every thread issues the same number of loads for every tile, with no branch around them: pieces that
-  // belong to no page read the start of the cache instead and are cleared when they are stored.
+  // ---- staging of one tile in registers. Wave w brings block w of the tile (keys k0 + 16 w .. + 15): one page
+  // lookup a wave, the 16 rows of K are one run of 16 D elements in their page, V^T is D runs of 16.
+  // PF_DEPTH tiles are in flight: a tile's trip from memory is longer than the work on a tile.
+  uint4 k_stages[PF_DEPTH][PF_PASSES], v_stages[PF_DEPTH][PF_PASSES];
+  const int block_shift = (block_size & (block_size - 1)) == 0 ? __builtin_ctz(block_size) : -1;
+  // Every lane issues the same loads for every tile, with no branch around them: a block that belongs to no
+  // page reads the start of the cache instead and is cleared when it is stored.
   auto block_live = [&](int key) { return key <= key_end && key + 15 >= key_begin; };
-  auto fetch = [&](int k0, uint4 (&k_stage)[PF_K_PER_THREAD], uint4 (&v_stage)[PF_V_PER_THREAD]) {
-    int64_t base[4];
-    int offset[4];
+  auto fetch = [&](int k0, uint4 (&k_stage)[PF_PASSES], uint4 (&v_stage)[PF_PASSES]) {
+    const int key = k0 + 16 * wave;
+    const bool live = block_live(key);
+    const int slot = block_shift >= 0 ? key >> block_shift : key / block_size;
+    const int offset = live ? (block_shift >= 0 ? key & (block_size - 1) : key % block_size) : 0;
+    const int page = live ? table[slot] : 0;
+    const int64_t base = live ? (static_cast<int64_t>(page) * kv_heads + kh) * block_size * D : 0;
+    const bf16_t* k_block = k_cache + base + static_cast<int64_t>(offset) * D;
+    const bf16_t* v_block = v_cache + base + offset;
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      const int key = k0 + 16 * b;
-      const bool live = block_live(key);
-      const int page = live ? table[key / block_size] : 0;
-      base[b] = live ? (static_cast<int64_t>(page) * kv_heads + kh) * block_size * D : 0;
-      offset[b] = live ? key % block_size : 0;
-    }
-#pragma unroll
-    for (int i = 0; i < PF_K_PER_THREAD; ++i) {
-      const int c = min(tid + i * PF_THREADS, PF_K_CHUNKS - 1);
-      const int row = c / (D / 8);
-      const int piece = c % (D / 8);
-      const int b = row / 16;
-      const int64_t base_b = b == 0 ? base[0] : (b == 1 ? base[1] : (b == 2 ? base[2] : base[3]));
-      const int offset_b = b == 0 ? offset[0] : (b == 1 ? offset[1] : (b == 2 ? offset[2] : offset[3]));
-      k_stage[i] = *reinterpret_cast<const uint4*>(k_cache + base_b + static_cast<int64_t>(offset_b + row % 16) * D + 8 * piece);
-    }
-#pragma unroll
-    for (int i = 0; i < PF_V_PER_THREAD; ++i) {
-      const int c = min(tid + i * PF_THREADS, PF_V_CHUNKS - 1);
-      const int d = c / 8;
-      const int piece = c % 8;              // 8 keys each
-      const int b = piece / 2;
-      const int64_t base_b = b == 0 ? base[0] : (b == 1 ? base[1] : (b == 2 ? base[2] : base[3]));
-      const int offset_b = b == 0 ? offset[0] : (b == 1 ? offset[1] : (b == 2 ? offset[2] : offset[3]));
-      v_stage[i] = *reinterpret_cast<const uint4*>(v_cache + base_b + static_cast<int64_t>(d) * block_size + offset_b + 8 * (piece % 2));
+    for (int p = 0; p < PF_PASSES; ++p) {
+      const int j = min(lane + p * DISTIE_WAVE, PF_BLOCK_CHUNKS - 1);
+      k_stage[p] = *reinterpret_cast<const uint4*>(k_block + 8 * j);
+      v_stage[p] = *reinterpret_cast<const uint4*>(v_block + static_cast<int64_t>(j / 2) * block_size + 8 * (j % 2));
     }
   };
-  auto stash = [&](int k0, const uint4 (&k_stage)[PF_K_PER_THREAD], const uint4 (&v_stage)[PF_V_PER_THREAD]) {
-    if (k0 >= key_begin && k0 + PF_BN - 1 <= key_end) {
-      // every key of the tile is one this workgroup reads: nothing to clear
+  auto stash = [&](int k0, const uint4 (&k_stage)[PF_PASSES], const uint4 (&v_stage)[PF_PASSES]) {
+    const int key = k0 + 16 * wave;
+    const bool live = block_live(key);
+    // Slots after the last key of this workgroup were not written by this request, and blocks outside the keys
+    // of this workgroup were not read: cleared (a weight of zero times NaN would still be NaN).
+    const bool whole = live && key + 15 <= key_end;
 #pragma unroll
-      for (int i = 0; i < PF_K_PER_THREAD; ++i) {
-        const int c = tid + i * PF_THREADS;
-        if (c < PF_K_CHUNKS) *reinterpret_cast<uint4*>(k_lds + (c / (D / 8)) * PF_K_STRIDE + 8 * (c % (D / 8))) = k_stage[i];
-      }
-#pragma unroll
-      for (int i = 0; i < PF_V_PER_THREAD; ++i) {
-        const int c = tid + i * PF_THREADS;
-        if (c < PF_V_CHUNKS) *reinterpret_cast<uint4*>(v_lds + (c / 8) * PF_V_STRIDE + 8 * (c % 8)) = v_stage[i];
-      }
-      return;
-    }
-#pragma unroll
-    for (int i = 0; i < PF_K_PER_THREAD; ++i) {
-      const int c = tid + i * PF_THREADS;
-      if (c < PF_K_CHUNKS) {
-        const int row = c / (D / 8);
-        const uint4 raw = block_live(k0 + row / 16 * 16) ? k_stage[i] : uint4{0u, 0u, 0u, 0u};
-        *reinterpret_cast<uint4*>(k_lds + row * PF_K_STRIDE + 8 * (c % (D / 8))) = raw;
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < PF_V_PER_THREAD; ++i) {
-      const int c = tid + i * PF_THREADS;
-      if (c < PF_V_CHUNKS) {
-        // slots after the last key of this workgroup were not written by this request, and blocks outside the
-        // keys of this workgroup were not read: cleared (a weight of zero times NaN would still be NaN)
-        const int first_key = k0 + 8 * (c % 8);
-        const int written = block_live(first_key / 16 * 16) ? key_end - first_key + 1 : 0;
-        const uint32_t w[4] = {v_stage[i].x, v_stage[i].y, v_stage[i].z, v_stage[i].w};
+    for (int p = 0; p < PF_PASSES; ++p) {
+      const int j = lane + p * DISTIE_WAVE;
+      if (j >= PF_BLOCK_CHUNKS) continue;
+      const uint4 k_raw = live ? k_stage[p] : uint4{0u, 0u, 0u, 0u};
+      *reinterpret_cast<uint4*>(k_lds + (16 * wave + j / (D / 8)) * PF_K_STRIDE + 8 * (j % (D / 8))) = k_raw;
+      uint4 v_raw = v_stage[p];
+      if (!whole) {
+        const int written = live ? key_end - (key + 8 * (j % 2)) + 1 : 0;        // of this piece's eight keys
+        const uint32_t w[4] = {v_raw.x, v_raw.y, v_raw.z, v_raw.w};
         uint32_t m[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e)
           m[e] = written >= 2 * e + 2 ? w[e] : (written == 2 * e + 1 ? (w[e] & 0x0000ffffu) : 0u);
-        *reinterpret_cast<uint4*>(v_lds + (c / 8) * PF_V_STRIDE + 8 * (c % 8)) = uint4{m[0], m[1], m[2], m[3]};
+        v_raw = uint4{m[0], m[1], m[2], m[3]};
       }
+      *reinterpret_cast<uint4*>(v_lds + (j / 2) * PF_V_STRIDE + 16 * wave + 8 * (j % 2)) = v_raw;
     }
   };
 
