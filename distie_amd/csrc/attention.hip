@@ -571,7 +571,10 @@ constexpr int PF_MB = 1;                                // blocks of 16 query co
 constexpr int PF_WAVE_COLS = 16 * PF_MB;
 constexpr int PF_BM = PF_WAVES * PF_WAVE_COLS;          // query tokens per workgroup
 constexpr int PF_DEPTH = 2;                             // key tiles whose loads are in flight
-constexpr int PF_K_STRIDE = D + 8;                      // elements; the padding spreads rows over the banks
+// Rows of K in LDS, in elements. Lane (r, g) reads 16 bytes at row r, byte 16 g (+ a constant): that is free
+// of bank conflicts when the row stride is 32 bytes more than a multiple of 64 (measured with the LDS
+// conflict counter: 16 or 48 bytes more cost every read twice).
+constexpr int PF_K_STRIDE = (D % 32 == 0) ? D + 16 : D;
 constexpr int PF_V_STRIDE = PF_BN + 8;
 constexpr int PF_BLOCK_CHUNKS = 2 * D;                  // 16-byte pieces of 16 keys of K, and of V^T: [16, D] or [D, 16]
 constexpr int PF_PASSES = (PF_BLOCK_CHUNKS + DISTIE_WAVE - 1) / DISTIE_WAVE;   // pieces a lane carries per block
