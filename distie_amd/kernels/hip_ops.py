@@ -116,8 +116,10 @@ class HipOps(Ops):
         import os
         import tempfile
 
-        import torch.cuda.tunable as tunable
-
+        try:
+            import torch.cuda.tunable as tunable
+        except ImportError:           # a torch without it: the library's own choice stands
+            return
         if on:
             # the library insists on a results file: keep it out of the working directory
             folder = tempfile.mkdtemp(prefix=f"distie_tune_{os.getuid()}_")
