@@ -137,3 +137,15 @@ def test_long_context_in_portions_then_decoding(tmp_path, ops, dtype_name):
     runner.cache.check()
     free = runner.cache.free_pages()
     assert free[0] == 160 and free[1] == 160
+
+
+def test_a_file_in_32_bit_under_a_bfloat16_engine(tmp_path, ops):
+    """Tensors that the file keeps in 32-bit stay so: the products then run on the float32 kernel with
+    bfloat16 activations, without packed copies and without the fused epilogues."""
+    cfg, block = CONFIGS["C"]
+    folder, weights = make_model_dir(tmp_path, cfg, seed=17, dtype=torch.float32)
+    runner = build_runner(folder, ops, torch.bfloat16, block_size=block)
+    assert runner.model.blocks[0].mixer.qkv_weight.dtype == torch.float32
+    assert not hasattr(runner.model.blocks[0].mixer.qkv_weight, "_distie_rotary")
+    ids = random_ids(cfg, 90, 8)
+    check_logits(replay_cut(runner, "a", ids, [50, 20, 3]), weights, cfg, ids, torch.bfloat16, folder)
