@@ -17,6 +17,7 @@ replay; nothing inside the graph depends on a Python number.
 from __future__ import annotations
 
 import bisect
+import gc
 import logging
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -124,8 +125,19 @@ class DecodeGraphs:
         graph = torch.cuda.CUDAGraph()
         if self._pool is None:
             self._pool = torch.cuda.graph_pool_handle()
-        with torch.cuda.graph(graph, pool=self._pool):
-            bucket.logits = self._forward(bucket)
+        # While a stream captures, calls such as freeing pinned memory or querying an event are errors, and one
+        # raised in a destructor ends the process. The garbage collector could run such destructors of
+        # objects that died earlier (an engine that was dropped) at any allocation in here: it is held
+        # off for the capture, and what other threads do is not this capture's business.
+        was_enabled = gc.isenabled()
+        gc.collect()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph, pool=self._pool, capture_error_mode="thread_local"):
+                bucket.logits = self._forward(bucket)
+        finally:
+            if was_enabled:
+                gc.enable()
         # capture launches nothing: replay once so that `logits` holds this step's result
         graph.replay()
         bucket.graph = graph

@@ -156,3 +156,21 @@ def test_tuned_library_products(tmp_path):
     finally:
         tunable.tuning_enable(False)
         tunable.enable(False)
+
+
+def test_engines_made_and_dropped_one_after_the_other(tmp_path):
+    """Every engine captures its decode steps anew while the remains of the one before (pinned buffers,
+    graphs) wait for the garbage collector: their destructors must not run inside a capture."""
+    from distie_amd import LLM, SamplingParams
+
+    cfg = plain.TINY_A
+    folder, weights = make_model_dir(tmp_path, cfg, seed=3)
+    prompts = [random_ids(cfg, n, 80 + n) for n in (3, 11, 6)]
+    first = None
+    for _ in range(8):
+        llm = LLM(folder, dtype="fp32", block_size=16, num_blocks=24, max_seqs=4)
+        outs = [o.token_ids for o in llm.generate(prompts, SamplingParams(max_new_tokens=10))]
+        assert llm.runner.graphs.captured and llm.steps_ahead > 0
+        first = first or outs
+        assert outs == first
+        llm.circular = llm            # a cycle: only the garbage collector can free this engine
