@@ -365,8 +365,10 @@ static __device__ __forceinline__ uint2 pack_bf16x4(const float v[4]) {
 }
 
 // blockIdx.x: row block; blockIdx.y: slice of K (PLAIN only; slices side by side in y, bias on slice 0, as
-// gemm_skinny_kernel). The WAVES waves of a workgroup share the slice's tiles and add their sums through
-// LDS; wave 0 writes. M <= 16.
+// gemm_skinny_kernel); blockIdx.z: a group of 16 rows of x (with more than 16 rows the weights are read once
+// per group, from the L2 after the first: the choice for weights too small to occupy the chip through the
+// wide kernel below). The WAVES waves of a workgroup share the slice's tiles and add their sums through
+// LDS; wave 0 writes.
 template <typename Y, int MODE, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void gemm_packed_kernel(const bf16_t* __restrict__ x,
                                                                  const bf16_t* __restrict__ w,
@@ -377,6 +379,19 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_packed_kernel(const bf16_t* _
   const int wave = threadIdx.x / 64;
   const int r = lane % 16;
   const int g = lane / 16;
+  const int m_all = M;
+  const int m0 = 16 * blockIdx.z;
+  x += static_cast<int64_t>(m0) * K;
+  M = min(16, M - m0);
+  if constexpr (MODE == PK_ROTARY) {
+    y += static_cast<int64_t>(m0) * N;
+    rotary.table += static_cast<int64_t>(m0) * (rotary.dim / 2);
+    if (rotary.slots != nullptr) rotary.slots += m0;
+  } else if constexpr (MODE == PK_GATED) {
+    y += static_cast<int64_t>(m0) * (N / 2);
+  } else {
+    y += static_cast<int64_t>(m0) * N;
+  }
   const int k_tiles = (K + 31) / 32;
   const int s_begin = blockIdx.y * tiles_per_slice;
   const int s_end = min(k_tiles, s_begin + tiles_per_slice);
@@ -468,7 +483,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_packed_kernel(const bf16_t* _
       }
     }
   } else {
-    Y* out = y + static_cast<int64_t>(blockIdx.y) * M * N;
+    Y* out = y + static_cast<int64_t>(blockIdx.y) * m_all * N;
     const bool with_bias = bias != nullptr && blockIdx.y == 0;
     if (r < M) {
 #pragma unroll
@@ -488,16 +503,16 @@ static int packed_waves(int K) {
 
 // y: as distie_gemm_skinny_bf16 (the same cut along K: slices go to other workgroups, hence to other
 // compute units, which a product with few rows of W needs to pull its bytes fast enough);
-// gated: [M, N / 2] of y_dtype, never cut.
+// gated: [M, N / 2] of y_dtype, never cut. Up to 64 rows of x, in groups of 16.
 extern "C" int distie_gemm_packed_bf16(const void* x, const void* w_packed, const float* bias, void* y, int y_dtype,
                                        int M, int N, int K, int gated, hipStream_t stream) {
   if (M <= 0) return 0;
-  if (M > 16 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
+  if (M > 64 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
   int slices = 1, k_per_slice = (K + SK_KSTEP - 1) / SK_KSTEP * SK_KSTEP;
   if (!gated) skinny_plan(N, K, &slices, &k_per_slice);
   if (slices > 1 && y_dtype != DISTIE_F32) return DISTIE_BAD_ARGUMENT;
   const int row_blocks = gated ? (N / 2 + 7) / 8 : (N + 15) / 16;
-  dim3 grid(row_blocks, slices);
+  dim3 grid(row_blocks, slices, (M + 15) / 16);
   const bf16_t* xb = static_cast<const bf16_t*>(x);
   const bf16_t* wb = static_cast<const bf16_t*>(w_packed);
   const RotaryOut none = {};
@@ -526,8 +541,7 @@ template <typename Y, int MODE, int MB>
 __global__ __launch_bounds__(256, 2) void gemm_packed_wide_kernel(const bf16_t* __restrict__ x,
                                                                const bf16_t* __restrict__ w,
                                                                const float* __restrict__ bias, Y* __restrict__ y,
-                                                               int M, int N, int K, int row_blocks, int tiles_per_slice,
-                                                               RotaryOut rotary) {
+                                                               int M, int N, int K, int row_blocks, int tiles_per_slice) {
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][MB * 16][WD_XROW];
   const int tid = threadIdx.x;
   const int lane = tid % 64;
@@ -638,51 +652,6 @@ __global__ __launch_bounds__(256, 2) void gemm_packed_wide_kernel(const bf16_t* 
         for (int i = 0; i < 4; ++i)
           if (n0 + i < half) y[static_cast<int64_t>(m) * half + n0 + i] = from_float<Y>(v[i]);
       }
-    } else if constexpr (MODE == PK_ROTARY) {
-      const int dim = rotary.dim;
-      const int half = dim / 2;
-      const int per_head = dim / 16;
-      const int rotated_blocks = (rotary.heads + rotary.kv_heads) * per_head;
-      const bool turns = block < rotated_blocks;
-      const int head = block / per_head;
-      const int sub = block % per_head;
-      const int d0 = turns ? (g / 2) * half + 8 * sub + 4 * (g % 2) : 16 * sub + 4 * g;
-      float own[4], other[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        own[i] = acc[b][i] + (bias != nullptr ? bias[static_cast<int64_t>(head) * dim + d0 + i] : 0.f);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) other[i] = __shfl_xor(own[i], 32, 64);
-      if (m >= M) continue;
-      float v[4];
-      if (turns) {
-        const float2* angles = rotary.table + static_cast<int64_t>(m) * half + 8 * sub + 4 * (g % 2);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float2 cs = angles[i];
-          v[i] = g < 2 ? own[i] * cs.x - other[i] * cs.y : own[i] * cs.x + other[i] * cs.y;
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = own[i];
-      }
-      const uint2 packed = pack_bf16x4(v);
-      *reinterpret_cast<uint2*>(y + static_cast<int64_t>(m) * N + static_cast<int64_t>(head) * dim + d0) = packed;
-      if (rotary.write && head >= rotary.heads) {
-        const int64_t slot = rotary.slots[m];
-        const int64_t page = slot / rotary.block_size;
-        const int offset = static_cast<int>(slot % rotary.block_size);
-        if (turns) {
-          const int kv_head = head - rotary.heads;
-          *reinterpret_cast<uint2*>(rotary.k_cache +
-                                    ((page * rotary.kv_heads + kv_head) * rotary.block_size + offset) * dim + d0) = packed;
-        } else {
-          const int kv_head = head - rotary.heads - rotary.kv_heads;
-          bf16_t* at = rotary.v_cache + ((page * rotary.kv_heads + kv_head) * dim + d0) * rotary.block_size + offset;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) at[static_cast<int64_t>(i) * rotary.block_size] = static_cast<bf16_t>(v[i]);
-        }
-      }
     } else {
       Y* out = y + static_cast<int64_t>(blockIdx.y) * M * N;
       const bool with_bias = bias != nullptr && blockIdx.y == 0;
@@ -716,9 +685,9 @@ extern "C" int distie_gemm_packed_wide_slices(int N, int K) {
 }
 
 // 17 to 64 rows of x. mode 0: y [M, N] of y_dtype, or float32 [slices, M, N] when the plan cuts K
-// (distie_gemm_packed_wide_slices); 1 (gated): [M, N / 2]; 2 (rotary): as distie_gemm_packed_rotary_bf16.
+// (distie_gemm_packed_wide_slices); 1 (gated): [M, N / 2].
 static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bias, void* y, int y_dtype, int M, int N,
-                              int K, int mode, const RotaryOut& rotary, hipStream_t stream) {
+                              int K, int mode, hipStream_t stream) {
   const int row_blocks = mode == PK_GATED ? (N / 2 + 7) / 8 : (N + 15) / 16;
   int slices = 1, tiles_per_slice = 4 * ((K + SK_KSTEP - 1) / SK_KSTEP);
   if (mode == PK_PLAIN) wide_plan(row_blocks, K, &slices, &tiles_per_slice);
@@ -727,7 +696,7 @@ static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bia
   const int mb = (M + 15) / 16;
 #define WIDE(MODE, MB)                                                                                   \
   DISTIE_DISPATCH(y_dtype, Y, (gemm_packed_wide_kernel<Y, MODE, MB><<<grid, 256, 0, stream>>>(           \
-                                  x, w, bias, static_cast<Y*>(y), M, N, K, row_blocks, tiles_per_slice, rotary)))
+                                  x, w, bias, static_cast<Y*>(y), M, N, K, row_blocks, tiles_per_slice)))
 #define WIDE_MB(MODE)                    \
   switch (mb) {                          \
     case 1: WIDE(MODE, 1); break;        \
@@ -737,8 +706,6 @@ static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bia
   }
   if (mode == PK_GATED) {
     WIDE_MB(PK_GATED);
-  } else if (mode == PK_ROTARY) {
-    WIDE_MB(PK_ROTARY);
   } else {
     WIDE_MB(PK_PLAIN);
   }
@@ -751,14 +718,14 @@ extern "C" int distie_gemm_packed_wide_bf16(const void* x, const void* w_packed,
                                             int y_dtype, int M, int N, int K, int gated, hipStream_t stream) {
   if (M <= 0) return 0;
   if (M > 64 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
-  const RotaryOut none = {};
   return packed_wide_launch(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w_packed), bias, y, y_dtype, M, N,
-                            K, gated ? PK_GATED : PK_PLAIN, none, stream);
+                            K, gated ? PK_GATED : PK_PLAIN, stream);
 }
 
 // The stacked q/k/v product with the rotation and the cache write in its epilogue. w_packed: the ROTARY
 // copy of the [(heads + 2 kv_heads) * dim, K] weight. y: bfloat16 [M, N], rotated. dim a multiple of 16;
-// table: [M, dim / 2] (cos, sin).
+// table: [M, dim / 2] (cos, sin). Up to 64 rows of x, in groups of 16: a workgroup owns one row block of
+// one group, so that even this small weight is pulled by hundreds of workgroups.
 extern "C" int distie_gemm_packed_rotary_bf16(const void* x, const void* w_packed, const float* bias, void* y,
                                               const void* table, const int32_t* slots, void* k_cache, void* v_cache,
                                               int M, int K, int heads, int kv_heads, int dim, int block_size,
@@ -773,9 +740,8 @@ extern "C" int distie_gemm_packed_rotary_bf16(const void* x, const void* w_packe
   const bf16_t* xb = static_cast<const bf16_t*>(x);
   const bf16_t* wb = static_cast<const bf16_t*>(w_packed);
   bf16_t* out = static_cast<bf16_t*>(y);
-  if (M > 16) return packed_wide_launch(xb, wb, bias, y, DISTIE_BF16, M, N, K, PK_ROTARY, rotary, stream);
   const int tiles = (K + 31) / 32;
-  dim3 grid(N / 16, 1);
+  dim3 grid(N / 16, 1, (M + 15) / 16);
 #define ROTARY(WAVES) \
   gemm_packed_kernel<bf16_t, PK_ROTARY, WAVES><<<grid, 64 * WAVES, 0, stream>>>(xb, wb, bias, out, M, N, K, tiles, rotary)
   switch (packed_waves(K)) {

@@ -72,7 +72,9 @@ class HipOps(Ops):
     SKINNY_MAX_ROWS = 16       # above this the library's tiles are faster than streaming with x from memory
     PREFILL_SPLIT_KEYS = 1024  # from this many visible keys on, a portion's walk over the keys is cut in two parts
     PREFILL_MAX_SPLITS = 4     # (three from four times as many, four from six times; measured: 2 beat 3 at 2,048)
-    PACKED_MAX_ROWS = 64       # ... unless the weight has a packed copy: then up to here x goes through LDS
+    PACKED_MAX_ROWS = 64       # ... unless the weight has a packed copy: then up to here x goes through LDS,
+    ROW_GROUPS_MAX_ELEMENTS = 4 << 20   # or, for a weight of at most this many elements (too few row blocks to occupy
+    #                            the chip that way), through the one-wave kernel once per 16 rows of x
 
     def __init__(self, device="cuda:0", packed_weights: bool = True) -> None:
         """`packed_weights`: keep a second copy of every bfloat16 weight in the order in which the
@@ -345,7 +347,8 @@ class HipOps(Ops):
             raise KernelError("linear: bias must be float32 [N]")
         both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
         packed = getattr(weight, "_distie_packed", None) if both_bf16 else None
-        if packed is not None and self.SKINNY_MAX_ROWS < M <= self.PACKED_MAX_ROWS and K % 8 == 0:
+        if packed is not None and self.SKINNY_MAX_ROWS < M <= self.PACKED_MAX_ROWS and K % 8 == 0 and \
+                N * K > self.ROW_GROUPS_MAX_ELEMENTS:
             if packed.numel() != self._packed_elements(N, K, False):
                 raise KernelError("linear: the packed copy does not belong to this weight")
             slices = self._ops.distie_gemm_packed_wide_slices(N, K)
@@ -359,7 +362,7 @@ class HipOps(Ops):
             if slices == 1:
                 return out
             return PartialSums(out, out_dtype) if partial_ok else self.dense(PartialSums(out, out_dtype))
-        if both_bf16 and M <= self.SKINNY_MAX_ROWS and K % 8 == 0:
+        if both_bf16 and K % 8 == 0 and (M <= self.SKINNY_MAX_ROWS or (packed is not None and M <= self.PACKED_MAX_ROWS)):
             if packed is not None:
                 if packed.numel() != self._packed_elements(N, K, False):
                     raise KernelError("linear: the packed copy does not belong to this weight")

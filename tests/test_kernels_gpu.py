@@ -124,14 +124,23 @@ def test_gemm_packed_bf16(ops, M, N, K):
     want = x.double() @ w.double().T
     got = ops.linear_f32out(x, w)
     close(got, want, torch.float32, scale=5 * want.abs().max().item())
-    part = ops.linear(x, w, b)
-    if M <= 16:
-        assert isinstance(part, PartialSums) == (K >= 768)
-    got = ops.dense(part)
-    assert got.dtype == torch.bfloat16
-    close(got, want + b.double(), torch.bfloat16, scale=want.abs().max().item())
-    # the packed and the natural kernel add the same products in another order: float32 rounding only
-    assert (got.float() - natural).abs().max().item() <= 2 ** -7 * want.abs().max().item()
+    # 17 to 64 rows: small weights go through the one-wave kernel once per 16 rows, large ones through
+    # the kernel that shares x in LDS; both are run for every shape
+    routes = [ops.ROW_GROUPS_MAX_ELEMENTS] if M <= 16 else [0, 1 << 40]
+    try:
+        for limit in routes:
+            ops.ROW_GROUPS_MAX_ELEMENTS = limit
+            part = ops.linear(x, w, b)
+            if M <= 16 or limit > 0:
+                assert isinstance(part, PartialSums) == (K >= 768)
+            got = ops.dense(part)
+            assert got.dtype == torch.bfloat16
+            close(got, want + b.double(), torch.bfloat16, scale=want.abs().max().item())
+            # the packed and the natural kernel add the same products in another order: float32 rounding only
+            assert (got.float() - natural).abs().max().item() <= 2 ** -7 * want.abs().max().item()
+    finally:
+        del ops.ROW_GROUPS_MAX_ELEMENTS
+    assert ops.ROW_GROUPS_MAX_ELEMENTS == type(ops).ROW_GROUPS_MAX_ELEMENTS
 
 
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 40, 64])
