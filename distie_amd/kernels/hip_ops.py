@@ -72,6 +72,7 @@ class HipOps(Ops):
     SKINNY_MAX_ROWS = 16       # above this the library's tiles are faster than streaming with x from memory
     PREFILL_SPLIT_KEYS = 1024  # from this many visible keys on, a portion's walk over the keys is cut in two parts
     PREFILL_MAX_SPLITS = 4     # (three from four times as many, four from six times; measured: 2 beat 3 at 2,048)
+    DECODE_WAVES = 1024        # decode attention cuts the keys into runs so that about this many waves are at work
     PACKED_MAX_ROWS = 64       # ... unless the weight has a packed copy: then up to here x goes through LDS,
     ROW_GROUPS_MAX_ELEMENTS = 4 << 20   # or, for a weight of at most this many elements (too few row blocks to occupy
     #                            the chip that way), through the one-wave kernel once per 16 rows of x
@@ -455,7 +456,7 @@ class HipOps(Ops):
             if split_decode:
                 # requests that bring one token: keys are cut into runs, one wave each, so that the chip is
                 # filled even when few requests decode
-                runs = max(1, min(64, 1024 // (singles * num_kv_heads)))
+                runs = max(1, min(64, self.DECODE_WAVES // (singles * num_kv_heads)))
                 split_len = max(64, -(-(-(-meta.max_kv // runs)) // 64) * 64)
                 max_splits = -(-meta.max_kv // split_len)
                 part_o = torch.empty((meta.num_requests, num_heads, max_splits, head_dim), dtype=torch.float32,
