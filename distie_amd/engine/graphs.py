@@ -12,6 +12,13 @@ cache slots again.
 
 The step's metadata reaches the device with one copy from pinned host memory before the
 replay; nothing inside the graph depends on a Python number.
+
+One number of the step is frozen into a graph all the same: the longest context it is made for,
+from which decode attention derives how it cuts the keys into runs. A graph made for the model's
+limit would cut a 2,000-token context into the few long runs that suit 32,768 tokens, so a bucket
+keeps one graph per class of context length (1,024, 1,536, 2,048, 3,072, ... up to the limit),
+each captured when a step first needs it; a step replays the graph of the smallest class that
+holds its longest request.
 """
 
 from __future__ import annotations
@@ -47,6 +54,21 @@ def bucket_for(buckets: Sequence[int], rows: int) -> int:
     return buckets[bisect.bisect_left(buckets, rows)]
 
 
+def context_classes(limit: int, first: int = 1024) -> Tuple[int, ...]:
+    """(4096) -> 1024, 1536, 2048, 3072, 4096; (700) -> 700: steps of a factor 1.5 or 1.33, so a
+    graph's runs of keys are at most that much longer than the step's own would be."""
+    if limit < 1 or first < 1:
+        raise ValueError("context lengths must be >= 1")
+    out = {limit}
+    c = first
+    while c < limit:
+        out.add(c)
+        if c + c // 2 < limit and c >= 2:
+            out.add(c + c // 2)
+        c *= 2
+    return tuple(sorted(out))
+
+
 class _Bucket:
     def __init__(self, size: int, builder, device) -> None:
         self.size = size
@@ -55,15 +77,18 @@ class _Bucket:
         self.host = torch.zeros(words, dtype=torch.int32, pin_memory=True)
         self.host_np = self.host.numpy()
         self.dev = torch.zeros(words, dtype=torch.int32, device=device)
-        self.graph: Optional[torch.cuda.CUDAGraph] = None
-        self.logits: Optional[torch.Tensor] = None
+        # per class of context length: (graph, its logits buffer)
+        self.graphs: Dict[int, Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
         self.copied = torch.cuda.Event()
 
 
 class DecodeGraphs:
+    FIRST_CONTEXT = 1024        # the shortest class of context length
+
     def __init__(self, runner, max_batch: int) -> None:
         self.runner = runner
         self.buckets = decode_buckets(max_batch)
+        self.contexts = context_classes(runner.max_model_len, self.FIRST_CONTEXT)
         self.max_batch = max_batch
         self._made: Dict[int, _Bucket] = {}
         self._pool = None
@@ -72,7 +97,13 @@ class DecodeGraphs:
 
     @property
     def captured(self) -> List[int]:
-        return sorted(size for size, b in self._made.items() if b.graph is not None)
+        """Batch sizes that have a graph."""
+        return sorted(size for size, b in self._made.items() if b.graphs)
+
+    @property
+    def captured_contexts(self) -> List[Tuple[int, int]]:
+        """(batch size, context class) of every graph."""
+        return sorted((size, limit) for size, b in self._made.items() for limit in b.graphs)
 
     def try_run(self, entries: Sequence[StepEntry], feed: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Logits [wanted, vocab] if this step went through a graph, None if it must run the
@@ -94,33 +125,36 @@ class DecodeGraphs:
         if bucket is None:
             bucket = self._made[size] = _Bucket(size, runner.builder, runner.ops.device)
         bucket.copied.synchronize()                      # the previous copy out of the pinned buffer is done
-        runner.builder.fill(bucket.host_np, entries, pad_requests=size - len(entries), want_all=True)
+        max_kv = runner.builder.fill(bucket.host_np, entries, pad_requests=size - len(entries), want_all=True)[5]
         bucket.dev.copy_(bucket.host, non_blocking=True)
         bucket.copied.record()
         if feed is not None:
             bucket.dev[:len(entries)].copy_(feed)        # the token ids lead the packed buffer
-        if bucket.graph is None:
-            self._capture(bucket)
+        limit = self.contexts[bisect.bisect_left(self.contexts, max_kv)]
+        made = bucket.graphs.get(limit)
+        if made is None:
+            logits = self._capture(bucket, limit)
         else:
-            bucket.graph.replay()
+            made[0].replay()
+            logits = made[1]
             self.replays += 1
         rows = [i for i, e in enumerate(entries) if len(e.want)]
         if not rows:
-            return bucket.logits[:0]
+            return logits[:0]
         if len(rows) == len(entries):
-            return bucket.logits[:len(entries)]
-        return bucket.logits[torch.tensor(rows, device=bucket.logits.device)]
+            return logits[:len(entries)]
+        return logits[torch.tensor(rows, device=logits.device)]
 
-    def _forward(self, bucket: _Bucket) -> torch.Tensor:
+    def _forward(self, bucket: _Bucket, limit: int) -> torch.Tensor:
         runner = self.runner
         n = bucket.size
-        ids, meta, want = runner.builder.meta_of(bucket.dev, bucket.offsets, n, n, n, 1, runner.max_model_len)
+        ids, meta, want = runner.builder.meta_of(bucket.dev, bucket.offsets, n, n, n, 1, limit)
         return runner.model.forward(runner.ops, ids, meta, runner.cache, runner.act_dtype, want)
 
-    def _capture(self, bucket: _Bucket) -> None:
+    def _capture(self, bucket: _Bucket, limit: int) -> torch.Tensor:
         # one ordinary run first: sizes scratch buffers and writes this step's keys and values
         torch.cuda.synchronize()
-        eager = self._forward(bucket)
+        eager = self._forward(bucket, limit)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         if self._pool is None:
@@ -134,12 +168,13 @@ class DecodeGraphs:
         gc.disable()
         try:
             with torch.cuda.graph(graph, pool=self._pool, capture_error_mode="thread_local"):
-                bucket.logits = self._forward(bucket)
+                logits = self._forward(bucket, limit)
         finally:
             if was_enabled:
                 gc.enable()
         # capture launches nothing: replay once so that `logits` holds this step's result
         graph.replay()
-        bucket.graph = graph
+        bucket.graphs[limit] = (graph, logits)
         self.replays += 1
         del eager
+        return logits

@@ -73,6 +73,7 @@ class HipOps(Ops):
     PREFILL_SPLIT_KEYS = 1024  # from this many visible keys on, a portion's walk over the keys is cut in two parts
     PREFILL_MAX_SPLITS = 4     # (three from four times as many, four from six times; measured: 2 beat 3 at 2,048)
     DECODE_WAVES = 1024        # decode attention cuts the keys into runs so that about this many waves are at work
+    DECODE_MAX_RUNS = 256      # places for partial results per request and head
     PACKED_MAX_ROWS = 64       # ... unless the weight has a packed copy: then up to here x goes through LDS,
     ROW_GROUPS_MAX_ELEMENTS = 4 << 20   # or, for a weight of at most this many elements (too few row blocks to occupy
     #                            the chip that way), through the one-wave kernel once per 16 rows of x
@@ -457,7 +458,11 @@ class HipOps(Ops):
                 # requests that bring one token: keys are cut into runs, one wave each, so that the chip is
                 # filled even when few requests decode
                 runs = max(1, min(64, self.DECODE_WAVES // (singles * num_kv_heads)))
-                split_len = max(64, -(-(-(-meta.max_kv // runs)) // 64) * 64)
+                # under a window only the runs that hold its keys do anything: cut by the window's length,
+                # but into no more than DECODE_MAX_RUNS places for partial results
+                visible = min(meta.max_kv, int(window)) if window else meta.max_kv
+                split_len = max(-(-visible // runs), -(-meta.max_kv // self.DECODE_MAX_RUNS))
+                split_len = max(64, -(-split_len // 64) * 64)
                 max_splits = -(-meta.max_kv // split_len)
                 part_o = torch.empty((meta.num_requests, num_heads, max_splits, head_dim), dtype=torch.float32,
                                      device=self.device)

@@ -2,7 +2,7 @@
 
 import pytest
 
-from distie_amd.engine.graphs import bucket_for, decode_buckets
+from distie_amd.engine.graphs import bucket_for, context_classes, decode_buckets
 
 
 def test_decode_buckets():
@@ -21,3 +21,15 @@ def test_bucket_for():
         bucket_for(buckets, 33)
     with pytest.raises(ValueError):
         bucket_for(buckets, 0)
+
+
+def test_context_classes():
+    assert context_classes(4096) == (1024, 1536, 2048, 3072, 4096)
+    assert context_classes(700) == (700,)
+    assert context_classes(1025) == (1024, 1025)
+    assert context_classes(40, first=2) == (2, 3, 4, 6, 8, 12, 16, 24, 32, 40)
+    classes = context_classes(32768)
+    assert classes[0] == 1024 and classes[-1] == 32768
+    assert all(b <= 1.5 * a for a, b in zip(classes, classes[1:]))
+    with pytest.raises(ValueError):
+        context_classes(0)

@@ -158,6 +158,41 @@ def test_tuned_library_products(tmp_path):
         tunable.enable(False)
 
 
+def test_captured_steps_per_class_of_context_length(tmp_path, monkeypatch):
+    """A captured decode step is made for a longest context (decode attention cuts the keys into runs by
+    it), so a bucket holds one graph per class of length; contexts that grow through several classes,
+    alone and three at a time, give the logits of the whole sequences."""
+    from distie_amd import LLM
+    from distie_amd.engine.batch import StepEntry
+    from distie_amd.engine.graphs import DecodeGraphs
+    from engine_util import check_logits
+
+    monkeypatch.setattr(DecodeGraphs, "FIRST_CONTEXT", 32)
+    cfg = plain.TINY_C
+    folder, weights = make_model_dir(tmp_path, cfg, seed=8, dtype=torch.bfloat16)
+    llm = LLM(folder, dtype="bf16", block_size=16, num_blocks=40, max_seqs=4)
+    assert llm.runner.graphs.contexts[:5] == (32, 48, 64, 96, 128)
+    seqs = {name: random_ids(cfg, n, 17 + n) for name, n in (("a", 150), ("b", 70), ("c", 101))}
+    got = {name: [] for name in seqs}
+    starts = {"a": 20, "b": 1, "c": 40}
+    for name, ids in seqs.items():                 # the first tokens as a portion, uncaptured
+        n = starts[name]
+        got[name].append(llm.step([StepEntry(name, ids[:n], list(range(n)))]).float().cpu())
+    at = dict(starts)
+    while any(at[name] < len(ids) for name, ids in seqs.items()):
+        live = [name for name, ids in seqs.items() if at[name] < len(ids)]
+        logits = llm.step([StepEntry(name, [seqs[name][at[name]]], [0]) for name in live]).float().cpu()
+        for row, name in enumerate(live):
+            got[name].append(logits[row:row + 1])
+            at[name] += 1
+    made = llm.runner.graphs.captured_contexts
+    assert {size for size, _ in made} == {1, 2, 4} and len({limit for _, limit in made}) >= 5, made
+    for name, ids in seqs.items():
+        llm.finish(name)
+        check_logits(torch.cat(got[name]), weights, cfg, ids, torch.bfloat16, folder)
+    llm.cache.check()
+
+
 def test_engines_made_and_dropped_one_after_the_other(tmp_path):
     """Every engine captures its decode steps anew while the remains of the one before (pinned buffers,
     graphs) wait for the garbage collector: their destructors must not run inside a capture."""
