@@ -69,20 +69,30 @@ class PartialSums:
 
 
 class HipOps(Ops):
-    SKINNY_MAX_ROWS = 16       # above this the library's tiles are faster than streaming with x from memory
-    PREFILL_SPLIT_KEYS = 1024  # from this many visible keys on, a portion's walk over the keys is cut in two parts
-    PREFILL_MAX_SPLITS = 4     # (three from four times as many, four from six times; measured: 2 beat 3 at 2,048)
-    DECODE_WAVES = 1024        # decode attention cuts the keys into runs so that about this many waves are at work
-    DECODE_MAX_RUNS = 256      # places for partial results per request and head
-    PACKED_MAX_ROWS = 64       # ... unless the weight has a packed copy: then up to here x goes through LDS,
-    ROW_GROUPS_MAX_ELEMENTS = 4 << 20   # or, for a weight of at most this many elements (too few row blocks to occupy
-    #                            the chip that way), through the one-wave kernel once per 16 rows of x
+    # bfloat16 products by rows of x: up to SKINNY_MAX_ROWS the weights are streamed by one wave per block
+    # of 16 weight rows, x straight from memory (above that, the library's tiles are faster);
+    SKINNY_MAX_ROWS = 16
+    # with a packed copy of the weight, up to PACKED_MAX_ROWS rows go through the kernel that shares the
+    # x tile of a workgroup in LDS,
+    PACKED_MAX_ROWS = 64
+    # or, for a weight of at most this many elements (too few row blocks to occupy the chip that way),
+    # through the one-wave kernel once per 16 rows of x
+    ROW_GROUPS_MAX_ELEMENTS = 4 << 20
+    # attention over a portion of a prompt: from PREFILL_SPLIT_KEYS visible keys on, the walk over the keys
+    # is cut in two parts (three from four times as many, four from six times; measured: 2 beat 3 at 2,048)
+    PREFILL_SPLIT_KEYS = 1024
+    PREFILL_MAX_SPLITS = 4
+    # decode attention cuts the keys into runs so that about DECODE_WAVES waves are at work, with at most
+    # DECODE_MAX_RUNS places for partial results per request and head
+    DECODE_WAVES = 1024
+    DECODE_MAX_RUNS = 256
 
     def __init__(self, device="cuda:0", packed_weights: bool = True) -> None:
         """`packed_weights`: keep a second copy of every bfloat16 weight in the order in which the
-        matrix cores take it, for products with at most `SKINNY_MAX_ROWS` rows (decode). It doubles
-        the memory of the weights and makes those products 15-25 % faster; without it they stream
-        the weights as they are stored."""
+        matrix cores take it, for products with at most `PACKED_MAX_ROWS` rows (decode). It doubles
+        the memory of the weights and makes those products 15-25 % faster, and it is what the fused
+        epilogues (activation, rotation and cache write) work on; without it products of up to
+        `SKINNY_MAX_ROWS` rows stream the weights as they are stored and larger ones go to the library."""
         self.device = torch.device(device)
         self.packed_weights = bool(packed_weights)
         if self.device.type != "cuda" or not torch.cuda.is_available():

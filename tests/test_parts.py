@@ -1,7 +1,8 @@
 """Each part alone against the plain implementation, and the generality of the assembly:
 a toy mixer with state of its own, defined here, is registered, built into a model beside
 attention layers and stepped; a run order that names a layer twice and lets a layer read
-another layer's cache. No file of the package changes for this.
+another layer's cache; two more toy architectures bring a position encoding and a routed
+feed-forward, and a norm and an arrangement of their own. No file of the package changes for this.
 
 Runs on the CPU test double, and on the HIP kernels when a GPU is there."""
 
@@ -455,6 +456,140 @@ def test_toy_architecture_with_learned_positions_and_a_routed_feed_forward(ops):
     seqs = {"a": a, "b": b}
     for step in [[("a", 0, 6)], [("a", 6, 8), ("b", 0, 4)], [("a", 8, 27), ("b", 4, 5)], [("b", 5, 11), ("a", 27, 28)],
                  [("a", 28, 29)]]:
+        logits = runner.step([StepEntry(r, seqs[r][lo:hi], list(range(hi - lo))) for r, lo, hi in step]).cpu()
+        at = 0
+        for r, lo, hi in step:
+            rows[r].append(logits[at:at + hi - lo])
+            at += hi - lo
+    assert (torch.cat(rows["a"]) - want_a.float()).abs().max() < 1e-4
+    assert (torch.cat(rows["b"]) - want_b.float()).abs().max() < 1e-4
+    runner.finish("a")
+    runner.finish("b")
+    cache.check()
+
+
+# ---------------------------------------------------------------------------------------------
+# a third toy architecture: a norm of its own (centred, with a bias) and an arrangement of its own
+# (post-norm: h = norm(h + sublayer(h))) in layer 0, beside the pre-norm RMS layer of the package in
+# layer 1: norm and arrangement are chosen layer by layer like every other part
+# ---------------------------------------------------------------------------------------------
+from distie_amd.parts import Block, Norm   # noqa: E402
+
+
+class CentredNorm(Norm):
+    def __init__(self, spec):
+        super().__init__(spec)
+        self.size, self.eps = int(spec.params["size"]), float(spec.params["eps"])
+        self.weight = self.bias = None
+
+    def param_specs(self):
+        return {"weight": ParamSpec((self.size,), "ones"), "bias": ParamSpec((self.size,))}
+
+    def load(self, tensors):
+        self.weight, self.bias = tensors["weight"].float(), tensors["bias"].float()
+
+    def apply(self, ops, x, out_dtype):
+        x = x.float()
+        x = x - x.mean(-1, keepdim=True)
+        return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight + self.bias).to(out_dtype)
+
+    def add_apply(self, ops, residual, delta, out_dtype):
+        residual += dense(ops, delta).float()
+        return self.apply(ops, residual, out_dtype)
+
+
+class PostNormResidual(Block):
+    def forward(self, ops, stream, ctx, cache, writes_cache):
+        if stream.pending is not None:                   # what the layer before left to be added
+            stream.hidden += dense(ops, stream.pending).float()
+            stream.pending = None
+        y = self.mixer.forward(ops, stream.hidden.to(ctx.act_dtype), ctx, cache, writes_cache)
+        stream.hidden = self.mixer_norm.apply(ops, stream.hidden + dense(ops, y).float(), torch.float32)
+        y = self.feed_forward.forward(ops, stream.hidden.to(ctx.act_dtype), ctx)
+        stream.hidden = self.feed_forward_norm.apply(ops, stream.hidden + dense(ops, y).float(), torch.float32)
+
+
+class PostNormToyConfig:
+    def __init__(self, data):
+        self.hidden, self.vocab, self.heads, self.eps = data["hidden"], data["vocab"], data["heads"], data["eps"]
+
+    @classmethod
+    def from_dict(cls, data):
+        return cls(data)
+
+    def model_spec(self):
+        h, d = self.hidden, self.hidden // self.heads
+        centred = lambda p: PartSpec("test_centred_norm", p, {"size": h, "eps": self.eps})
+        rms = lambda p: PartSpec("rmsnorm", p, {"size": h, "eps": self.eps})
+        attention = lambda p: PartSpec("attention", p, {
+            "hidden_size": h, "num_heads": self.heads, "num_kv_heads": 1, "head_dim": d, "qkv_bias": False,
+            "position": PartSpec("rope", "", {"dim": d, "theta": 300.0})})
+        ffn = lambda p: PartSpec("swiglu", p, {"hidden_size": h, "intermediate_size": 2 * h + 8})
+        layers = [LayerSpec(PartSpec("test_postnorm_residual"), attention("l0.attn."), ffn("l0.ffn."), centred("l0.n1."),
+                            centred("l0.n2.")),
+                  LayerSpec(PartSpec("prenorm_residual"), attention("l1.attn."), ffn("l1.ffn."), rms("l1.n1."), rms("l1.n2."))]
+        return ModelSpec("PostNormToyForCausalLM", self.vocab, h, 128, PartSpec("token_embedding", "emb."), layers,
+                         (LayerCall(0), LayerCall(1)), centred("final."), PartSpec("lm_head", "head.", {"tied": False}))
+
+
+def postnorm_toy_plain(weights, cfg, ids, norm_first=False):
+    """float64, whole sequence, no cache. `norm_first`: layer 0 arranged pre-norm instead (the mistake the
+    test must tell from the right arrangement)."""
+    w = {k: v.double() for k, v in weights.items()}
+    n, h = len(ids), cfg.hidden
+    att_cfg = {"num_attention_heads": cfg.heads, "num_key_value_heads": 1, "head_dim": h // cfg.heads, "rope_theta": 300.0}
+
+    def centred(t, p):
+        t = t - t.mean(-1, keepdim=True)
+        return t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + cfg.eps) * w[p + "weight"] + w[p + "bias"]
+
+    def attention(t, p):
+        named = dict(w)
+        for name, rows in (("q", h), ("k", h // cfg.heads), ("v", h // cfg.heads)):
+            named[p + f"{name}_proj.bias"] = torch.zeros(rows, dtype=torch.float64)
+        return plain.self_attention(t, named, p, torch.arange(n), att_cfg, None)
+
+    ffn = lambda t, p: plain.swiglu(t, w[p + "gate_proj.weight"], w[p + "up_proj.weight"], w[p + "down_proj.weight"])
+    rms = lambda t, p: plain.rms_norm(t, w[p + "weight"], cfg.eps)
+    x = w["emb.weight"][torch.tensor(ids)]
+    if norm_first:
+        x = x + attention(centred(x, "l0.n1."), "l0.attn.")
+        x = x + ffn(centred(x, "l0.n2."), "l0.ffn.")
+    else:
+        x = centred(x + attention(x, "l0.attn."), "l0.n1.")
+        x = centred(x + ffn(x, "l0.ffn."), "l0.n2.")
+    x = x + attention(rms(x, "l1.n1."), "l1.attn.")
+    x = x + ffn(rms(x, "l1.n2."), "l1.ffn.")
+    return centred(x, "final.") @ w["head.weight"].T
+
+
+def test_toy_architecture_with_a_norm_and_an_arrangement_of_its_own(ops):
+    register_part("norm", "test_centred_norm", CentredNorm)
+    register_part("block", "test_postnorm_residual", PostNormResidual)
+    register_architecture("PostNormToyForCausalLM", PostNormToyConfig)
+    from distie_amd.config import config_from_dict
+
+    cfg = config_from_dict({"architectures": ["PostNormToyForCausalLM"], "hidden": 48, "vocab": 77, "heads": 3, "eps": 1e-4})
+    model = Model(cfg.model_spec())
+    specs = model.param_specs()
+    assert {"l0.n1.bias", "l0.n2.weight", "final.bias", "l1.n1.weight"} <= set(specs) and "l1.n1.bias" not in specs
+    gen = torch.Generator().manual_seed(21)
+    weights = {n: (torch.ones(s.shape) + 0.2 * torch.randn(s.shape, generator=gen) if s.init == "ones"
+                   else torch.randn(s.shape, generator=gen) * 0.25) for n, s in specs.items()}
+    model.load_tensors(lambda name: weights[name].to(ops.device))
+    cache = CacheManager(model.cache_requirements(), 4, 32, 4, device=ops.device, dtype=torch.float32)
+    runner = ModelRunner(model, cache, ops, torch.float32, 64)
+    a = torch.randint(0, 77, (23,), generator=gen).tolist()
+    b = torch.randint(0, 77, (9,), generator=gen).tolist()
+    want_a, want_b = postnorm_toy_plain(weights, cfg, a), postnorm_toy_plain(weights, cfg, b)
+    # the pin of the plain side: the other arrangement of the same parts gives other logits
+    assert (postnorm_toy_plain(weights, cfg, a, norm_first=True) - want_a).abs().max() > 1e-2
+    got = runner.step([StepEntry("a", a, list(range(23)))]).cpu()
+    assert (got - want_a.float()).abs().max() < 1e-4
+    runner.finish("a")
+    rows = {"a": [], "b": []}
+    seqs = {"a": a, "b": b}
+    for step in [[("a", 0, 5)], [("a", 5, 7), ("b", 0, 3)], [("a", 7, 22), ("b", 3, 4)], [("b", 4, 9), ("a", 22, 23)]]:
         logits = runner.step([StepEntry(r, seqs[r][lo:hi], list(range(hi - lo))) for r, lo, hi in step]).cpu()
         at = 0
         for r, lo, hi in step:
