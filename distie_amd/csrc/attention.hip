@@ -562,15 +562,24 @@ extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, c
 //    [64, D] and the V^T tile [D, 64] are put into LDS once per workgroup (global loads of the next tile
 //    are in flight while the current one is used) and every wave multiplies its own 16 * PF_MB query
 //    columns against them with the same two products and the same register layout as attn_decode.
+//    The kernel is bound by its reads from LDS (every wave reads the whole tile): two blocks of columns
+//    per wave halve them per product, for the registers of head sizes up to 128 (with one tile of loads in
+//    flight instead of two; at 32,768 keys 570 instead of 850 us for 2,048 tokens of 12 heads).
 //    Requests that bring fewer than `min_q_len` tokens are left to the decode kernel.
 // ===================================================================================================
 constexpr int PF_BN = 64;                               // keys per tile
 constexpr int PF_WAVES = 4;
 constexpr int PF_THREADS = PF_WAVES * DISTIE_WAVE;
-constexpr int PF_MB = 1;                                // blocks of 16 query columns per wave
+#ifndef DISTIE_PF_MB
+#define DISTIE_PF_MB ((D <= 128) ? 2 : 1)
+#endif
+#ifndef DISTIE_PF_DEPTH
+#define DISTIE_PF_DEPTH ((DISTIE_PF_MB == 2) ? 1 : 2)
+#endif
+constexpr int PF_MB = DISTIE_PF_MB;                     // blocks of 16 query columns per wave
 constexpr int PF_WAVE_COLS = 16 * PF_MB;
 constexpr int PF_BM = PF_WAVES * PF_WAVE_COLS;          // query tokens per workgroup
-constexpr int PF_DEPTH = 2;                             // key tiles whose loads are in flight
+constexpr int PF_DEPTH = DISTIE_PF_DEPTH;                             // key tiles whose loads are in flight
 // Rows of K in LDS, in elements. Lane (r, g) reads 16 bytes at row r, byte 16 g (+ a constant): that is free
 // of bank conflicts when the row stride is 32 bytes more than a multiple of 64 (measured with the LDS
 // conflict counter: 16 or 48 bytes more cost every read twice).
@@ -589,7 +598,7 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
   __shared__ __attribute__((aligned(16))) bf16_t k_lds[PF_BN * PF_K_STRIDE];
   __shared__ __attribute__((aligned(16))) bf16_t v_lds[D * PF_V_STRIDE];
   const int tid = threadIdx.x;
-  const int wave = tid / DISTIE_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / DISTIE_WAVE);   // uniform: what depends on it alone stays scalar
   const int lane = tid % DISTIE_WAVE;
   const int r = lane % 16;
   const int g = lane / 16;
@@ -653,12 +662,19 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
   // Every lane issues the same loads for every tile, with no branch around them: a block that belongs to no
   // page reads the start of the cache instead and is cleared when it is stored.
   auto block_live = [&](int key) { return key <= key_end && key + 15 >= key_begin; };
-  auto fetch = [&](int k0, uint4 (&k_stage)[PF_PASSES], uint4 (&v_stage)[PF_PASSES]) {
+  // The page of a block is looked up two tiles before its keys are asked for (a scalar load, the block being
+  // the same for the whole wave): asked for together, every tile would cost the wave two trips to memory
+  // one after the other.
+  auto lookup = [&](int k0) {
+    const int key = k0 + 16 * wave;
+    const int slot = block_shift >= 0 ? key >> block_shift : key / block_size;
+    return table[min(slot, table_width - 1)];
+  };
+  auto fetch = [&](int k0, int page_of_block, uint4 (&k_stage)[PF_PASSES], uint4 (&v_stage)[PF_PASSES]) {
     const int key = k0 + 16 * wave;
     const bool live = block_live(key);
-    const int slot = block_shift >= 0 ? key >> block_shift : key / block_size;
     const int offset = live ? (block_shift >= 0 ? key & (block_size - 1) : key % block_size) : 0;
-    const int page = live ? table[slot] : 0;
+    const int page = live ? page_of_block : 0;
     const int64_t base = live ? (static_cast<int64_t>(page) * kv_heads + kh) * block_size * D : 0;
     const bf16_t* k_block = k_cache + base + static_cast<int64_t>(offset) * D;
     const bf16_t* v_block = v_cache + base + offset;
@@ -805,8 +821,17 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
   const int per_split = (all_tiles + gridDim.z - 1) / gridDim.z;
   const int tile0 = all_tile0 + static_cast<int>(blockIdx.z) * per_split * PF_BN;
   const int loop_end = min(key_end, tile0 + per_split * PF_BN - 1);            // last key of this workgroup's walk
+  int pages_ahead[PF_DEPTH];
+  {
+    int first_pages[PF_DEPTH];
 #pragma unroll
-  for (int d = 0; d < PF_DEPTH; ++d) fetch(tile0 + d * PF_BN, k_stages[d], v_stages[d]);
+    for (int d = 0; d < PF_DEPTH; ++d) first_pages[d] = lookup(tile0 + d * PF_BN);
+#pragma unroll
+    for (int d = 0; d < PF_DEPTH; ++d) {
+      fetch(tile0 + d * PF_BN, first_pages[d], k_stages[d], v_stages[d]);
+      pages_ahead[d] = lookup(tile0 + (PF_DEPTH + d) * PF_BN);
+    }
+  }
   for (int k0 = tile0; k0 <= loop_end; k0 += PF_DEPTH * PF_BN) {
 #pragma unroll
     for (int d = 0; d < PF_DEPTH; ++d) {
@@ -815,7 +840,8 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
       __syncthreads();                       // every wave is done with the tile in LDS
       stash(k, k_stages[d], v_stages[d]);
       __syncthreads();
-      fetch(k + PF_DEPTH * PF_BN, k_stages[d], v_stages[d]);
+      fetch(k + PF_DEPTH * PF_BN, pages_ahead[d], k_stages[d], v_stages[d]);
+      pages_ahead[d] = lookup(k + 2 * PF_DEPTH * PF_BN);
       compute(k);
     }
   }
@@ -855,7 +881,7 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
 
 // Combines the `splits` parts of attn_prefill_kernel with gridDim.z > 1, in order: one block per token; tokens
 // of requests that the kernel skipped (fewer than min_q_len tokens) are skipped here as well.
-constexpr int PF_MAX_SPLITS = 8;
+constexpr int PF_MAX_SPLITS = 16;
 
 __global__ void attn_prefill_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                           const int32_t* __restrict__ token_request, const int32_t* __restrict__ cu_q,

@@ -78,10 +78,10 @@ class HipOps(Ops):
     # or, for a weight of at most this many elements (too few row blocks to occupy the chip that way),
     # through the one-wave kernel once per 16 rows of x
     ROW_GROUPS_MAX_ELEMENTS = 4 << 20
-    # attention over a portion of a prompt: from PREFILL_SPLIT_KEYS visible keys on, the walk over the keys
-    # is cut in two parts (three from four times as many, four from six times; measured: 2 beat 3 at 2,048)
-    PREFILL_SPLIT_KEYS = 1024
-    PREFILL_MAX_SPLITS = 4
+    # attention over a portion of a prompt: from so many visible keys on, the walk over the keys is cut into so
+    # many parts that run side by side (measured at 12 heads of 128, 2,048 new tokens: 3 parts are best up to
+    # 4,096 keys, 5 at 8,192, 8 from 16,384 on; the kernel takes up to 16)
+    PREFILL_PARTS = ((1024, 3), (8192, 5), (16384, 8))
     # decode attention cuts the keys into runs so that about DECODE_WAVES waves are at work, with at most
     # DECODE_MAX_RUNS places for partial results per request and head
     DECODE_WAVES = 1024
@@ -487,9 +487,11 @@ class HipOps(Ops):
             if singles < meta.num_requests or not split_decode:
                 # portions of prompts (and single tokens too, if the decode kernel did not take them). Long
                 # walks over the keys are cut into parts that run side by side.
+                visible = min(meta.max_kv, int(window) + 128) if window else meta.max_kv
                 parts = 1
-                if meta.max_kv >= self.PREFILL_SPLIT_KEYS:
-                    parts = max(2, min(self.PREFILL_MAX_SPLITS, 1 + meta.max_kv // (2 * self.PREFILL_SPLIT_KEYS)))
+                for keys, cut in self.PREFILL_PARTS:
+                    if visible >= keys:
+                        parts = cut
                 part_o = part_ml = None
                 if parts > 1:
                     part_o = torch.empty((parts, T, num_heads, head_dim), dtype=torch.float32, device=self.device)

@@ -376,18 +376,15 @@ def test_paged_attention_long_portions(ops, dtype, heads, kv_heads, dim, P, wind
 
 @pytest.mark.parametrize("heads,kv_heads,dim,P,window", [(4, 2, 16, 16, None), (12, 2, 128, 16, None), (3, 1, 48, 16, 700),
                                                          (2, 1, 256, 32, 100), (6, 2, 64, 64, None)])
-@pytest.mark.parametrize("parts", [2, 3, 4])
+@pytest.mark.parametrize("parts", [2, 3, 5, 8, 16])
 def test_paged_attention_keys_walked_in_parts(ops, heads, kv_heads, dim, P, window, parts, monkeypatch):
-    """From 1,024 visible keys on, the tiled kernel cuts the walk over the keys in two and merges: a long
+    """From 1,024 visible keys on, the tiled kernel cuts the walk over the keys into parts and merges: a long
     portion without a past, one that starts in the middle of a tile after a long past, a short one, a
     two-token one, and single tokens (which the decode kernel takes, or the tiled kernel too)."""
     dtype = torch.bfloat16
     lens, q_lens = [1300, 1500, 90, 777, 40, 1100], [1300, 100, 90, 1, 2, 1]
     meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, lens, q_lens, dtype, seed=5)
-    assert meta.max_kv >= ops.PREFILL_SPLIT_KEYS
-    if parts > 2:       # as a longer context would have it
-        monkeypatch.setattr(type(ops), "PREFILL_SPLIT_KEYS", meta.max_kv // (2 * (parts - 1)))
-        assert 1 + meta.max_kv // (2 * ops.PREFILL_SPLIT_KEYS) == parts
+    monkeypatch.setattr(type(ops), "PREFILL_PARTS", ((64, parts),))      # as a longer context would have it
     want = TorchOps("cuda").paged_attention(qkv.double(), meta, 0, k.double(), v.double(), heads, kv_heads, dim,
                                             dim ** -0.5, window)
     got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
@@ -396,7 +393,7 @@ def test_paged_attention_keys_walked_in_parts(ops, heads, kv_heads, dim, P, wind
     got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
     close(got, want, dtype, scale=want.abs().max().item())
     # in one walk, the same within rounding
-    monkeypatch.setattr(type(ops), "PREFILL_SPLIT_KEYS", 1 << 30)
+    monkeypatch.setattr(type(ops), "PREFILL_PARTS", ())
     whole = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
     close(whole, want, dtype, scale=want.abs().max().item())
 
