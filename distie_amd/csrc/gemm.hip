@@ -16,6 +16,7 @@
 // 231-233, 301); bfloat16 products of more than 64 rows (prefill) are left to the library here as well.
 
 #include "common.h"
+#include <algorithm>
 
 // ---------------------------------------------------------------- generic
 #define GT 64   // tile of M and of N
@@ -541,8 +542,16 @@ template <typename Y, int MODE, int MB>
 __global__ __launch_bounds__(256, 2) void gemm_packed_wide_kernel(const bf16_t* __restrict__ x,
                                                                const bf16_t* __restrict__ w,
                                                                const float* __restrict__ bias, Y* __restrict__ y,
-                                                               int M, int N, int K, int row_blocks, int tiles_per_slice) {
+                                                               int M, int N, int K, int row_blocks, int tiles_per_slice,
+                                                               int m_group) {
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][MB * 16][WD_XROW];
+  // blockIdx.z: a group of m_group rows of x. The groups run one after the other over the whole weight, so
+  // the second reads it from the memory-side cache (if it fits there; the launcher decides).
+  const int m_all = M;
+  const int m0 = blockIdx.z * m_group;
+  x += static_cast<int64_t>(m0) * K;
+  y += static_cast<int64_t>(m0) * (MODE == PK_GATED ? N / 2 : N);
+  M = min(m_group, M - m0);
   const int tid = threadIdx.x;
   const int lane = tid % 64;
   const int wave = tid / 64;
@@ -653,7 +662,7 @@ __global__ __launch_bounds__(256, 2) void gemm_packed_wide_kernel(const bf16_t* 
           if (n0 + i < half) y[static_cast<int64_t>(m) * half + n0 + i] = from_float<Y>(v[i]);
       }
     } else {
-      Y* out = y + static_cast<int64_t>(blockIdx.y) * M * N;
+      Y* out = y + static_cast<int64_t>(blockIdx.y) * m_all * N;
       const bool with_bias = bias != nullptr && blockIdx.y == 0;
       if (m < M) {
 #pragma unroll
@@ -687,16 +696,22 @@ extern "C" int distie_gemm_packed_wide_slices(int N, int K) {
 // 17 to 64 rows of x. mode 0: y [M, N] of y_dtype, or float32 [slices, M, N] when the plan cuts K
 // (distie_gemm_packed_wide_slices); 1 (gated): [M, N / 2].
 static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bias, void* y, int y_dtype, int M, int N,
-                              int K, int mode, hipStream_t stream) {
+                              int K, int mode, int two_pass, hipStream_t stream) {
   const int row_blocks = mode == PK_GATED ? (N / 2 + 7) / 8 : (N + 15) / 16;
   int slices = 1, tiles_per_slice = 4 * ((K + SK_KSTEP - 1) / SK_KSTEP);
   if (mode == PK_PLAIN) wide_plan(row_blocks, K, &slices, &tiles_per_slice);
   if (slices > 1 && y_dtype != DISTIE_F32) return DISTIE_BAD_ARGUMENT;
-  dim3 grid((row_blocks + 3) / 4, slices);
-  const int mb = (M + 15) / 16;
+  // two_pass: more than 32 rows of x are taken in two passes of 32 rows over the weight, with twice the
+  // workgroups and half the registers and LDS each; worth it if the weight fits the memory-side cache, from
+  // which the second pass then reads it (measured at 64 rows, cold: down 19.1 -> 16.1 us, gate+up 33.3 ->
+  // 26.2 us; a weight of 270 MB gets slower, being fetched from memory twice).
+  const int m_group = (M > 32 && two_pass) ? 32 : 64;
+  const int groups = (M + m_group - 1) / m_group;
+  dim3 grid((row_blocks + 3) / 4, slices, groups);
+  const int mb = (std::min(M, m_group) + 15) / 16;
 #define WIDE(MODE, MB)                                                                                   \
   DISTIE_DISPATCH(y_dtype, Y, (gemm_packed_wide_kernel<Y, MODE, MB><<<grid, 256, 0, stream>>>(           \
-                                  x, w, bias, static_cast<Y*>(y), M, N, K, row_blocks, tiles_per_slice)))
+                                  x, w, bias, static_cast<Y*>(y), M, N, K, row_blocks, tiles_per_slice, m_group)))
 #define WIDE_MB(MODE)                    \
   switch (mb) {                          \
     case 1: WIDE(MODE, 1); break;        \
@@ -715,11 +730,12 @@ static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bia
 }
 
 extern "C" int distie_gemm_packed_wide_bf16(const void* x, const void* w_packed, const float* bias, void* y,
-                                            int y_dtype, int M, int N, int K, int gated, hipStream_t stream) {
+                                            int y_dtype, int M, int N, int K, int gated, int two_pass,
+                                            hipStream_t stream) {
   if (M <= 0) return 0;
   if (M > 64 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
   return packed_wide_launch(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w_packed), bias, y, y_dtype, M, N,
-                            K, gated ? PK_GATED : PK_PLAIN, stream);
+                            K, gated ? PK_GATED : PK_PLAIN, two_pass, stream);
 }
 
 // The stacked q/k/v product with the rotation and the cache write in its epilogue. w_packed: the ROTARY

@@ -78,6 +78,9 @@ class HipOps(Ops):
     # or, for a weight of at most this many elements (too few row blocks to occupy the chip that way),
     # through the one-wave kernel once per 16 rows of x
     ROW_GROUPS_MAX_ELEMENTS = 4 << 20
+    # ... and that kernel takes more than 32 rows in two passes of 32 over a weight of at most this many elements
+    # (144 MB: the second pass reads it from the memory-side cache; larger ones would come from memory twice)
+    TWO_PASS_MAX_ELEMENTS = 72 << 20
     # attention over a portion of a prompt: from so many visible keys on, the walk over the keys is cut into so
     # many parts that run side by side (measured at 12 heads of 128, 2,048 new tokens: 3 parts are best up to
     # 4,096 keys, 5 at 8,192, 8 from 16,384 on; the kernel takes up to 16)
@@ -120,7 +123,7 @@ class HipOps(Ops):
         o.distie_gemm_skinny_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _P]
         o.distie_pack_rows.argtypes = [_P, _P, _P, _I, _I, _P]
         o.distie_gemm_packed_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
-        o.distie_gemm_packed_wide_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
+        o.distie_gemm_packed_wide_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
         o.distie_gemm_packed_wide_slices.argtypes = [_I, _I]
         o.distie_gemm_packed_rotary_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         o.distie_argmax.argtypes = [_P, _P, _I, _I, _P, _P, _P]
@@ -298,9 +301,13 @@ class HipOps(Ops):
         if packed.numel() != self._packed_elements(N, K, True):
             raise KernelError("linear_silu_mul: the packed copy does not belong to this weight")
         out = torch.empty((M, N // 2), dtype=x.dtype, device=self.device)
-        kernel = self._ops.distie_gemm_packed_bf16 if M <= self.SKINNY_MAX_ROWS else self._ops.distie_gemm_packed_wide_bf16
-        _check(kernel(x.data_ptr(), packed.data_ptr(), None, out.data_ptr(), _code(out), M, N, K, 1, self._stream()),
-               "gemm_packed_bf16")
+        if M <= self.SKINNY_MAX_ROWS:
+            _check(self._ops.distie_gemm_packed_bf16(x.data_ptr(), packed.data_ptr(), None, out.data_ptr(), _code(out),
+                                                     M, N, K, 1, self._stream()), "gemm_packed_bf16")
+        else:
+            _check(self._ops.distie_gemm_packed_wide_bf16(
+                x.data_ptr(), packed.data_ptr(), None, out.data_ptr(), _code(out), M, N, K, 1,
+                1 if N * K <= self.TWO_PASS_MAX_ELEMENTS else 0, self._stream()), "gemm_packed_wide_bf16")
         return out
 
     def linear_rope_kv_write(self, x, weight, bias, meta, group, k_cache, v_cache, inv_freq, num_heads, num_kv_heads,
@@ -370,7 +377,8 @@ class HipOps(Ops):
                 out = torch.empty((slices, M, N), dtype=torch.float32, device=self.device)
             _check(self._ops.distie_gemm_packed_wide_bf16(
                 x.data_ptr(), packed.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(),
-                _code(out), M, N, K, 0, self._stream()), "gemm_packed_wide_bf16")
+                _code(out), M, N, K, 0, 1 if N * K <= self.TWO_PASS_MAX_ELEMENTS else 0, self._stream()),
+                "gemm_packed_wide_bf16")
             if slices == 1:
                 return out
             return PartialSums(out, out_dtype) if partial_ok else self.dense(PartialSums(out, out_dtype))

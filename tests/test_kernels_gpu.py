@@ -126,10 +126,11 @@ def test_gemm_packed_bf16(ops, M, N, K):
     close(got, want, torch.float32, scale=5 * want.abs().max().item())
     # 17 to 64 rows: small weights go through the one-wave kernel once per 16 rows, large ones through
     # the kernel that shares x in LDS; both are run for every shape
-    routes = [ops.ROW_GROUPS_MAX_ELEMENTS] if M <= 16 else [0, 1 << 40]
+    # (and that one takes more than 32 rows in one pass or in two, by the weight's size)
+    routes = [(ops.ROW_GROUPS_MAX_ELEMENTS, ops.TWO_PASS_MAX_ELEMENTS)] if M <= 16 else [(0, 0), (0, 1 << 40), (1 << 40, 0)]
     try:
-        for limit in routes:
-            ops.ROW_GROUPS_MAX_ELEMENTS = limit
+        for limit, two_pass in routes:
+            ops.ROW_GROUPS_MAX_ELEMENTS, ops.TWO_PASS_MAX_ELEMENTS = limit, two_pass
             part = ops.linear(x, w, b)
             if M <= 16 or limit > 0:
                 assert isinstance(part, PartialSums) == (K >= 768)
@@ -139,7 +140,7 @@ def test_gemm_packed_bf16(ops, M, N, K):
             # the packed and the natural kernel add the same products in another order: float32 rounding only
             assert (got.float() - natural).abs().max().item() <= 2 ** -7 * want.abs().max().item()
     finally:
-        del ops.ROW_GROUPS_MAX_ELEMENTS
+        del ops.ROW_GROUPS_MAX_ELEMENTS, ops.TWO_PASS_MAX_ELEMENTS
     assert ops.ROW_GROUPS_MAX_ELEMENTS == type(ops).ROW_GROUPS_MAX_ELEMENTS
 
 
@@ -156,9 +157,14 @@ def test_linear_silu_mul_fused(ops, M, I, K):
     close(unfused, want, torch.bfloat16, scale=2 * want.abs().max().item())
     ops.prepare_linear(w, gated=True)
     assert w._distie_gated.numel() == -(-I // 8) * -(-K // 32) * 512
-    got = ops.linear_silu_mul(x, w)
-    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (M, I)
-    close(got, want, torch.bfloat16, scale=want.abs().max().item())
+    for two_pass in (1 << 40, 0):           # more than 32 rows in two passes over the weight, or in one
+        ops.TWO_PASS_MAX_ELEMENTS = two_pass
+        try:
+            got = ops.linear_silu_mul(x, w)
+        finally:
+            del ops.TWO_PASS_MAX_ELEMENTS
+        assert got.dtype == torch.bfloat16 and tuple(got.shape) == (M, I)
+        close(got, want, torch.bfloat16, scale=want.abs().max().item())
     # more rows than the fused kernel takes: the unfused path, same result
     big = rand(70, K, dtype=torch.bfloat16, seed=2)
     gu = big.double() @ w.double().T
