@@ -696,16 +696,16 @@ extern "C" int distie_gemm_packed_wide_slices(int N, int K) {
 // 17 to 64 rows of x. mode 0: y [M, N] of y_dtype, or float32 [slices, M, N] when the plan cuts K
 // (distie_gemm_packed_wide_slices); 1 (gated): [M, N / 2].
 static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bias, void* y, int y_dtype, int M, int N,
-                              int K, int mode, int two_pass, hipStream_t stream) {
+                              int K, int mode, int pass_blocks, hipStream_t stream) {
   const int row_blocks = mode == PK_GATED ? (N / 2 + 7) / 8 : (N + 15) / 16;
   int slices = 1, tiles_per_slice = 4 * ((K + SK_KSTEP - 1) / SK_KSTEP);
   if (mode == PK_PLAIN) wide_plan(row_blocks, K, &slices, &tiles_per_slice);
   if (slices > 1 && y_dtype != DISTIE_F32) return DISTIE_BAD_ARGUMENT;
-  // two_pass: more than 32 rows of x are taken in two passes of 32 rows over the weight, with twice the
-  // workgroups and half the registers and LDS each; worth it if the weight fits the memory-side cache, from
-  // which the second pass then reads it (measured at 64 rows, cold: down 19.1 -> 16.1 us, gate+up 33.3 ->
-  // 26.2 us; a weight of 270 MB gets slower, being fetched from memory twice).
-  const int m_group = (M > 32 && two_pass) ? 32 : 64;
+  // pass_blocks: the rows of x are taken in passes of 16 * pass_blocks rows over the weight (0: all at once),
+  // with more workgroups and fewer registers and less LDS each; worth it if the weight fits the memory-side
+  // cache, from which the later passes then read it (measured at 64 rows in two passes, cold: down 18.3 ->
+  // 15.4 us, gate+up 22.4 -> 21.3 us; a weight of 270 MB gets slower, being fetched from memory twice).
+  const int m_group = (pass_blocks >= 1 && pass_blocks <= 4) ? 16 * pass_blocks : 64;
   const int groups = (M + m_group - 1) / m_group;
   dim3 grid((row_blocks + 3) / 4, slices, groups);
   const int mb = (std::min(M, m_group) + 15) / 16;
@@ -730,12 +730,12 @@ static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bia
 }
 
 extern "C" int distie_gemm_packed_wide_bf16(const void* x, const void* w_packed, const float* bias, void* y,
-                                            int y_dtype, int M, int N, int K, int gated, int two_pass,
+                                            int y_dtype, int M, int N, int K, int gated, int pass_blocks,
                                             hipStream_t stream) {
   if (M <= 0) return 0;
   if (M > 64 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
   return packed_wide_launch(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w_packed), bias, y, y_dtype, M, N,
-                            K, gated ? PK_GATED : PK_PLAIN, two_pass, stream);
+                            K, gated ? PK_GATED : PK_PLAIN, pass_blocks, stream);
 }
 
 // The stacked q/k/v product with the rotation and the cache write in its epilogue. w_packed: the ROTARY

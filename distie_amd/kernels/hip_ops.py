@@ -79,8 +79,8 @@ class HipOps(Ops):
     # through the one-wave kernel once per 16 rows of x
     ROW_GROUPS_MAX_ELEMENTS = 4 << 20
     # ... and that kernel takes more than 32 rows in two passes of 32 over a weight of at most this many elements
-    # (144 MB: the second pass reads it from the memory-side cache; larger ones would come from memory twice)
-    TWO_PASS_MAX_ELEMENTS = 72 << 20
+    # (64 MB: the second pass reads it from the memory-side cache; much larger ones would come from memory twice)
+    TWO_PASS_MAX_ELEMENTS = 32 << 20
     # attention over a portion of a prompt: from so many visible keys on, the walk over the keys is cut into so
     # many parts that run side by side (measured at 12 heads of 128, 2,048 new tokens: 3 parts are best up to
     # 4,096 keys, 5 at 8,192, 8 from 16,384 on; the kernel takes up to 16)
@@ -307,7 +307,7 @@ class HipOps(Ops):
         else:
             _check(self._ops.distie_gemm_packed_wide_bf16(
                 x.data_ptr(), packed.data_ptr(), None, out.data_ptr(), _code(out), M, N, K, 1,
-                1 if N * K <= self.TWO_PASS_MAX_ELEMENTS else 0, self._stream()), "gemm_packed_wide_bf16")
+                self._pass_blocks(M, N * K), self._stream()), "gemm_packed_wide_bf16")
         return out
 
     def linear_rope_kv_write(self, x, weight, bias, meta, group, k_cache, v_cache, inv_freq, num_heads, num_kv_heads,
@@ -341,6 +341,12 @@ class HipOps(Ops):
             table.data_ptr(), slots.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), M, K, num_heads,
             num_kv_heads, head_dim, meta.block_size, 1 if write else 0, self._stream()), "gemm_packed_rotary_bf16")
         return out
+
+    def _pass_blocks(self, rows: int, elements: int) -> int:
+        """Blocks of 16 rows of x per pass of the wide product over a weight of `elements` (0: one pass)."""
+        if elements > self.TWO_PASS_MAX_ELEMENTS:
+            return 0
+        return 2 if rows > 32 else 0
 
     def _rope_table(self, meta, inv_freq):
         """Cosines and sines of the step's positions, float32 [T, pairs, 2]: computed by the first layer
@@ -377,7 +383,7 @@ class HipOps(Ops):
                 out = torch.empty((slices, M, N), dtype=torch.float32, device=self.device)
             _check(self._ops.distie_gemm_packed_wide_bf16(
                 x.data_ptr(), packed.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(),
-                _code(out), M, N, K, 0, 1 if N * K <= self.TWO_PASS_MAX_ELEMENTS else 0, self._stream()),
+                _code(out), M, N, K, 0, self._pass_blocks(M, N * K), self._stream()),
                 "gemm_packed_wide_bf16")
             if slices == 1:
                 return out
