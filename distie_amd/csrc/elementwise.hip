@@ -165,7 +165,9 @@ static int rmsnorm_launch_out(float* residual, const D* delta, int slices, const
         aligned16(out)) {
       const int quads = width / 4;
       int threads = (quads + 63) / 64 * 64;
-      const int nv = threads > 1024 ? 2 : 1;
+      // two groups of four a thread for rows beyond 4,096 elements, and when one group a thread would make
+      // more waves than the chip holds at once (256 compute units x 32): the rows then fit in one round
+      const int nv = (threads > 1024 || (quads > 64 && static_cast<int64_t>(rows) * (threads / 64) > 8192)) ? 2 : 1;
       if (nv == 2) threads = ((quads + 1) / 2 + 63) / 64 * 64;
       if (nv == 1) {
         DISTIE_DISPATCH(out_dtype, O, (rmsnorm_vec_kernel<D, W, O, 1><<<rows, threads, 0, stream>>>(

@@ -43,16 +43,17 @@ def test_embed(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width", [40, 1000, 1002, 3000, 5000, 8200])
-def test_rmsnorm_and_fused_add(ops, dtype, width):
-    x = rand(7, width, seed=1, scale=3.0)
+@pytest.mark.parametrize("rows,width", [(7, 40), (7, 1000), (7, 1002), (7, 3000), (7, 5000), (7, 8200),
+                                        (2100, 1536), (5000, 332), (9000, 64)])     # many rows: two groups a thread
+def test_rmsnorm_and_fused_add(ops, dtype, rows, width):
+    x = rand(rows, width, seed=1, scale=3.0)
     w = rand(width, dtype=dtype, seed=2)
     eps = 1e-5
     want = x.double() * torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True) + eps) * w.double()
     got = ops.rmsnorm(x, w, eps, dtype)
     assert got.dtype == dtype
     close(got, want, dtype, scale=want.abs().max().item())
-    delta = rand(7, width, dtype=dtype, seed=3)
+    delta = rand(rows, width, dtype=dtype, seed=3)
     res = x.clone()
     got = ops.add_rmsnorm(res, delta, w, eps, dtype)
     s = x.double() + delta.double()
