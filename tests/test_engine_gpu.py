@@ -149,3 +149,41 @@ def test_a_file_in_32_bit_under_a_bfloat16_engine(tmp_path, ops):
     assert not hasattr(runner.model.blocks[0].mixer.qkv_weight, "_distie_rotary")
     ids = random_ids(cfg, 90, 8)
     check_logits(replay_cut(runner, "a", ids, [50, 20, 3]), weights, cfg, ids, torch.bfloat16, folder)
+
+
+def test_layer_sizes_of_the_1_5b_model(tmp_path, ops):
+    """Two layers with the sizes the benchmark runs (width 1,536, 12 heads over 2 kv heads of 128, feed-forward
+    8,960, vocabulary 151,936, tied head): sizes the tiny configurations do not reach (products cut along
+    8,960, rows of the head beyond 2^17, head size 128). One file in bfloat16 serves both engines, since the
+    float32 engine keeps every tensor in 32-bit whatever the file holds."""
+    cfg = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 2, "hidden_size": 1536,
+           "num_attention_heads": 12, "num_key_value_heads": 2, "head_dim": 128, "intermediate_size": 8960,
+           "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
+           "max_position_embeddings": 4096, "hidden_act": "silu"}
+    folder, weights = make_model_dir(tmp_path, cfg, seed=19, std=0.03, dtype=torch.bfloat16)
+    seqs = {"a": random_ids(cfg, 120, 1), "b": random_ids(cfg, 45, 2)}
+    want = {name: plain.forward(weights, cfg, ids, torch.float64).float() for name, ids in seqs.items()}
+    for dtype in (torch.float32, torch.bfloat16):
+        runner = build_runner(folder, ops, dtype, block_size=16, num_blocks=24, max_model_len=4096)
+        got = {name: [] for name in seqs}
+        # a whole, then: a portion of a beside all of b; the rest of a in a portion of 70 and single tokens,
+        # the first of them beside b's last token
+        whole = replay_whole(runner, "w", seqs["a"])
+        steps = [[("a", 0, 40), ("b", 0, 44)], [("a", 40, 110)], [("a", 110, 111), ("b", 44, 45)]] + \
+                [[("a", at, at + 1)] for at in range(111, 120)]
+        for step in steps:
+            logits = runner.step([StepEntry(r, seqs[r][lo:hi], list(range(hi - lo))) for r, lo, hi in step]).float().cpu()
+            at = 0
+            for r, lo, hi in step:
+                got[r].append(logits[at:at + hi - lo])
+                at += hi - lo
+        for name in seqs:
+            runner.finish(name)
+        runner.cache.check()
+        for name, rows in [("a", whole)] + [(n, torch.cat(g)) for n, g in got.items()]:
+            diff = rows - want[name]
+            scale = want[name].abs().max().item()
+            if dtype == torch.float32:
+                assert diff.abs().max().item() < 1e-4 * max(1.0, scale), (name, diff.abs().max().item(), scale)
+            else:
+                assert diff.abs().max().item() < scale / 16 and diff.pow(2).mean().sqrt().item() < scale / 64, name
