@@ -30,12 +30,19 @@ class StepEntry:
 
 
 class BatchBuilder:
+    STAGING_BUFFERS = 3
+
     def __init__(self, cache: CacheManager, max_model_len: int, device, vocab_size: int) -> None:
         self.cache = cache
         self.device = device
         self.vocab_size = vocab_size
         self.max_model_len = int(max_model_len)
         self.table_width = max(1, -(-self.max_model_len // cache.block_size))
+        # pinned staging buffers for the step descriptions, used in turn: [host tensor, its numpy view, event of
+        # the last copy out of it]. With them the copy to the device does not wait for the work queued before
+        # it, so the host can prepare a step while the one before still runs.
+        self._staging = [[None, None, None] for _ in range(self.STAGING_BUFFERS)]
+        self._next_staging = 0
 
     def layout(self, T: int, B: int, R: int):
         """Offsets of the fields inside the packed int32 buffer of a step with T tokens, B requests
@@ -146,7 +153,23 @@ class BatchBuilder:
         """-> (ids int32 [T], BatchMeta, want_rows int32 [R] or None), on the device, with one copy."""
         T = sum(len(e.tokens) for e in entries)
         R = sum(len(e.want) for e in entries)
-        host = np.empty(int(self.layout(T, len(entries), R)[-1]), dtype=np.int32)
-        offsets, T, B, R, max_q, max_kv, cu_q, past = self.fill(host, entries)
-        dev = torch.from_numpy(host).to(self.device, non_blocking=False)
+        words = int(self.layout(T, len(entries), R)[-1])
+        if torch.device(self.device).type != "cuda":
+            host = np.empty(words, dtype=np.int32)
+            offsets, T, B, R, max_q, max_kv, cu_q, past = self.fill(host, entries)
+            dev = torch.from_numpy(host).to(self.device)
+            return self.meta_of(dev, offsets, T, B, R, max_q, max_kv, cu_q, past)
+        slot = self._staging[self._next_staging]
+        self._next_staging = (self._next_staging + 1) % len(self._staging)
+        if slot[2] is not None:
+            slot[2].synchronize()                       # the copy made out of this buffer some steps ago is done
+        if slot[0] is None or slot[0].numel() < words:
+            slot[0] = torch.empty(max(words, 2 * (slot[0].numel() if slot[0] is not None else 0)), dtype=torch.int32,
+                                  pin_memory=True)
+            slot[1] = slot[0].numpy()
+            slot[2] = torch.cuda.Event()
+        offsets, T, B, R, max_q, max_kv, cu_q, past = self.fill(slot[1], entries)
+        dev = torch.empty(words, dtype=torch.int32, device=self.device)
+        dev.copy_(slot[0][:words], non_blocking=True)
+        slot[2].record()
         return self.meta_of(dev, offsets, T, B, R, max_q, max_kv, cu_q, past)

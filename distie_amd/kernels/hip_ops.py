@@ -481,7 +481,7 @@ class HipOps(Ops):
             if split_decode:
                 # requests that bring one token: keys are cut into runs, one wave each, so that the chip is
                 # filled even when few requests decode
-                runs = max(1, min(64, self.DECODE_WAVES // (singles * num_kv_heads)))
+                runs = max(1, min(self.DECODE_MAX_RUNS, self.DECODE_WAVES // (singles * num_kv_heads)))
                 # under a window only the runs that hold its keys do anything: cut by the window's length,
                 # but into no more than DECODE_MAX_RUNS places for partial results
                 visible = min(meta.max_kv, int(window)) if window else meta.max_kv
