@@ -7,13 +7,13 @@
 //    (v_mfma_f32_16x16x32_bf16): a wave owns 16 rows of W and a slice of K, reads W straight from
 //    memory into the A operand (every weight byte is read once), and the small x is the B operand.
 //    Slices of K are written side by side and added, in order, by the kernel that reads them.
-//  * pack_rows + gemm_packed (up to 16 rows of x) and gemm_packed_wide (17 to 64 rows): the same streaming on a
+//  * pack_rows + gemm_packed (up to 16 rows of x) and gemm_packed_wide (17 to 64 rows a pass): the same streaming on a
 //    second copy of W laid out tile by tile in the matrix cores' lane order, with epilogues that finish
 //    what follows the product (gated activation; bias, rotation and cache write of q/k/v). Described at
 //    their definitions.
 //
 // The reference leaves these products to a library (worker/src/inference/qwen2/model.py:149-152,
-// 231-233, 301); bfloat16 products of more than 64 rows (prefill) are left to the library here as well.
+// 231-233, 301); bfloat16 products of many rows (prefill) are left to the library here as well.
 
 #include "common.h"
 #include <algorithm>
@@ -504,11 +504,11 @@ static int packed_waves(int K) {
 
 // y: as distie_gemm_skinny_bf16 (the same cut along K: slices go to other workgroups, hence to other
 // compute units, which a product with few rows of W needs to pull its bytes fast enough);
-// gated: [M, N / 2] of y_dtype, never cut. Up to 64 rows of x, in groups of 16.
+// gated: [M, N / 2] of y_dtype, never cut. Up to 256 rows of x, in groups of 16.
 extern "C" int distie_gemm_packed_bf16(const void* x, const void* w_packed, const float* bias, void* y, int y_dtype,
                                        int M, int N, int K, int gated, hipStream_t stream) {
   if (M <= 0) return 0;
-  if (M > 64 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
+  if (M > 256 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
   int slices = 1, k_per_slice = (K + SK_KSTEP - 1) / SK_KSTEP * SK_KSTEP;
   if (!gated) skinny_plan(N, K, &slices, &k_per_slice);
   if (slices > 1 && y_dtype != DISTIE_F32) return DISTIE_BAD_ARGUMENT;
@@ -527,7 +527,7 @@ extern "C" int distie_gemm_packed_bf16(const void* x, const void* w_packed, cons
   return launch_status();
 }
 
-// ---------------------------------------------------------------- packed weights, 17 to 64 rows of x
+// ---------------------------------------------------------------- packed weights, 17 to 64 rows of x a pass
 // A workgroup of four waves owns four row blocks (one a wave) and one slice of K. Per k-step of 128 the
 // weights go straight into registers, four k-steps ahead; the x tile ([16 MB rows, 128 k], the same for
 // all four waves) is fetched four k-steps ahead as well, into registers, and put into LDS (two stages)
@@ -693,7 +693,7 @@ extern "C" int distie_gemm_packed_wide_slices(int N, int K) {
   return slices;
 }
 
-// 17 to 64 rows of x. mode 0: y [M, N] of y_dtype, or float32 [slices, M, N] when the plan cuts K
+// 17 to 256 rows of x, at most 64 a pass. mode 0: y [M, N] of y_dtype, or float32 [slices, M, N] when the plan cuts K
 // (distie_gemm_packed_wide_slices); 1 (gated): [M, N / 2].
 static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bias, void* y, int y_dtype, int M, int N,
                               int K, int mode, int pass_blocks, hipStream_t stream) {
@@ -733,21 +733,21 @@ extern "C" int distie_gemm_packed_wide_bf16(const void* x, const void* w_packed,
                                             int y_dtype, int M, int N, int K, int gated, int pass_blocks,
                                             hipStream_t stream) {
   if (M <= 0) return 0;
-  if (M > 64 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
+  if (M > 256 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
   return packed_wide_launch(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w_packed), bias, y, y_dtype, M, N,
                             K, gated ? PK_GATED : PK_PLAIN, pass_blocks, stream);
 }
 
 // The stacked q/k/v product with the rotation and the cache write in its epilogue. w_packed: the ROTARY
 // copy of the [(heads + 2 kv_heads) * dim, K] weight. y: bfloat16 [M, N], rotated. dim a multiple of 16;
-// table: [M, dim / 2] (cos, sin). Up to 64 rows of x, in groups of 16: a workgroup owns one row block of
+// table: [M, dim / 2] (cos, sin). Up to 256 rows of x, in groups of 16: a workgroup owns one row block of
 // one group, so that even this small weight is pulled by hundreds of workgroups.
 extern "C" int distie_gemm_packed_rotary_bf16(const void* x, const void* w_packed, const float* bias, void* y,
                                               const void* table, const int32_t* slots, void* k_cache, void* v_cache,
                                               int M, int K, int heads, int kv_heads, int dim, int block_size,
                                               int write, hipStream_t stream) {
   if (M <= 0) return 0;
-  if (M > 64 || K <= 0 || K % 8 != 0 || heads < 1 || kv_heads < 1 || dim < 16 || dim % 16 != 0 || block_size < 1 ||
+  if (M > 256 || K <= 0 || K % 8 != 0 || heads < 1 || kv_heads < 1 || dim < 16 || dim % 16 != 0 || block_size < 1 ||
       table == nullptr || (write && (slots == nullptr || k_cache == nullptr || v_cache == nullptr)))
     return DISTIE_BAD_ARGUMENT;
   const int N = (heads + 2 * kv_heads) * dim;
