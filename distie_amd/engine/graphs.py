@@ -149,7 +149,11 @@ class DecodeGraphs:
         runner = self.runner
         n = bucket.size
         ids, meta, want = runner.builder.meta_of(bucket.dev, bucket.offsets, n, n, n, 1, limit)
-        return runner.model.forward(runner.ops, ids, meta, runner.cache, runner.act_dtype, want)
+        runner.ops.captured = True
+        try:
+            return runner.model.forward(runner.ops, ids, meta, runner.cache, runner.act_dtype, want)
+        finally:
+            runner.ops.captured = False
 
     def _capture(self, bucket: _Bucket, limit: int) -> torch.Tensor:
         # one ordinary run first: sizes scratch buffers and writes this step's keys and values

@@ -72,10 +72,14 @@ class HipOps(Ops):
     # bfloat16 products by rows of x: up to SKINNY_MAX_ROWS the weights are streamed by one wave per block
     # of 16 weight rows, x straight from memory (above that, the library's tiles are faster);
     SKINNY_MAX_ROWS = 16
-    # with a packed copy of the weight, up to PACKED_MAX_ROWS rows (in passes of at most 64; measured in the decode
-    # step: 9 % faster than the library at 72 rows, 5 % at 96, 4 % slower at 128) go through the kernel that shares the
-    # x tile of a workgroup in LDS,
+    # with a packed copy of the weight, more rows go through the kernel that shares the x tile of a workgroup in
+    # LDS, in passes of at most 64: up to PACKED_MAX_ROWS in a captured step (measured in the decode step: 9 %
+    # faster than the library at 72 rows, 5 % at 96, 4 % slower at 128), and up to PACKED_MAX_ROWS_EAGER in a step
+    # that is launched kernel by kernel, which the host bounds at these sizes: the library's products cost it
+    # 18 us each and the activation and rotation kernels beside them more launches (a prompt of 128 tokens:
+    # 2.7 instead of 3.9 ms, of 192: 3.5 instead of 3.9 ms, of 256: 4.3 instead of 3.9 ms),
     PACKED_MAX_ROWS = 96
+    PACKED_MAX_ROWS_EAGER = 192
     # or, for a weight of at most this many elements (too few row blocks to occupy the chip that way),
     # through the one-wave kernel once per 16 rows of x
     ROW_GROUPS_MAX_ELEMENTS = 4 << 20
@@ -93,7 +97,7 @@ class HipOps(Ops):
 
     def __init__(self, device="cuda:0", packed_weights: bool = True) -> None:
         """`packed_weights`: keep a second copy of every bfloat16 weight in the order in which the
-        matrix cores take it, for products with at most `PACKED_MAX_ROWS` rows (decode). It doubles
+        matrix cores take it, for products with at most `PACKED_MAX_ROWS_EAGER` rows (decode, short portions). It doubles
         the memory of the weights and makes those products 15-25 % faster, and it is what the fused
         epilogues (activation, rotation and cache write) work on; without it products of up to
         `SKINNY_MAX_ROWS` rows stream the weights as they are stored and larger ones go to the library."""
@@ -134,7 +138,8 @@ class HipOps(Ops):
     def tune_library_products(self, on: bool) -> None:
         """While on, the library times its candidate kernels for every new shape of a large product and
         keeps the fastest; afterwards it uses what it found (its own choice for shapes it has not
-        seen). Products of up to `PACKED_MAX_ROWS` rows do not go to the library at all."""
+        seen). Products of up to `PACKED_MAX_ROWS` rows do not go to the library at all (`PACKED_MAX_ROWS_EAGER`
+        outside captured steps)."""
         import os
         import tempfile
 
@@ -292,7 +297,7 @@ class HipOps(Ops):
     def linear_silu_mul(self, x, gate_up_weight):
         packed = getattr(gate_up_weight, "_distie_gated", None)
         x = self.dense(x)
-        if packed is None or x.dtype != torch.bfloat16 or x.shape[0] > self.PACKED_MAX_ROWS:
+        if packed is None or x.dtype != torch.bfloat16 or x.shape[0] > self._packed_rows():
             return self.silu_mul(self.linear(x, gate_up_weight))
         self._own(x)
         M, K = x.shape
@@ -316,7 +321,7 @@ class HipOps(Ops):
         held = getattr(weight, "_distie_rotary", None)
         x = self.dense(x)
         fused = held is not None and held[1] == (num_heads, num_kv_heads, head_dim) and \
-            x.dtype == torch.bfloat16 and x.shape[0] <= self.PACKED_MAX_ROWS and \
+            x.dtype == torch.bfloat16 and x.shape[0] <= self._packed_rows() and \
             inv_freq is not None and 2 * inv_freq.shape[0] == head_dim and k_cache.dtype == torch.bfloat16
         if not fused:
             return self.rope_kv_write(self.linear(x, weight, bias), meta, group, k_cache, v_cache, inv_freq,
@@ -342,6 +347,9 @@ class HipOps(Ops):
             table.data_ptr(), slots.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), M, K, num_heads,
             num_kv_heads, head_dim, meta.block_size, 1 if write else 0, self._stream()), "gemm_packed_rotary_bf16")
         return out
+
+    def _packed_rows(self) -> int:
+        return self.PACKED_MAX_ROWS if self.captured else self.PACKED_MAX_ROWS_EAGER
 
     def _pass_blocks(self, rows: int, elements: int) -> int:
         """Blocks of 16 rows of x per pass of the wide product over a weight of `elements` (0: one pass)."""
@@ -373,7 +381,7 @@ class HipOps(Ops):
             raise KernelError("linear: bias must be float32 [N]")
         both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
         packed = getattr(weight, "_distie_packed", None) if both_bf16 else None
-        if packed is not None and self.SKINNY_MAX_ROWS < M <= self.PACKED_MAX_ROWS and K % 8 == 0 and \
+        if packed is not None and self.SKINNY_MAX_ROWS < M <= self._packed_rows() and K % 8 == 0 and \
                 N * K > self.ROW_GROUPS_MAX_ELEMENTS:
             if packed.numel() != self._packed_elements(N, K, False):
                 raise KernelError("linear: the packed copy does not belong to this weight")
@@ -389,7 +397,7 @@ class HipOps(Ops):
             if slices == 1:
                 return out
             return PartialSums(out, out_dtype) if partial_ok else self.dense(PartialSums(out, out_dtype))
-        if both_bf16 and K % 8 == 0 and (M <= self.SKINNY_MAX_ROWS or (packed is not None and M <= self.PACKED_MAX_ROWS)):
+        if both_bf16 and K % 8 == 0 and (M <= self.SKINNY_MAX_ROWS or (packed is not None and M <= self._packed_rows())):
             if packed is not None:
                 if packed.numel() != self._packed_elements(N, K, False):
                     raise KernelError("linear: the packed copy does not belong to this weight")

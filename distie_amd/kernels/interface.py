@@ -54,6 +54,9 @@ class BatchMeta:
 
 class Ops(abc.ABC):
     device: torch.device
+    # True while the engine warms or records a captured step: launches then cost the host nothing when the
+    # step is replayed, so an implementation may choose kernels by their time on the device alone
+    captured: bool = False
 
     @abc.abstractmethod
     def embed(self, ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
