@@ -77,9 +77,9 @@ class HipOps(Ops):
     # faster than the library at 72 rows, 5 % at 96, 4 % slower at 128), and up to PACKED_MAX_ROWS_EAGER in a step
     # that is launched kernel by kernel, which the host bounds at these sizes: the library's products cost it
     # 18 us each and the activation and rotation kernels beside them more launches (a prompt of 128 tokens:
-    # 2.7 instead of 3.9 ms, of 192: 3.5 instead of 3.9 ms, of 256: 4.3 instead of 3.9 ms),
+    # 2.7 instead of 3.9 ms, of 192: 3.3, of 224: 3.8, of 256: 4.1 instead of 3.9 ms),
     PACKED_MAX_ROWS = 96
-    PACKED_MAX_ROWS_EAGER = 192
+    PACKED_MAX_ROWS_EAGER = 224
     # or, for a weight of at most this many elements (too few row blocks to occupy the chip that way),
     # through the one-wave kernel once per 16 rows of x
     ROW_GROUPS_MAX_ELEMENTS = 4 << 20
@@ -355,7 +355,8 @@ class HipOps(Ops):
         """Blocks of 16 rows of x per pass of the wide product over a weight of `elements` (0: one pass)."""
         if elements > self.TWO_PASS_MAX_ELEMENTS:
             return 0 if rows <= 64 else 4
-        return 2 if rows > 32 else 0        # (a single pass takes at most 64 rows)
+        # (a single pass takes at most 64 rows; beyond 128 rows passes of 48 were 5 % faster than of 32 or 64)
+        return 0 if rows <= 32 else (2 if rows <= 128 else 3)
 
     def _rope_table(self, meta, inv_freq):
         """Cosines and sines of the step's positions, float32 [T, pairs, 2]: computed by the first layer

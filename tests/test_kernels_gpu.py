@@ -111,7 +111,7 @@ def test_gemm_skinny_bf16(ops, M, N, K):
     close(got, want + b.double(), torch.bfloat16, scale=want.abs().max().item())
 
 
-@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 50, 64, 65, 96, 130, 192])
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 50, 64, 65, 96, 130, 224])
 @pytest.mark.parametrize("N,K", [(48, 128), (100, 264), (1536, 1536), (333, 8960), (2050, 72), (16, 8), (7, 40)])
 def test_gemm_packed_bf16(ops, M, N, K):
     """The same products through the weight's packed copy (what `prepare_linear` leaves): rows and
@@ -146,7 +146,7 @@ def test_gemm_packed_bf16(ops, M, N, K):
 
 
 def test_fewer_rows_through_the_packed_kernels_in_a_captured_step(ops):
-    """Launched kernel by kernel, a step of up to 192 tokens is bound by the host and takes the packed
+    """Launched kernel by kernel, a step of up to 224 tokens is bound by the host and takes the packed
     kernels with their fused epilogues; in a captured step only up to 96 rows do, the library's products
     being faster on the device beyond."""
     from distie_amd.kernels.hip_ops import PartialSums
@@ -190,13 +190,13 @@ def test_linear_silu_mul_fused(ops, M, I, K):
         assert got.dtype == torch.bfloat16 and tuple(got.shape) == (M, I)
         close(got, want, torch.bfloat16, scale=want.abs().max().item())
     # more rows than the fused kernel takes: the unfused path, same result
-    big = rand(200, K, dtype=torch.bfloat16, seed=2)
+    big = rand(230, K, dtype=torch.bfloat16, seed=2)
     gu = big.double() @ w.double().T
     want = gu[:, :I] / (1 + torch.exp(-gu[:, :I])) * gu[:, I:]
     close(ops.linear_silu_mul(big, w), want, torch.bfloat16, scale=2 * want.abs().max().item())
 
 
-@pytest.mark.parametrize("M", [1, 5, 16, 17, 45, 64, 70, 96, 129, 192])
+@pytest.mark.parametrize("M", [1, 5, 16, 17, 45, 64, 70, 96, 129, 224])
 @pytest.mark.parametrize("heads,kv_heads,dim,K,P", [(3, 1, 32, 2048, 4), (12, 2, 128, 1536, 16), (4, 4, 16, 72, 16),
                                                     (5, 5, 48, 240, 8), (2, 1, 80, 520, 16), (7, 1, 256, 136, 32)])
 @pytest.mark.parametrize("with_bias,write", [(True, True), (False, True), (True, False)])
