@@ -210,13 +210,14 @@ class Scheduler:
         """The step after `plan` (launched, not yet completed), planned before `plan`'s tokens are known, so that it can be launched
         while the host still waits for them; None where that is not plain. It is plain when
         every request of `plan` decodes from here on (each item samples), every running request is
-        in it, nothing waits to be admitted, and the next page of every request is there: then the
+        in it, no waiting request could take a seat in the next step (none waits, or the requests
+        that go on fill every seat), and the next page of every request is there: then the
         next step holds the same requests with one token each, except those that reach their
         length with the pending token. A request that turns out to have ended with the pending
         token (end of sequence, abort) has a row of the next step computed for nothing;
         `complete` skips it."""
         self._reap_aborted()
-        if self._waiting or not plan.items or len(plan.items) != len(self._running):
+        if not plan.items or len(plan.items) != len(self._running):
             return None
         if any(not item.samples or item.seq.state is not SeqState.RUNNING for item in plan.items):
             return None
@@ -228,6 +229,8 @@ class Scheduler:
             rows.append((i, item))
         if not rows or len(rows) > self.token_budget:
             return None
+        if self._waiting and len(rows) < self.max_seqs:
+            return None                                   # a seat is free: the plain schedule admits
         items = []
         for _, item in rows:
             if not self.cache.can_reserve(item.seq.request_id, 1):

@@ -282,3 +282,20 @@ def test_the_step_after_is_planned_ahead_only_when_that_is_plain():
         cache2.commit(item.seq.request_id, len(item.token_ids))
     assert names(plan) == ["e"] and small.schedule_ahead(plan) is None          # f waits
     small.complete(plan, [1])
+    # a request waits, but those that go on fill every seat: the step after is planned; not when one of them
+    # reaches its length with the pending token and leaves its seat
+    two, cache3 = make(8, block=4, max_seqs=2)
+    for s_ in (seq("g", 2, max_new=2), seq("h", 3, max_new=9), seq("i", 2, max_new=9)):
+        two.submit(s_)
+    plan = two.schedule()
+    assert names(plan) == ["g", "h"]
+    for item in plan.items:
+        cache3.commit(item.seq.request_id, len(item.token_ids))
+    ahead = two.schedule_ahead(plan)
+    assert names(ahead) == ["g", "h"]
+    two.complete(plan, [1, 2])
+    for item in ahead.items:
+        cache3.commit(item.seq.request_id, 1)
+    assert two.schedule_ahead(ahead) is None            # g ends with the pending token: i can have its seat
+    two.complete(ahead, [3, 4])
+    assert names(two.schedule()) == ["h", "i"]
