@@ -128,8 +128,8 @@ class DecodeGraphs:
         max_kv = runner.builder.fill(bucket.host_np, entries, pad_requests=size - len(entries), want_all=True)[5]
         bucket.dev.copy_(bucket.host, non_blocking=True)
         bucket.copied.record()
-        if feed is not None:
-            bucket.dev[:len(entries)].copy_(feed)        # the token ids lead the packed buffer
+        if feed is not None and feed.shape[0]:
+            bucket.dev[:feed.shape[0]].copy_(feed)       # the token ids lead the packed buffer
         limit = self.contexts[bisect.bisect_left(self.contexts, max_kv)]
         made = bucket.graphs.get(limit)
         if made is None:

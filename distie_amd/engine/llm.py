@@ -274,7 +274,9 @@ class LLM:
                     sampled_row[i] = len(sampled_row)
             rows = [sampled_row[i] for i in ahead.feeds]
             feed = chosen
-            if rows != list(range(chosen.shape[0])):
+            if not rows:
+                feed = None                              # nothing of it hangs on a pending token
+            elif rows != list(range(chosen.shape[0])):
                 index = torch.tensor(rows, dtype=torch.int32, device=chosen.device)
                 feed = self.ops.gather_rows(chosen.view(-1, 1), index).view(-1)
             self._ahead = (ahead, self.runner.step(self._entries(ahead), reserve=False, feed=feed))

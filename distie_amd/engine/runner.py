@@ -36,11 +36,12 @@ class ModelRunner:
         """-> float32 [wanted, vocab] in the order of the entries and of their `want`
         (None if nothing is wanted). A request not yet known to the cache is added.
 
-        `feed` (int32 [len(entries)], on the device): every entry brings one token, and the token of
-        entry i is feed[i], which need not have reached the host (the entries' own tokens are
-        placeholders)."""
-        if feed is not None and (any(len(e.tokens) != 1 for e in entries) or feed.shape[0] != len(entries)):
-            raise ValueError("a fed step takes one token for each entry")
+        `feed` (int32 [F], on the device, F <= len(entries)): each of the first F entries brings one
+        token, and the token of entry i is feed[i], which need not have reached the host (those
+        entries' own tokens are placeholders)."""
+        if feed is not None and (feed.shape[0] > len(entries) or
+                                 any(len(e.tokens) != 1 for e in entries[:feed.shape[0]])):
+            raise ValueError("a fed step takes one token for each of its first entries")
         if not entries:
             raise ValueError("empty step")
         for entry in entries:
@@ -64,8 +65,8 @@ class ModelRunner:
                 logits = None
         if not ran:
             ids, meta, want_rows = self.builder.build(entries)
-            if feed is not None:
-                ids.copy_(feed)
+            if feed is not None and feed.shape[0]:
+                ids[:feed.shape[0]].copy_(feed)           # one-token entries lead the step: entry i is token i
             logits = self.model.forward(self.ops, ids, meta, self.cache, self.act_dtype, want_rows)
         for entry in entries:
             self.cache.commit(entry.request_id, len(entry.tokens))

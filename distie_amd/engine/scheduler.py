@@ -207,40 +207,70 @@ class Scheduler:
     PENDING = 0        # stands in a planned-ahead item for the token that the step before is still sampling
 
     def schedule_ahead(self, plan: StepPlan) -> Optional[StepPlan]:
-        """The step after `plan` (launched, not yet completed), planned before `plan`'s tokens are known, so that it can be launched
-        while the host still waits for them; None where that is not plain. It is plain when
-        every request of `plan` decodes from here on (each item samples), every running request is
-        in it, no waiting request could take a seat in the next step (none waits, or the requests
-        that go on fill every seat), and the next page of every request is there: then the
-        next step holds the same requests with one token each, except those that reach their
-        length with the pending token. A request that turns out to have ended with the pending
-        token (end of sequence, abort) has a row of the next step computed for nothing;
-        `complete` skips it."""
+        """The step after `plan` (launched, not yet completed), planned before `plan`'s tokens are
+        known, so that it can be launched while the host still waits for them; None where that is not
+        plain. Every running request must be in `plan`. The step after then holds, in this order:
+        the requests of `plan` that sample, with the pending token as their one token (`feeds` names
+        their places in `plan`; those that reach their length with the pending token are left out);
+        the next portions of prompts that `plan` has not finished; and waiting requests for which a
+        seat, a state slot and pages are free now (the seat of a request that ends with the pending
+        token is free one step later). Nobody is preempted for it: if a page is missing the answer is
+        None and the plain schedule decides who gives way. A request that turns out to have ended
+        with the pending token (end of sequence, abort) has a row of the next step computed for
+        nothing; `complete` skips it."""
         self._reap_aborted()
         if not plan.items or len(plan.items) != len(self._running):
             return None
-        if any(not item.samples or item.seq.state is not SeqState.RUNNING for item in plan.items):
+        if any(item.seq.state is not SeqState.RUNNING for item in plan.items):
             return None
-        rows = []
+        budget = self.token_budget
+        items: List[ScheduledSeq] = []
+        feeds: List[int] = []
+        # called after `plan` was launched and before it is completed: its tokens are the pending ones
         for i, item in enumerate(plan.items):
-            # called after `plan` was launched and before it is completed: its token is the pending one
+            if not item.samples:
+                continue
             if len(item.seq.output_ids) + 1 >= item.seq.max_new_tokens:
                 continue                                  # ends with the pending token, whatever it is
-            rows.append((i, item))
-        if not rows or len(rows) > self.token_budget:
-            return None
-        if self._waiting and len(rows) < self.max_seqs:
-            return None                                   # a seat is free: the plain schedule admits
-        items = []
-        for _, item in rows:
-            if not self.cache.can_reserve(item.seq.request_id, 1):
+            if budget < 1 or not self.cache.can_reserve(item.seq.request_id, 1):
                 # pages run out: the plain schedule decides who gives way. What was taken so far stays
                 # with requests that need it for their next token anyway.
                 return None
             self.cache.reserve(item.seq.request_id, 1)
             items.append(ScheduledSeq(seq=item.seq, token_ids=[self.PENDING],
                                       past_len=item.past_len + len(item.token_ids), samples=True))
-        return StepPlan(items=tuple(items), feeds=tuple(i for i, _ in rows))
+            feeds.append(i)
+            budget -= 1
+        for item in plan.items:
+            if item.samples:
+                continue
+            seq = item.seq
+            begin = item.past_len + len(item.token_ids)
+            n = min(seq.num_tokens - begin, budget)
+            if n < 1:
+                return None                               # every running request is in a step, or the step is not plain
+            if not self.cache.can_reserve(seq.request_id, n):
+                return None
+            self.cache.reserve(seq.request_id, n)
+            items.append(ScheduledSeq(seq=seq, token_ids=seq.tokens(begin, begin + n), past_len=begin,
+                                      samples=begin + n == seq.num_tokens))
+            budget -= n
+        while self._waiting and len(self._running) < self.max_seqs and budget > 0:
+            seq = self._waiting[0]
+            n = min(seq.num_tokens, budget)
+            if self.cache.slots.num_free < 1 or not self.cache.can_reserve(seq.request_id, seq.num_tokens):
+                break
+            self._waiting.popleft()
+            self.cache.add(seq.request_id)
+            self.cache.reserve(seq.request_id, n)
+            seq.num_computed = 0
+            seq.state = SeqState.RUNNING
+            self._running.append(seq)
+            items.append(self._item(seq, n))
+            budget -= n
+        if not items:
+            return None
+        return StepPlan(items=tuple(items), feeds=tuple(feeds))
 
     def _item(self, seq: Sequence, n: int) -> ScheduledSeq:
         begin = seq.num_computed

@@ -148,13 +148,16 @@ def test_steps_planned_ahead_change_nothing(tiny):
     """Decoding steps are launched before the tokens of the step before have reached the host: the
     same tokens as step by step, with requests that end at different lengths, one that stops at an
     end-of-sequence token (its row of the step after is computed for nothing), sampling with a
-    temperature, and a pool so tight that planning ahead has to give way to preemption."""
+    temperature, a pool so tight that planning ahead has to give way to preemption, prompts in portions
+    (the next portion goes into the step planned ahead) and fewer seats than requests (a waiting
+    request is admitted by a step planned ahead)."""
     cfg, folder, weights = tiny
     prompts = [random_ids(cfg, n, 70 + n) for n in (3, 12, 7, 20)]
     stop = plain_greedy(weights, cfg, prompts[1], 9)[5]
     params = [SamplingParams(max_new_tokens=9), SamplingParams(max_new_tokens=14, eos_id=stop),
               SamplingParams(max_new_tokens=2), SamplingParams(max_new_tokens=11, temperature=0.8, seed=3)]
-    for options in ({}, {"num_blocks": 7}, {"token_budget": 5}):
+    for options in ({}, {"num_blocks": 7}, {"token_budget": 5}, {"max_seqs": 2}, {"max_seqs": 2, "token_budget": 4},
+                    {"max_seqs": 3, "token_budget": 6, "num_blocks": 8}):
         plain_loop = engine(folder, lookahead=False, **options)
         want = plain_loop.generate(prompts, params)
         assert plain_loop.steps_ahead == 0

@@ -266,24 +266,50 @@ def test_the_step_after_is_planned_ahead_only_when_that_is_plain():
     assert sched.complete(again, [4]) == [] and b.output_ids == [8, 6, EOS]
     cache.check()
     assert cache.free_pages() == [8]
-    # a request that waits, a prompt still in portions, or a page that is not there: no planning ahead
+    # a request that waits is admitted by the step planned ahead if a seat, a slot and its pages are free now
     sched.submit(seq("d", 2))
     plan = sched.schedule()
     for item in plan.items:
         cache.commit(item.seq.request_id, len(item.token_ids))
     sched.submit(c)
-    assert sched.schedule_ahead(plan) is None
+    ahead = sched.schedule_ahead(plan)
+    assert names(ahead) == ["d", "c"] and ahead.feeds == (0,)
+    assert [(i.token_ids, i.past_len, i.samples) for i in ahead.items] == [([sched.PENDING], 2, True), (list(range(1, 10)), 0, True)]
     sched.complete(plan, [1])
-    small, cache2 = make(2, block=4, budget=4)
-    small.submit(seq("e", 4, max_new=3))
-    small.submit(seq("f", 4, max_new=3))
+    for item in ahead.items:
+        cache.commit(item.seq.request_id, len(item.token_ids))
+    sched.complete(ahead, [2, 3])
+    assert c.output_ids == [3] and c.num_computed == 9
+    # a prompt in portions goes on in the step planned ahead; a waiting request without pages stays out of it
+    small, cache2 = make(3, block=4, budget=4)
+    e, f = seq("e", 7, max_new=3), seq("f", 8, max_new=3)
+    small.submit(e)
+    small.submit(f)
     plan = small.schedule()
+    assert [(i.seq.request_id, i.token_ids, i.samples) for i in plan.items] == [("e", [1, 2, 3, 4], False)]   # f: no pages
     for item in plan.items:
         cache2.commit(item.seq.request_id, len(item.token_ids))
-    assert names(plan) == ["e"] and small.schedule_ahead(plan) is None          # f waits
-    small.complete(plan, [1])
-    # a request waits, but those that go on fill every seat: the step after is planned; not when one of them
-    # reaches its length with the pending token and leaves its seat
+    ahead = small.schedule_ahead(plan)
+    assert [(i.seq.request_id, i.token_ids, i.past_len, i.samples) for i in ahead.items] == [("e", [5, 6, 7], 4, True)]
+    assert ahead.feeds == () and small.num_waiting == 1
+    small.complete(plan, [None])
+    for item in ahead.items:
+        cache2.commit(item.seq.request_id, len(item.token_ids))
+    after = small.schedule_ahead(ahead)
+    assert names(after) == ["e"] and after.feeds == (0,)
+    small.complete(ahead, [1])
+    # a page that is not there: no planning ahead, the plain schedule decides who gives way
+    tight, cache4 = make(2, block=4)
+    tight.submit(seq("j", 4, max_new=4))
+    tight.submit(seq("k", 3, max_new=1))
+    plan = tight.schedule()
+    assert names(plan) == ["j", "k"]
+    for item in plan.items:
+        cache4.commit(item.seq.request_id, len(item.token_ids))
+    assert tight.schedule_ahead(plan) is None             # j needs a second page, none is free
+    tight.complete(plan, [1, 2])
+    # a request waits and those that go on fill every seat: the step after is planned without it; the seat of a
+    # request that ends with the pending token is free one step later
     two, cache3 = make(8, block=4, max_seqs=2)
     for s_ in (seq("g", 2, max_new=2), seq("h", 3, max_new=9), seq("i", 2, max_new=9)):
         two.submit(s_)
@@ -296,6 +322,10 @@ def test_the_step_after_is_planned_ahead_only_when_that_is_plain():
     two.complete(plan, [1, 2])
     for item in ahead.items:
         cache3.commit(item.seq.request_id, 1)
-    assert two.schedule_ahead(ahead) is None            # g ends with the pending token: i can have its seat
+    after = two.schedule_ahead(ahead)
+    assert names(after) == ["h"] and after.feeds == (1,)      # g ends with the pending token; its seat is still taken
     two.complete(ahead, [3, 4])
-    assert names(two.schedule()) == ["h", "i"]
+    cache3.commit("h", 1)
+    last = two.schedule_ahead(after)
+    assert names(last) == ["h", "i"] and last.feeds == (0,)   # now i has g's seat
+    two.complete(after, [5])
