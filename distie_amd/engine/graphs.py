@@ -151,7 +151,7 @@ class DecodeGraphs:
         ids, meta, want = runner.builder.meta_of(bucket.dev, bucket.offsets, n, n, n, 1, limit)
         runner.ops.captured = True
         try:
-            return runner.model.forward(runner.ops, ids, meta, runner.cache, runner.act_dtype, want)
+            return runner.model.forward(runner.ops, ids, meta, runner.cache, runner.act_dtype, want, every_row=True)
         finally:
             runner.ops.captured = False
 

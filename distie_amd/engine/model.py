@@ -102,9 +102,11 @@ class Model:
         return total
 
     # ------------------------------------------------------------ the step
-    def forward(self, ops, ids: torch.Tensor, meta, cache, act_dtype, want_rows: Optional[torch.Tensor]):
+    def forward(self, ops, ids: torch.Tensor, meta, cache, act_dtype, want_rows: Optional[torch.Tensor],
+                every_row: bool = False):
         """ids int32 [T] -> float32 logits [R, vocab] at `want_rows` (int32 [R]); None if no
-        row is wanted (the step then only fills the cache)."""
+        row is wanted (the step then only fills the cache). `every_row`: `want_rows` names every row
+        in order (a captured decode step), so nothing needs to be gathered."""
         stream = ResidualStream(ops.embed(ids, self.embedding))
         if self.position is not None:
             self.position.on_embedding(ops, stream.hidden, meta)
@@ -115,6 +117,9 @@ class Model:
             self.blocks[call.layer].forward(ops, stream, ctx, view, call.writes_cache)
         if want_rows is None:
             return None
+        if every_row:
+            normed = self.final_norm.of_stream(ops, stream, act_dtype)
+            return ops.linear_f32out(normed, self.head)
         hidden = ops.gather_rows(stream.hidden, want_rows)
         if stream.pending is not None:
             normed = self.final_norm.add_apply(ops, hidden, ops.gather_rows(stream.pending, want_rows), act_dtype)
