@@ -187,3 +187,30 @@ def test_layer_sizes_of_the_1_5b_model(tmp_path, ops):
                 assert diff.abs().max().item() < 1e-4 * max(1.0, scale), (name, diff.abs().max().item(), scale)
             else:
                 assert diff.abs().max().item() < scale / 16 and diff.pow(2).mean().sqrt().item() < scale / 64, name
+
+
+ODD_SIZES = [
+    dict(hidden_size=48, num_attention_heads=3, num_key_value_heads=1, head_dim=16, intermediate_size=100, vocab_size=1001),
+    dict(hidden_size=336, num_attention_heads=7, num_key_value_heads=1, head_dim=48, intermediate_size=250, vocab_size=333,
+         layer_types=["sliding_attention", "full_attention"], sliding_window=40),
+    dict(hidden_size=1056, num_attention_heads=66, num_key_value_heads=1, head_dim=16, intermediate_size=64, vocab_size=130),
+    dict(hidden_size=1024, num_attention_heads=4, num_key_value_heads=2, head_dim=256, intermediate_size=36, vocab_size=9,
+         tie_word_embeddings=False),
+]
+
+
+@pytest.mark.parametrize("sizes", ODD_SIZES, ids=lambda s: f"{s['num_attention_heads']}x{s['head_dim']}")
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_odd_sizes(tmp_path, ops, sizes, dtype_name):
+    """Sizes at the edges of what the kernels take: a feed-forward width and a vocabulary that are no multiple
+    of 8, seven and 66 query heads on one kv head (more than the decode kernel's columns), head sizes 16 and
+    256, a vocabulary of nine."""
+    dtype = DTYPES[dtype_name]
+    cfg = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 2, "rope_theta": 10000.0,
+           "rms_norm_eps": 1e-5, "tie_word_embeddings": True, "max_position_embeddings": 512, "hidden_act": "silu", **sizes}
+    folder, weights = make_model_dir(tmp_path, cfg, seed=23, std=min(0.3, 2.0 / cfg["hidden_size"] ** 0.5), dtype=dtype)
+    runner = build_runner(folder, ops, dtype, block_size=16, num_blocks=24, max_model_len=512)
+    ids = random_ids(cfg, 150, 9)
+    check_logits(replay_whole(runner, "a", ids), weights, cfg, ids, dtype, folder)
+    check_logits(replay_cut(runner, "b", ids, [70, 3, 40, 2, 17]), weights, cfg, ids, dtype, folder)
+    runner.cache.check()
