@@ -184,7 +184,7 @@ def ensure(name: str) -> Path:
     return build(name, force=False)
 
 
-DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128, 256)
+DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 256)
 
 
 def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True) -> List[Path]:
