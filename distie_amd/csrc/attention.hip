@@ -158,7 +158,7 @@ extern "C" int distie_attention_generic(const void* qkv, int dtype, int64_t q_st
 //  between lanes except the maxima and the rescaling factors.
 //
 //  * attn_decode: requests that bring one token. Columns = the G query heads that share one kv head. The
-//    keys are cut into runs of `split_len`, one wave each (this is where the parallelism comes from when
+//    keys of a request are cut into runs of equal length, one wave each (this is where the parallelism comes from when
 //    few requests decode); a wave takes its run in chunks of DC_KEYS keys and issues every load of a chunk
 //    (pages, K rows, V^T rows) before it computes, so a chunk costs one trip to memory. It writes
 //    unnormalised partial results that attn_reduce combines.
@@ -177,12 +177,34 @@ constexpr int DB16 = D / 16;            // 16-wide blocks of the output
 constexpr int DC_BLOCKS = (D <= 128) ? 4 : 2;   // blocks of 16 keys whose loads are in flight together
 constexpr int DC_KEYS = 16 * DC_BLOCKS;
 
+// How one request's keys are cut into runs. The visible keys (all of them, or the window's), counted from the
+// 64-key boundary at or before the first of them, are cut into at most `max_splits` runs of one length, a
+// multiple of RUN_STEP: the request's own length decides, not the longest of the batch, so that every request
+// keeps all of its waves busy whatever else the step holds. Both kernels derive the same numbers.
+constexpr int RUN_STEP = 64;            // a multiple of DC_KEYS for every head size
+struct KeyRuns {
+  int first;      // first visible key
+  int origin;     // where run 0 begins
+  int length;     // keys per run
+  int count;      // runs that hold a key
+};
+__device__ __forceinline__ KeyRuns key_runs(int q_pos, int window, int max_splits) {
+  KeyRuns runs;
+  runs.first = window > 0 ? max(0, q_pos - window + 1) : 0;
+  runs.origin = runs.first / RUN_STEP * RUN_STEP;
+  const int span = q_pos - runs.origin + 1;
+  const int step = max_splits * RUN_STEP;
+  runs.length = (span + step - 1) / step * RUN_STEP;        // ceil(span / max_splits), rounded up to RUN_STEP
+  runs.count = (span + runs.length - 1) / runs.length;      // <= max_splits
+  return runs;
+}
+
 template <int MB>
 __global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ qkv, int64_t q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ kv_len, const int32_t* __restrict__ cu_q,
     const int32_t* __restrict__ block_table, int table_width, float* __restrict__ part_o,
-    float* __restrict__ part_ml, int heads, int kv_heads, int block_size, float scale, int window, int split_len,
+    float* __restrict__ part_ml, int heads, int kv_heads, int block_size, float scale, int window, int split_hint,
     int max_splits, int dense_rows) {
   const int lane = threadIdx.x;
   const int r = lane % 16;
@@ -192,20 +214,23 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
   const int request = blockIdx.z;
   const int kh = blockIdx.y;
   const int32_t* table = block_table + static_cast<int64_t>(request) * table_width;
-  // The pages of the run's first chunk are asked for before it is known whether the run holds a key at all
-  // (the entry is inside the table either way): one trip to memory less on the way to the keys.
-  const int run_begin = static_cast<int>(blockIdx.x) * split_len;
+  // The pages of the run's first chunk are asked for before the request's length says where the run begins:
+  // at the place it has if the runs are `split_hint` long and begin at key 0, which the host derives from the
+  // longest request of the step (the entry is inside the table either way). Where the guess holds, which it
+  // does when few requests of similar length decode, that is one trip to memory less on the way to the keys.
+  const int guess_begin = static_cast<int>(blockIdx.x) * split_hint;
   int pages[DC_BLOCKS];
 #pragma unroll
-  for (int b = 0; b < DC_BLOCKS; ++b) pages[b] = table[min((run_begin + 16 * b) / block_size, table_width - 1)];
+  for (int b = 0; b < DC_BLOCKS; ++b) pages[b] = table[min((guess_begin + 16 * b) / block_size, table_width - 1)];
   // dense_rows: every request brings one token, so request i's token is row i
   const int token = dense_rows ? request : cu_q[request];
   if (!dense_rows && cu_q[request + 1] - token != 1) return;        // a portion of a prompt: the tiled kernel's
   const int q_pos = kv_len[request] - 1;              // the new token is the last one cached
-  const int first = window > 0 ? max(0, q_pos - window + 1) : 0;
-  const int key_begin = max(first, run_begin);
-  const int key_end = min(q_pos, run_begin + split_len - 1);
-  if (key_begin > key_end) return;
+  const KeyRuns runs = key_runs(q_pos, window, max_splits);
+  if (static_cast<int>(blockIdx.x) >= runs.count) return;
+  const int run_begin = runs.origin + static_cast<int>(blockIdx.x) * runs.length;
+  const int key_begin = max(runs.first, run_begin);
+  const int key_end = min(q_pos, run_begin + runs.length - 1);
 
   // ---- the query of this lane's column (head kh * G + 16 mb + r; columns past the group repeat the last)
   bf16x8 q_reg[MB][DK32 > 0 ? DK32 : 1];
@@ -230,8 +255,8 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
 
   // every chunk of the walk holds at least one visible key (the running maximum is then finite): under a
   // window the walk starts at the chunk of the first visible key, whose pages are asked for now
-  const int chunk_begin = max(run_begin, key_begin / DC_KEYS * DC_KEYS);      // split_len is a multiple of DC_KEYS
-  if (chunk_begin != run_begin) {
+  const int chunk_begin = max(run_begin, key_begin / DC_KEYS * DC_KEYS);      // runs begin at multiples of DC_KEYS
+  if (chunk_begin != guess_begin) {
 #pragma unroll
     for (int b = 0; b < DC_BLOCKS; ++b) pages[b] = table[min((chunk_begin + 16 * b) / block_size, table_width - 1)];
   }
@@ -395,7 +420,7 @@ constexpr int RD_FAST_RUNS = RD_FAST_PER_WAVE * RD_WAVES;
 template <bool FAST>
 __global__ __launch_bounds__(RD_THREADS) void attn_reduce_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int32_t* __restrict__ kv_len,
-    const int32_t* __restrict__ cu_q, bf16_t* __restrict__ out, int heads, int window, int split_len, int max_splits,
+    const int32_t* __restrict__ cu_q, bf16_t* __restrict__ out, int heads, int window, int max_splits,
     int dense_rows) {
   __shared__ float weight_s[FAST ? RD_FAST_RUNS : RD_MAX_RUNS];
   __shared__ float sum_s[RD_WAVES][D];
@@ -425,15 +450,12 @@ __global__ __launch_bounds__(RD_THREADS) void attn_reduce_kernel(
   const int token = dense_rows ? request : cu_q[request];
   if (!dense_rows && cu_q[request + 1] - token != 1) return;
   const int q_pos = kv_len[request] - 1;
-  const int first = window > 0 ? max(0, q_pos - window + 1) : 0;
-  const int s_first = first / split_len;
-  const int runs = q_pos / split_len - s_first + 1;
-  const int64_t base = base0 + s_first;
+  const int runs = key_runs(q_pos, window, max_splits).count;     // the first `runs` places hold results
+  const int64_t base = base0;
   bf16_t* o = out + (static_cast<int64_t>(token) * heads + head) * D;
 
   if constexpr (FAST) {
-    // run j (counted from the buffers' start) exists iff s_first <= j < s_first + runs
-    const bool mine = tid >= s_first && tid < s_first + runs;
+    const bool mine = tid < runs;
     float m = mine ? early_ml.x : -INFINITY;
     m = wave_max(m);
     if (lane == 0) scratch[wave] = m;
@@ -450,7 +472,7 @@ __global__ __launch_bounds__(RD_THREADS) void attn_reduce_kernel(
 #pragma unroll
       for (int u = 0; u < RD_FAST_PER_WAVE; ++u) {
         const int j = wave + RD_WAVES * u;
-        const bool exists = j >= s_first && j < s_first + runs;
+        const bool exists = j < runs;
         a = exists ? fmaf(weight_s[j], early[u][i], a) : a;
       }
       sum_s[wave][d] = a;
@@ -514,18 +536,19 @@ constexpr int DECODE_MAX_MB = (D <= 128) ? 4 : 2;   // registers: the output til
 extern "C" int distie_attention_decode_columns() { return 16 * DECODE_MAX_MB; }
 
 // The requests of a step that bring one token (others are skipped). kv_len: tokens cached after the step, per
-// request. part_o: float32 [requests, heads, max_splits, D], part_ml: float32 [requests, heads, max_splits, 2];
-// max_splits * split_len must cover every position.
+// request. part_o: float32 [requests, heads, max_splits, D], part_ml: float32 [requests, heads, max_splits, 2]:
+// every request's keys are cut into at most max_splits runs by its own length. split_hint, a multiple of 64, is
+// the run length the caller expects of the longest request; it only saves time where it is right.
 extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, const void* k_cache, const void* v_cache,
                                             const int32_t* kv_len, const int32_t* cu_q, const int32_t* block_table,
                                             int table_width, void* out, float* part_o, float* part_ml,
                                             int num_requests, int heads, int kv_heads, int block_size, float scale,
-                                            int window, int split_len, int max_splits, int dense_rows,
+                                            int window, int split_hint, int max_splits, int dense_rows,
                                             hipStream_t stream) {
   if (num_requests <= 0) return 0;
   const int group = kv_heads > 0 ? heads / kv_heads : 0;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size % 16 != 0 || table_width < 1 || window < 0 ||
-      split_len < DC_KEYS || split_len % DC_KEYS != 0 || max_splits < 1 || max_splits > RD_MAX_RUNS ||
+      split_hint < RUN_STEP || split_hint % RUN_STEP != 0 || max_splits < 1 || max_splits > RD_MAX_RUNS ||
       group > 16 * DECODE_MAX_MB || kv_heads > 65535 || num_requests > 65535 || heads > 65535)
     return DISTIE_BAD_ARGUMENT;
   dim3 grid(max_splits, kv_heads, num_requests);
@@ -535,7 +558,7 @@ extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, c
 #define DECODE_LAUNCH(MB)                                                                                             \
   attn_decode_kernel<MB><<<grid, DISTIE_WAVE, 0, stream>>>(q, q_stride, kc, vc, kv_len, cu_q, block_table, table_width, \
                                                            part_o, part_ml, heads, kv_heads, block_size, scale, window, \
-                                                           split_len, max_splits, dense_rows)
+                                                           split_hint, max_splits, dense_rows)
   if (group <= 16) {
     DECODE_LAUNCH(1);
   } else if (group <= 32) {
@@ -548,10 +571,10 @@ extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, c
   if (status != 0) return status;
   if (max_splits <= RD_FAST_RUNS) {
     attn_reduce_kernel<true><<<dim3(heads, num_requests), RD_THREADS, 0, stream>>>(
-        part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, split_len, max_splits, dense_rows);
+        part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, max_splits, dense_rows);
   } else {
     attn_reduce_kernel<false><<<dim3(heads, num_requests), RD_THREADS, 0, stream>>>(
-        part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, split_len, max_splits, dense_rows);
+        part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, max_splits, dense_rows);
   }
   return launch_status();
 }

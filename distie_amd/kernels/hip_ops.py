@@ -490,14 +490,13 @@ class HipOps(Ops):
             split_decode = singles > 0 and group <= lib.distie_attention_decode_columns()
             if split_decode:
                 # requests that bring one token: keys are cut into runs, one wave each, so that the chip is
-                # filled even when few requests decode
-                runs = max(1, min(self.DECODE_MAX_RUNS, self.DECODE_WAVES // (singles * num_kv_heads)))
-                # under a window only the runs that hold its keys do anything: cut by the window's length,
-                # but into no more than DECODE_MAX_RUNS places for partial results
-                visible = min(meta.max_kv, int(window)) if window else meta.max_kv
-                split_len = max(-(-visible // runs), -(-meta.max_kv // self.DECODE_MAX_RUNS))
-                split_len = max(64, -(-split_len // 64) * 64)
-                max_splits = -(-meta.max_kv // split_len)
+                # filled even when few requests decode. The kernel cuts every request's visible keys (counted
+                # from a 64-key boundary) into at most `max_splits` runs by the request's own length; the length
+                # of the longest request's runs is passed along as a hint for the first lookups of pages.
+                visible = min(meta.max_kv, int(window) + 63) if window else meta.max_kv
+                max_splits = max(1, min(self.DECODE_MAX_RUNS, self.DECODE_WAVES // (singles * num_kv_heads),
+                                        -(-visible // 64)))
+                split_len = -(-visible // (64 * max_splits)) * 64
                 part_o = torch.empty((meta.num_requests, num_heads, max_splits, head_dim), dtype=torch.float32,
                                      device=self.device)
                 part_ml = torch.empty((meta.num_requests, num_heads, max_splits, 2), dtype=torch.float32,

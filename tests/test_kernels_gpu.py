@@ -372,7 +372,7 @@ def paged_case(heads, kv_heads, dim, P, lens, q_lens, dtype, seed=0):
 ATTENTION_SHAPES = [
     (4, 2, 16, 4, None), (3, 1, 32, 8, 8), (5, 5, 48, 16, 20), (12, 2, 128, 16, None),
     (6, 3, 64, 5, 33), (8, 1, 80, 16, None), (2, 2, 256, 32, 100), (4, 2, 16, 16, 7), (40, 2, 32, 16, None),
-    (12, 2, 128, 64, 150)]
+    (12, 2, 128, 64, 150), (4, 2, 64, 16, 1000)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -440,10 +440,18 @@ def test_paged_attention_decode_step(ops, dtype, heads, kv_heads, dim, P, window
                                             dim ** -0.5, window)
     got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
     close(got, want, dtype, scale=want.abs().max().item())
-    # as in a captured step: the launch is sized for the longest context the model allows
-    # (20,000: more runs than the quick combination of partial results takes; under a window the runs are
-    # cut by the window's length and most of them hold no visible key)
+    # as in a captured step: the launch is sized for the longest context the model allows (more places for
+    # partial results than any of these requests fills, and a wrong guess of where their runs begin)
     for limit in (4096, 20000):
+        meta.max_kv = limit
+        got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
+        close(got, want, dtype, scale=want.abs().max().item())
+    # two requests, one of them long: more runs than the quick combination of partial results takes, while
+    # the short request fills two of its places
+    meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, [5000, 70], [1, 1], dtype, seed=3)
+    want = TorchOps("cuda").paged_attention(qkv.double(), meta, 0, k.double(), v.double(), heads, kv_heads, dim,
+                                            dim ** -0.5, window)
+    for limit in (5000, 32768):
         meta.max_kv = limit
         got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
         close(got, want, dtype, scale=want.abs().max().item())
