@@ -14,11 +14,11 @@ The step's metadata reaches the device with one copy from pinned host memory bef
 replay; nothing inside the graph depends on a Python number.
 
 One number of the step is frozen into a graph all the same: the longest context it is made for,
-from which decode attention derives how it cuts the keys into runs. A graph made for the model's
-limit would cut a 2,000-token context into the few long runs that suit 32,768 tokens, so a bucket
-keeps one graph per class of context length (1,024, 1,536, 2,048, 3,072, ... up to the limit),
-each captured when a step first needs it; a step replays the graph of the smallest class that
-holds its longest request.
+from which decode attention derives how many runs of keys a request may be cut into and where a
+wave first looks for its pages. A graph made for the model's limit would suit a 2,000-token
+context badly, so a bucket keeps one graph per class of context length (1,024, 1,536, 2,048,
+3,072, ... up to the limit), each captured when a step first needs it; a step replays the graph
+of the smallest class that holds its longest request.
 """
 
 from __future__ import annotations
