@@ -177,10 +177,160 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
   }
 }
 
+// Large vocabularies: one block per row walks 150,000 logits three times, alone (0.4 ms). As for argmax the row
+// is cut into pieces (grid: parts x rows): a block writes its piece's best and, for rows that draw, the piece's
+// sum of weights relative to that best. A second launch, one block per row, puts the pieces together (the
+// row's best, every piece's sum rescaled to it, added in order), finds the piece in which the cumulative
+// weight passes the target and walks that piece alone.
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_pieces_kernel(const float* __restrict__ logits,
+                                                                       const float* __restrict__ temperature,
+                                                                       float* __restrict__ piece_value,
+                                                                       int32_t* __restrict__ piece_index,
+                                                                       float* __restrict__ piece_sum, int vocab,
+                                                                       int piece_len) {
+  __shared__ Best scratch[SAMPLE_THREADS / DISTIE_WAVE];
+  __shared__ float reduce_scratch[16];
+  const float* row = logits + static_cast<int64_t>(blockIdx.y) * vocab;
+  const int begin = blockIdx.x * piece_len;
+  const int end = min(vocab, begin + piece_len);
+  Best mine{-INFINITY, 0x7fffffff};
+  for (int i = begin + threadIdx.x; i < end; i += blockDim.x) mine = better(mine, Best{row[i], i});
+  const Best best = block_best(mine, scratch);
+  const float t = temperature[blockIdx.y];
+  float sum = 0.f;
+  if (t > 0.f && best.value > -INFINITY) {
+    const float inv_t = 1.f / t;
+    for (int i = begin + threadIdx.x; i < end; i += blockDim.x) sum += expf((row[i] - best.value) * inv_t);
+    sum = block_sum(sum, reduce_scratch);
+  }
+  if (threadIdx.x == 0) {
+    const int slot = blockIdx.y * gridDim.x + blockIdx.x;
+    piece_value[slot] = best.value;
+    piece_index[slot] = best.index;
+    piece_sum[slot] = sum;
+  }
+}
+
+constexpr int SAMPLE_MAX_PARTS = 64;
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_pick_kernel(
+    const float* __restrict__ logits, const float* __restrict__ temperature, const int64_t* __restrict__ seeds,
+    const int64_t* __restrict__ counters, const float* __restrict__ piece_value,
+    const int32_t* __restrict__ piece_index, const float* __restrict__ piece_sum, int32_t* __restrict__ out, int parts,
+    int vocab, int piece_len) {
+  __shared__ float scaled[SAMPLE_MAX_PARTS];
+  __shared__ float sums[SAMPLE_THREADS];
+  __shared__ float before_s, target_s;
+  __shared__ int piece_s;
+  const int tid = threadIdx.x;
+  const int r = blockIdx.x;
+  // every wave finds the row's best among the pieces for itself
+  const int lane = tid % DISTIE_WAVE;
+  Best best{-INFINITY, 0x7fffffff};
+  if (lane < parts) best = Best{piece_value[r * parts + lane], piece_index[r * parts + lane]};
+  const float own_value = best.value;
+#pragma unroll
+  for (int o = DISTIE_WAVE / 2; o > 0; o >>= 1) {
+    Best other{__shfl_xor(best.value, o, DISTIE_WAVE), __shfl_xor(best.index, o, DISTIE_WAVE)};
+    best = better(best, other);
+  }
+  if (best.index >= vocab) best.index = 0;           // a row of NaN or -inf
+  const float t = temperature[r];
+  if (!(t > 0.f) || !(best.value > -INFINITY)) {
+    if (tid == 0) out[r] = best.index;
+    return;
+  }
+  const float inv_t = 1.f / t;
+  if (tid < parts) {
+    const float s = piece_sum[r * parts + tid];
+    scaled[tid] = s > 0.f ? s * expf((own_value - best.value) * inv_t) : 0.f;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    float total = 0.f;
+    for (int p = 0; p < parts; ++p) total += scaled[p];
+    const float target = uniform_of(static_cast<uint64_t>(seeds[r]), static_cast<uint64_t>(counters[r])) * total;
+    // the piece in which the cumulative weight passes the target; rounding may leave the target beyond the
+    // last piece: then the last piece with weight
+    float before = 0.f;
+    int piece = -1, last = 0;
+    for (int p = 0; p < parts; ++p) {
+      if (!(scaled[p] > 0.f)) continue;
+      last = p;
+      if (before + scaled[p] > target) {
+        piece = p;
+        break;
+      }
+      before += scaled[p];
+    }
+    if (piece < 0) {
+      piece = last;
+      before -= scaled[last];
+    }
+    piece_s = piece;
+    before_s = before;
+    target_s = target;
+  }
+  __syncthreads();
+  const float target = target_s;
+  const int begin = piece_s * piece_len;
+  const int end = min(vocab, begin + piece_len);
+  const float* row = logits + static_cast<int64_t>(r) * vocab;
+  // every thread owns a contiguous run of the piece
+  const int per = (end - begin + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  const int mine_begin = min(end, begin + tid * per);
+  const int mine_end = min(end, mine_begin + per);
+  float mine = 0.f;
+  for (int i = mine_begin; i < mine_end; ++i) mine += expf((row[i] - best.value) * inv_t);
+  sums[tid] = mine;
+  __syncthreads();
+  if (tid == 0) {
+    float running = before_s;
+    int owner = 0;
+    for (; owner < SAMPLE_THREADS - 1; ++owner) {
+      if (running + sums[owner] > target) break;
+      running += sums[owner];
+    }
+    const int b = min(end, begin + owner * per), e = min(end, b + per);
+    int pick = -1;
+    for (int i = b; i < e; ++i) {
+      running += expf((row[i] - best.value) * inv_t);
+      if (running > target) {
+        pick = i;
+        break;
+      }
+    }
+    if (pick < 0) {
+      // rounding left the target beyond the piece's end: its last token with weight
+      pick = best.index;
+      for (int i = end - 1; i >= begin; --i)
+        if (expf((row[i] - best.value) * inv_t) > 0.f) {
+          pick = i;
+          break;
+        }
+    }
+    out[r] = pick;
+  }
+}
+
+// scratch: piece_value and piece_sum float [rows * parts], piece_index int32 [rows * parts], parts from
+// distie_argmax_parts; may be null when that is 1
 extern "C" int distie_sample(const float* logits, const float* temperature, const int64_t* seeds,
-                             const int64_t* counters, int32_t* out, int rows, int vocab, hipStream_t stream) {
+                             const int64_t* counters, int32_t* out, int rows, int vocab, float* piece_value,
+                             int32_t* piece_index, float* piece_sum, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (vocab <= 0) return DISTIE_BAD_ARGUMENT;
-  sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, temperature, seeds, counters, out, vocab);
+  const int parts = distie_argmax_parts(rows, vocab);
+  if (parts == 1) {
+    sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, temperature, seeds, counters, out, vocab);
+    return launch_status();
+  }
+  if (piece_value == nullptr || piece_index == nullptr || piece_sum == nullptr || parts > SAMPLE_MAX_PARTS)
+    return DISTIE_BAD_ARGUMENT;
+  const int piece_len = (vocab + parts - 1) / parts;
+  sample_pieces_kernel<<<dim3(parts, rows), SAMPLE_THREADS, 0, stream>>>(logits, temperature, piece_value, piece_index,
+                                                                        piece_sum, vocab, piece_len);
+  sample_pick_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, temperature, seeds, counters, piece_value,
+                                                          piece_index, piece_sum, out, parts, vocab, piece_len);
   return launch_status();
 }

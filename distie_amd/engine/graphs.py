@@ -143,7 +143,7 @@ class DecodeGraphs:
             return logits[:0]
         if len(rows) == len(entries):
             return logits[:len(entries)]
-        return logits[torch.tensor(rows, device=logits.device)]
+        return logits[runner.ops.upload(np.asarray(rows, dtype=np.int64))]
 
     def _forward(self, bucket: _Bucket, limit: int) -> torch.Tensor:
         runner = self.runner

@@ -19,6 +19,7 @@ from dataclasses import dataclass, field
 from pathlib import Path
 from typing import Dict, Hashable, Iterator, List, Optional, Sequence as Seq, Union
 
+import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
@@ -277,7 +278,7 @@ class LLM:
             if not rows:
                 feed = None                              # nothing of it hangs on a pending token
             elif rows != list(range(chosen.shape[0])):
-                index = torch.tensor(rows, dtype=torch.int32, device=chosen.device)
+                index = self.ops.upload(np.asarray(rows, dtype=np.int32))
                 feed = self.ops.gather_rows(chosen.view(-1, 1), index).view(-1)
             self._ahead = (ahead, self.runner.step(self._entries(ahead), reserve=False, feed=feed))
             self.steps_ahead += 1

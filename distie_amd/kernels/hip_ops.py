@@ -15,6 +15,7 @@ from __future__ import annotations
 import ctypes
 from typing import Dict, Optional
 
+import numpy as np
 import torch
 
 from ..csrc import build
@@ -112,8 +113,36 @@ class HipOps(Ops):
         self._ops = ctypes.CDLL(str(build.ensure("ops")))
         self._declare()
         self._attn: Dict[int, ctypes.CDLL] = {}
+        # pinned staging buffers for `upload`, used in turn: [host tensor, its numpy view, event of the last copy]
+        self._uploads = [[None, None, None] for _ in range(self.UPLOAD_BUFFERS)]
+        self._next_upload = 0
 
     # ------------------------------------------------------------ plumbing
+    UPLOAD_BUFFERS = 8
+
+    def upload(self, values: np.ndarray) -> torch.Tensor:
+        """Through pinned memory, so that the copy is queued like a kernel: `torch.tensor(..., device=...)` copies
+        from pageable memory and returns only when everything queued before it is done, which made the host
+        wait for the running step three times per sampled step."""
+        values = np.ascontiguousarray(values)
+        dtype = torch.from_numpy(np.empty(0, dtype=values.dtype)).dtype
+        nbytes = values.nbytes
+        if nbytes == 0:
+            return torch.empty(values.shape, dtype=dtype, device=self.device)
+        slot = self._uploads[self._next_upload]
+        self._next_upload = (self._next_upload + 1) % len(self._uploads)
+        if slot[2] is not None:
+            slot[2].synchronize()                       # the copy made out of this buffer some calls ago is done
+        if slot[0] is None or slot[0].numel() < nbytes:
+            slot[0] = torch.empty(max(4096, 2 * nbytes), dtype=torch.uint8, pin_memory=True)
+            slot[1] = slot[0].numpy()
+            slot[2] = torch.cuda.Event()
+        slot[1][:nbytes] = values.reshape(-1).view(np.uint8)
+        dev = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+        dev.copy_(slot[0][:nbytes], non_blocking=True)
+        slot[2].record()
+        return dev.view(dtype).view(values.shape)
+
     def _declare(self) -> None:
         o = self._ops
         o.distie_embed.argtypes = [_P, _P, _I, _P, _I, _I, _I, _P]
@@ -133,7 +162,7 @@ class HipOps(Ops):
         o.distie_gemm_packed_rotary_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         o.distie_argmax.argtypes = [_P, _P, _I, _I, _P, _P, _P]
         o.distie_argmax_parts.argtypes = [_I, _I]
-        o.distie_sample.argtypes = [_P, _P, _P, _P, _P, _I, _I, _P]
+        o.distie_sample.argtypes = [_P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P]
 
     def tune_library_products(self, on: bool) -> None:
         """While on, the library times its candidate kernels for every new shape of a large product and
@@ -575,8 +604,17 @@ class HipOps(Ops):
         if logits.dtype != torch.float32 or temperature.dtype != torch.float32 or \
                 seeds.dtype != torch.int64 or counters.dtype != torch.int64:
             raise KernelError("sample: logits/temperature float32, seeds/counters int64")
-        out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
+        rows, vocab = logits.shape
+        out = torch.empty(rows, dtype=torch.int32, device=self.device)
+        parts = self._ops.distie_argmax_parts(rows, vocab)
+        values = indexes = sums = None
+        if parts > 1:
+            values = torch.empty(rows * parts, dtype=torch.float32, device=self.device)
+            indexes = torch.empty(rows * parts, dtype=torch.int32, device=self.device)
+            sums = torch.empty(rows * parts, dtype=torch.float32, device=self.device)
         _check(self._ops.distie_sample(logits.data_ptr(), temperature.data_ptr(), seeds.data_ptr(),
-                                       counters.data_ptr(), out.data_ptr(), logits.shape[0], logits.shape[1],
-                                       self._stream()), "sample")
+                                       counters.data_ptr(), out.data_ptr(), rows, vocab,
+                                       values.data_ptr() if parts > 1 else None,
+                                       indexes.data_ptr() if parts > 1 else None,
+                                       sums.data_ptr() if parts > 1 else None, self._stream()), "sample")
         return out

@@ -17,6 +17,7 @@ import abc
 from dataclasses import dataclass, field
 from typing import List, Optional
 
+import numpy as np
 import torch
 
 
@@ -57,6 +58,11 @@ class Ops(abc.ABC):
     # True while the engine warms or records a captured step: launches then cost the host nothing when the
     # step is replayed, so an implementation may choose kernels by their time on the device alone
     captured: bool = False
+
+    def upload(self, values: np.ndarray) -> torch.Tensor:
+        """A small host array (row indexes, sampling parameters) as a device tensor of the same dtype and
+        shape. An implementation makes this a copy that does not wait for the work queued before it."""
+        return torch.from_numpy(np.ascontiguousarray(values)).to(self.device)
 
     @abc.abstractmethod
     def embed(self, ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:

@@ -14,6 +14,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import List, Optional, Sequence
 
+import numpy as np
 import torch
 
 _MASK = (1 << 64) - 1
@@ -61,12 +62,10 @@ class Sampler:
             raise ValueError("one temperature per row of logits")
         if all(t <= 0 for t in temperatures):
             return self.ops.argmax(logits)
-        dev = self.ops.device
         # int64 two's complement carries the unsigned 64-bit seed unchanged
         wrap = lambda v: ((int(v) & _MASK) ^ (1 << 63)) - (1 << 63)
-        picks = self.ops.sample(
+        return self.ops.sample(
             logits,
-            torch.tensor(list(temperatures), dtype=torch.float32, device=dev),
-            torch.tensor([wrap(s) for s in seeds], dtype=torch.int64, device=dev),
-            torch.tensor([wrap(c) for c in counters], dtype=torch.int64, device=dev))
-        return picks
+            self.ops.upload(np.asarray(list(temperatures), dtype=np.float32)),
+            self.ops.upload(np.asarray([wrap(s) for s in seeds], dtype=np.int64)),
+            self.ops.upload(np.asarray([wrap(c) for c in counters], dtype=np.int64)))

@@ -521,6 +521,25 @@ def test_argmax_and_sample(ops):
         hits += int((got == want.cuda()).sum())
     # the float32 cumulative sum may step over a boundary that float64 does not; that is rare
     assert hits >= 6 * trials - 3
+    # large vocabularies are drawn from in pieces: the pick's interval of the cumulative distribution (float64)
+    # holds the target within float32 rounding; a stretch without weight as long as a piece changes nothing
+    from distie_amd.sampling import uniform_of
+    for rows, vocab, scale in ((3, 151936, 1.0), (70, 40001, 4.0), (64, 151936, 6.0), (1, 151936, 3.0)):
+        logits = rand(rows, vocab, seed=10 + rows, scale=scale)
+        logits[0, 5000:30000] = -float("inf")
+        temps = torch.tensor([(0.0, 0.7, 1.0, 1.6)[(i + 1) % 4] for i in range(rows)], device="cuda")
+        seeds = torch.arange(rows, device="cuda", dtype=torch.int64) * 77 + 5
+        counters = torch.arange(rows, device="cuda", dtype=torch.int64) + 3
+        got = ops.sample(logits, temps, seeds, counters).tolist()
+        for i, (row, t) in enumerate(zip(logits.double().cpu(), temps.tolist())):
+            if t <= 0:
+                assert got[i] == int(row.argmax())
+                continue
+            w = torch.exp((row - row.max()) / t)
+            c = torch.cumsum(w, 0) / w.sum()
+            u = uniform_of(int(seeds[i]), int(counters[i]))
+            below = float(c[got[i] - 1]) if got[i] else 0.0
+            assert w[got[i]] > 0 and below - 1e-5 <= u <= float(c[got[i]]) + 1e-5, (rows, vocab, i, got[i])
     # the draws follow the distribution: chi-square-free check on a small vocabulary
     small = torch.tensor([[0.0, 1.0, 2.0, -1.0]], device="cuda").repeat(4000, 1)
     draws = ops.sample(small, torch.ones(4000, device="cuda"), torch.full((4000,), 12345, device="cuda", dtype=torch.int64),
