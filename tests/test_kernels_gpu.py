@@ -499,6 +499,24 @@ def test_silu_mul_and_gather(ops, dtype):
     assert torch.equal(ops.gather_rows(x, rows), x[rows.long()])
 
 
+def test_upload_of_small_host_arrays(ops):
+    """More uploads in a row than there are staging buffers, of several types and sizes (one beyond a
+    buffer's first size): each arrives as it was, whatever was uploaded after it."""
+    rng = np.random.default_rng(0)
+    sent = []
+    for i in range(3 * ops.UPLOAD_BUFFERS + 1):
+        dtype = (np.int32, np.int64, np.float32)[i % 3]
+        n = (1, 7, 64, 3000)[i % 4]
+        values = (rng.standard_normal(n) * 1000).astype(dtype)
+        sent.append((values, ops.upload(values)))
+    sent.append((np.zeros((0,), np.int32), ops.upload(np.zeros((0,), np.int32))))
+    sent.append((np.arange(12, dtype=np.int64).reshape(3, 4), ops.upload(np.arange(12, dtype=np.int64).reshape(3, 4))))
+    for values, dev in sent:
+        assert dev.device.type == "cuda" and tuple(dev.shape) == values.shape
+        assert dev.dtype == torch.from_numpy(np.empty(0, values.dtype)).dtype
+        assert np.array_equal(dev.cpu().numpy(), values)
+
+
 def test_argmax_and_sample(ops):
     logits = rand(6, 1001, seed=8, scale=2.0)
     logits[1, 7] = logits[1, 900] = 50.0          # equals: the lowest index wins
