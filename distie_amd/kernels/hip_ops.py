@@ -512,49 +512,30 @@ class HipOps(Ops):
         out = torch.empty((T, num_heads * head_dim), dtype=qkv.dtype, device=self.device)
         bf16 = qkv.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16
         if bf16 and meta.block_size % 16 == 0:
-            group = num_heads // num_kv_heads
-            singles = meta.num_requests if meta.all_decode else 0
-            if not meta.all_decode and meta.host_cu_q is not None:
-                singles = int((meta.host_cu_q[1:] - meta.host_cu_q[:-1] == 1).sum())
-            split_decode = singles > 0 and group <= lib.distie_attention_decode_columns()
-            if split_decode:
-                # requests that bring one token: keys are cut into runs, one wave each, so that the chip is
-                # filled even when few requests decode. The kernel cuts every request's visible keys (counted
-                # from a 64-key boundary) into at most `max_splits` runs by the request's own length; the length
-                # of the longest request's runs is passed along as a hint for the first lookups of pages.
-                visible = min(meta.max_kv, int(window) + 63) if window else meta.max_kv
-                max_splits = max(1, min(self.DECODE_MAX_RUNS, self.DECODE_WAVES // (singles * num_kv_heads),
-                                        -(-visible // 64)))
-                split_len = -(-visible // (64 * max_splits)) * 64
-                part_o = torch.empty((meta.num_requests, num_heads, max_splits, head_dim), dtype=torch.float32,
-                                     device=self.device)
-                part_ml = torch.empty((meta.num_requests, num_heads, max_splits, 2), dtype=torch.float32,
-                                      device=self.device)
+            # how the step is launched, and its buffers for partial results, are the same for every layer
+            # with these sizes: worked out once per step (the layers run one after the other, so they can
+            # share the buffers)
+            key = ("attention", int(window or 0), num_heads, num_kv_heads, head_dim, meta.max_kv, meta.all_decode,
+                   self.PREFILL_PARTS, self.DECODE_WAVES, self.DECODE_MAX_RUNS)
+            plan = meta.scratch.get(key)
+            if plan is None or plan["cu_q"] is not meta.host_cu_q:
+                plan = meta.scratch[key] = self._attention_plan(lib, meta, T, num_heads, num_kv_heads, head_dim, window)
+            if plan["decode"]:
                 _check(lib.distie_attention_decode_bf16(
                     qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), meta.kv_len.data_ptr(),
-                    meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], out.data_ptr(), part_o.data_ptr(),
-                    part_ml.data_ptr(), meta.num_requests, num_heads, num_kv_heads, meta.block_size, float(scale),
-                    int(window or 0), split_len, max_splits, 1 if meta.all_decode else 0, self._stream()),
-                    "attention_decode_bf16")
-            if singles < meta.num_requests or not split_decode:
-                # portions of prompts (and single tokens too, if the decode kernel did not take them). Long
-                # walks over the keys are cut into parts that run side by side.
-                visible = min(meta.max_kv, int(window) + 128) if window else meta.max_kv
-                parts = 1
-                for keys, cut in self.PREFILL_PARTS:
-                    if visible >= keys:
-                        parts = cut
-                part_o = part_ml = None
-                if parts > 1:
-                    part_o = torch.empty((parts, T, num_heads, head_dim), dtype=torch.float32, device=self.device)
-                    part_ml = torch.empty((parts, T, num_heads, 2), dtype=torch.float32, device=self.device)
+                    meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], out.data_ptr(),
+                    plan["decode_o"].data_ptr(), plan["decode_ml"].data_ptr(), meta.num_requests, num_heads,
+                    num_kv_heads, meta.block_size, float(scale), int(window or 0), plan["split_len"],
+                    plan["max_splits"], 1 if meta.all_decode else 0, self._stream()), "attention_decode_bf16")
+            if plan["prefill"]:
+                parts = plan["parts"]
                 _check(lib.distie_attention_prefill_bf16(
                     qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), meta.positions.data_ptr(),
                     meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], out.data_ptr(), T, meta.num_requests,
                     num_heads, num_kv_heads, meta.block_size, float(scale), int(window or 0),
-                    2 if split_decode else 1, meta.token_request.data_ptr(),
-                    part_o.data_ptr() if parts > 1 else None, part_ml.data_ptr() if parts > 1 else None, parts,
-                    self._stream()),
+                    2 if plan["decode"] else 1, meta.token_request.data_ptr(),
+                    plan["prefill_o"].data_ptr() if parts > 1 else None,
+                    plan["prefill_ml"].data_ptr() if parts > 1 else None, parts, self._stream()),
                     "attention_prefill_bf16")
             return out
         _check(lib.distie_attention_generic(
@@ -563,6 +544,41 @@ class HipOps(Ops):
             out.data_ptr(), T, num_heads, num_kv_heads, meta.block_size, float(scale), int(window or 0),
             self._stream()), "attention_generic")
         return out
+
+    def _attention_plan(self, lib, meta: BatchMeta, T, num_heads, num_kv_heads, head_dim, window) -> dict:
+        group = num_heads // num_kv_heads
+        singles = meta.num_requests if meta.all_decode else 0
+        if not meta.all_decode and meta.host_cu_q is not None:
+            singles = int((meta.host_cu_q[1:] - meta.host_cu_q[:-1] == 1).sum())
+        plan = {"cu_q": meta.host_cu_q, "decode": singles > 0 and group <= lib.distie_attention_decode_columns()}
+        if plan["decode"]:
+            # requests that bring one token: keys are cut into runs, one wave each, so that the chip is
+            # filled even when few requests decode. The kernel cuts every request's visible keys (counted
+            # from a 64-key boundary) into at most `max_splits` runs by the request's own length; the length
+            # of the longest request's runs is passed along as a hint for the first lookups of pages.
+            visible = min(meta.max_kv, int(window) + 63) if window else meta.max_kv
+            max_splits = max(1, min(self.DECODE_MAX_RUNS, self.DECODE_WAVES // (singles * num_kv_heads),
+                                    -(-visible // 64)))
+            plan["max_splits"] = max_splits
+            plan["split_len"] = -(-visible // (64 * max_splits)) * 64
+            plan["decode_o"] = torch.empty((meta.num_requests, num_heads, max_splits, head_dim), dtype=torch.float32,
+                                           device=self.device)
+            plan["decode_ml"] = torch.empty((meta.num_requests, num_heads, max_splits, 2), dtype=torch.float32,
+                                            device=self.device)
+        plan["prefill"] = singles < meta.num_requests or not plan["decode"]
+        if plan["prefill"]:
+            # portions of prompts (and single tokens too, if the decode kernel did not take them). Long
+            # walks over the keys are cut into parts that run side by side.
+            visible = min(meta.max_kv, int(window) + 128) if window else meta.max_kv
+            parts = 1
+            for keys, cut in self.PREFILL_PARTS:
+                if visible >= keys:
+                    parts = cut
+            plan["parts"] = parts
+            if parts > 1:
+                plan["prefill_o"] = torch.empty((parts, T, num_heads, head_dim), dtype=torch.float32, device=self.device)
+                plan["prefill_ml"] = torch.empty((parts, T, num_heads, 2), dtype=torch.float32, device=self.device)
+        return plan
 
     def silu_mul(self, gate_up):
         slices, source, dtype = 1, gate_up, gate_up.dtype
