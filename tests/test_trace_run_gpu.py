@@ -99,9 +99,15 @@ def test_replay_step_without_wanted_rows_and_a_pause(tmp_path):
     assert replay.run([{"id": "a", "tokens": ids[:7], "want": []}]) is None
     replay.run([{"id": "b", "tokens": other, "want": [5]}], end=["b"])          # a sits out
     logits = replay.run([{"id": "a", "tokens": ids[7:], "want": [0, 12]}], end=["a"])
-    replay.close()
     want = oracle(weights, cfg, ids)
     assert (logits - want[[7, 19]]).abs().max() < 1e-4
+    # a name that was given back names a new request; a request may be ended by a step it sits out
+    replay.run([{"id": "a", "tokens": other[:4], "want": []}, {"id": "c", "tokens": ids[:3], "want": []}])
+    again = replay.run([{"id": "a", "tokens": other[4:], "want": [1]}], end=["c"])
+    assert (again - oracle(weights, cfg, other)[[5]]).abs().max() < 1e-4
+    last = replay.run([{"id": "c", "tokens": other, "want": [5]}], end=["a", "c"])
+    assert (last - oracle(weights, cfg, other)[[5]]).abs().max() < 1e-4
+    replay.close()
 
 
 def test_generation_through_the_entry_point_and_the_command_line(tmp_path):
