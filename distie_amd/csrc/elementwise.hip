@@ -108,7 +108,7 @@ __global__ __launch_bounds__(1024) void rmsnorm_vec_kernel(float* __restrict__ r
                                                            const W* __restrict__ weight, O* __restrict__ out, int width,
                                                            float eps) {
   __shared__ float scratch[16];
-  constexpr int GROUP = 8;                     // slices loaded together
+  constexpr int GROUP = 8;                     // slices loaded together (16 changes nothing: 4.2 us at 14 slices)
   const int64_t row = blockIdx.x;
   const int quads = width / 4;
   float4 v[NV], wq[NV];
@@ -121,7 +121,9 @@ __global__ __launch_bounds__(1024) void rmsnorm_vec_kernel(float* __restrict__ r
     const float4 x4 = *reinterpret_cast<const float4*>(residual + at);
     wq[e] = load_weights4(weight + 4 * (in ? q : 0));
     float4 sum = {0.f, 0.f, 0.f, 0.f};
-    if (delta != nullptr) {
+    if (delta != nullptr && slices == 1) {
+      sum = load_weights4(delta + at);
+    } else if (delta != nullptr) {
       const int last = slices - 1;
       for (int s0 = 0; s0 < slices; s0 += GROUP) {
         float4 part[GROUP];
