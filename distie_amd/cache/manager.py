@@ -175,7 +175,20 @@ class CacheManager:
             out.append(max(0, last - first))
         return out
 
+    def _holds(self, entry: Optional[RequestCache], num_new: int) -> bool:
+        """The request's tables already reach over its next `num_new` positions (most decoded tokens:
+        one in `block_size` needs a page)."""
+        if entry is None:
+            return False
+        last = pages_needed(entry.num_cached + num_new, self.block_size)
+        for table in entry.tables:
+            if len(table) < last:
+                return False
+        return True
+
     def can_reserve(self, request_id, num_new: int, spare: int = 0) -> bool:
+        if spare <= 0 and self._holds(self._requests.get(request_id), num_new):
+            return True
         return all(short + spare <= group.pool.num_free
                    for short, group in zip(self.pages_short(request_id, num_new), self.groups))
 
@@ -185,6 +198,8 @@ class CacheManager:
         if num_new < 1:
             raise ValueError("num_new must be >= 1")
         entry = self._requests[request_id]
+        if self._holds(entry, num_new):
+            return
         short = self.pages_short(request_id, num_new)
         for need, group in zip(short, self.groups):
             if need > group.pool.num_free:

@@ -91,26 +91,44 @@ class BatchBuilder:
             past = state.num_cached
             if past + n > self.max_model_len:
                 raise ValueError(f"request {entry.request_id!r}: {past + n} tokens exceed the limit of {self.max_model_len}")
-            toks = np.asarray(entry.tokens, dtype=np.int64)
-            if toks.min() < 0 or toks.max() >= self.vocab_size:
-                raise ValueError(f"request {entry.request_id!r}: token id outside 0..{self.vocab_size - 1}")
-            ids[t0:t0 + n] = toks
-            pos = np.arange(past, past + n, dtype=np.int64)
-            positions[t0:t0 + n] = pos
-            token_request[t0:t0 + n] = b
             cu_q[b + 1] = t0 + n
             kv_len[b] = past + n
             slots_state[b] = state.slot
             host_past[b] = past
-            for g in range(G):
-                table = np.asarray(state.tables[g], dtype=np.int64)
-                if len(table) * P < past + n:
-                    raise ValueError(f"request {entry.request_id!r}: pages were not reserved for this step")
-                tables[g][b, :len(table)] = table
-                pages = table[pos // P]
-                if (pages < 0).any():
-                    raise AssertionError("a new token would be written to a page that was given back")
-                slots[g][t0:t0 + n] = pages * P + pos % P
+            if n == 1:
+                # a decoded token: the same as below without an array per field (most rows of most steps)
+                tok = int(entry.tokens[0])
+                if tok < 0 or tok >= self.vocab_size:
+                    raise ValueError(f"request {entry.request_id!r}: token id outside 0..{self.vocab_size - 1}")
+                ids[t0] = tok
+                positions[t0] = past
+                token_request[t0] = b
+                for g in range(G):
+                    table = state.tables[g]
+                    if len(table) * P <= past:
+                        raise ValueError(f"request {entry.request_id!r}: pages were not reserved for this step")
+                    page = table[past // P]
+                    if page < 0:
+                        raise AssertionError("a new token would be written to a page that was given back")
+                    tables[g][b, :len(table)] = table
+                    slots[g][t0] = page * P + past % P
+            else:
+                toks = np.asarray(entry.tokens, dtype=np.int64)
+                if toks.min() < 0 or toks.max() >= self.vocab_size:
+                    raise ValueError(f"request {entry.request_id!r}: token id outside 0..{self.vocab_size - 1}")
+                ids[t0:t0 + n] = toks
+                pos = np.arange(past, past + n, dtype=np.int64)
+                positions[t0:t0 + n] = pos
+                token_request[t0:t0 + n] = b
+                for g in range(G):
+                    table = np.asarray(state.tables[g], dtype=np.int64)
+                    if len(table) * P < past + n:
+                        raise ValueError(f"request {entry.request_id!r}: pages were not reserved for this step")
+                    tables[g][b, :len(table)] = table
+                    pages = table[pos // P]
+                    if (pages < 0).any():
+                        raise AssertionError("a new token would be written to a page that was given back")
+                    slots[g][t0:t0 + n] = pages * P + pos % P
             if not want_all:
                 for w in entry.want:
                     if not 0 <= int(w) < n:
