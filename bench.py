@@ -20,7 +20,7 @@ sys.path.insert(0, str(Path(__file__).resolve().parent))
 HBM_PEAK_GBS = 8000.0
 PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
 
-# BASELINE.json configs[2]
+# the layer sizes of Qwen2.5-1.5B, the configuration the headline figures are quoted on
 SHAPE = {
     "architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 28, "hidden_size": 1536,
     "num_attention_heads": 12, "num_key_value_heads": 2, "head_dim": 128, "intermediate_size": 8960,
