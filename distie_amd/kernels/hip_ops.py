@@ -91,6 +91,7 @@ class HipOps(Ops):
     # many parts that run side by side (measured at 12 heads of 128, 2,048 new tokens: 3 parts are best up to
     # 4,096 keys, 5 at 8,192, 8 from 16,384 on; the kernel takes up to 16)
     PREFILL_PARTS = ((1024, 3), (8192, 5), (16384, 8))
+    PREFILL_WORKGROUPS = 512         # as many workgroups a short portion's attention should have, if its keys allow
     # decode attention cuts the keys into runs so that about DECODE_WAVES waves are at work, with at most
     # DECODE_MAX_RUNS places for partial results per request and head
     DECODE_WAVES = 1024
@@ -516,7 +517,7 @@ class HipOps(Ops):
             # with these sizes: worked out once per step (the layers run one after the other, so they can
             # share the buffers)
             key = ("attention", int(window or 0), num_heads, num_kv_heads, head_dim, meta.max_kv, meta.all_decode,
-                   self.PREFILL_PARTS, self.DECODE_WAVES, self.DECODE_MAX_RUNS)
+                   self.PREFILL_PARTS, self.PREFILL_WORKGROUPS, self.DECODE_WAVES, self.DECODE_MAX_RUNS)
             plan = meta.scratch.get(key)
             if plan is None or plan["cu_q"] is not meta.host_cu_q:
                 plan = meta.scratch[key] = self._attention_plan(lib, meta, T, num_heads, num_kv_heads, head_dim, window)
@@ -574,6 +575,11 @@ class HipOps(Ops):
             for keys, cut in self.PREFILL_PARTS:
                 if visible >= keys:
                     parts = cut
+            # few new tokens make few workgroups (one per 128 tokens of a request and head), each walking all
+            # the keys alone: more parts then, down to 128 keys a part
+            tiles = -(-T // 128) + meta.num_requests
+            wanted = -(-self.PREFILL_WORKGROUPS // (tiles * num_heads))
+            parts = max(parts, min(wanted, visible // 128, 16))
             plan["parts"] = parts
             if parts > 1:
                 plan["prefill_o"] = torch.empty((parts, T, num_heads, head_dim), dtype=torch.float32, device=self.device)
