@@ -37,6 +37,7 @@ CXX_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-pthread"]
 OPS_SOURCES = ["elementwise.hip", "gemm.hip", "sampling.hip"]
 ATTN_SOURCES = ["attention.hip"]
 HEADERS = ["common.h"]
+OPS_HEADERS = ["no_alloc.h"]
 
 
 class BuildError(RuntimeError):
@@ -49,7 +50,8 @@ def _say(text: str) -> None:
 
 def _hash(files: List[str], flags: List[str]) -> str:
     h = hashlib.sha256()
-    for name in files + HEADERS:
+    headers = HEADERS + (OPS_HEADERS if files == OPS_SOURCES else [])
+    for name in files + headers:
         path = SRC / name
         if path.is_file():
             h.update(name.encode())

@@ -9,6 +9,9 @@
 //           cumulative weight exceeds u * total.
 
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 #define SAMPLE_THREADS 256
 
@@ -105,6 +108,61 @@ extern "C" int distie_argmax(const float* logits, int32_t* out, int rows, int vo
     return launch_status();
   }
   if (piece_value == nullptr || piece_index == nullptr) return DISTIE_BAD_ARGUMENT;
+  const int piece_len = (vocab + parts - 1) / parts;
+  argmax_pieces_kernel<<<dim3(parts, rows), SAMPLE_THREADS, 0, stream>>>(logits, piece_value, piece_index, vocab, piece_len);
+  argmax_combine_kernel<<<rows, DISTIE_WAVE, 0, stream>>>(piece_value, piece_index, out, parts, vocab);
+  return launch_status();
+}
+
+// ---- the same pick with the scratch in a device array of this file (see no_alloc.h)
+//
+// In host code `scratch` is only a stand-in for the device array: its address on a device comes from
+// hipGetSymbolAddress, once per device with that device current, and only that address is handed to kernels.
+static __device__ __align__(256) unsigned char scratch[DISTIE_ARGMAX_STATIC_ENTRIES * (sizeof(float) + sizeof(int32_t))];
+
+constexpr int STATIC_MAX_DEVICES = 64;
+static void* scratch_of_device[STATIC_MAX_DEVICES];
+static std::mutex scratch_lookup;
+
+// -> 0 and the array's address on the current device, or a hipError_t
+static int static_scratch(void** address) {
+  int device = -1;
+  hipError_t status = hipGetDevice(&device);
+  if (status != hipSuccess) return static_cast<int>(status);
+  if (device < 0 || device >= STATIC_MAX_DEVICES) return static_cast<int>(hipErrorInvalidDevice);
+  std::lock_guard<std::mutex> hold(scratch_lookup);
+  if (scratch_of_device[device] == nullptr) {
+    void* found = nullptr;
+    status = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+    if (status != hipSuccess) return static_cast<int>(status);
+    if (found == nullptr) return static_cast<int>(hipErrorInvalidSymbol);
+    scratch_of_device[device] = found;
+  }
+  *address = scratch_of_device[device];
+  return 0;
+}
+
+extern "C" void distie_argmax_static_limits(int* max_rows, int* max_entries) {
+  if (max_rows != nullptr) *max_rows = DISTIE_ARGMAX_STATIC_MAX_ROWS;
+  if (max_entries != nullptr) *max_entries = DISTIE_ARGMAX_STATIC_ENTRIES;
+}
+
+extern "C" int distie_argmax_static(const float* logits, int32_t* out, int rows, int vocab, hipStream_t stream) {
+  if (rows < 0 || vocab <= 0 || (rows > 0 && (logits == nullptr || out == nullptr))) return DISTIE_BAD_ARGUMENT;
+  if (rows == 0) return 0;
+  if (rows > DISTIE_ARGMAX_STATIC_MAX_ROWS) return DISTIE_TOO_LARGE;
+  const int parts = distie_argmax_parts(rows, vocab);
+  if (parts == 1) {
+    argmax_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, out, vocab);
+    return launch_status();
+  }
+  if (static_cast<int64_t>(rows) * parts > DISTIE_ARGMAX_STATIC_ENTRIES) return DISTIE_TOO_LARGE;
+  void* base = nullptr;
+  const int status = static_scratch(&base);
+  if (status != 0) return status;
+  // every entry that the second launch reads is written by the first: nothing has to be cleared
+  float* piece_value = static_cast<float*>(base);
+  int32_t* piece_index = reinterpret_cast<int32_t*>(piece_value + DISTIE_ARGMAX_STATIC_ENTRIES);
   const int piece_len = (vocab + parts - 1) / parts;
   argmax_pieces_kernel<<<dim3(parts, rows), SAMPLE_THREADS, 0, stream>>>(logits, piece_value, piece_index, vocab, piece_len);
   argmax_combine_kernel<<<rows, DISTIE_WAVE, 0, stream>>>(piece_value, piece_index, out, parts, vocab);
