@@ -56,7 +56,7 @@ def decode_run(llm, batch, steps, warmup, vocab, seed):
     # requests admitted early decode while later prompts are still prefilled: leave room for that
     params = SamplingParams(max_new_tokens=warmup + steps + 2 * batch + 8, ignore_eos=True)
     ids = [llm.add_request(p, params) for p in prompts(batch, CONTEXT, vocab, seed)]
-    seqs = [llm.scheduler._ids[i] for i in ids]
+    seqs = [llm.scheduler.request(i) for i in ids]
     while any(len(s.output_ids) == 0 for s in seqs):      # prefill, in portions under the token budget
         llm.run_step()
     for _ in range(warmup):

@@ -2,7 +2,7 @@ from .batch import StepEntry
 from .llm import LLM, RequestOutput, Trace
 from .model import Model
 from .runner import ModelRunner
-from .scheduler import BlockPoolExhausted, Emission, Scheduler, Sequence, SeqState, StepPlan
+from .scheduler import BlockPoolExhausted, Emission, Scheduler, Phase, Portion, Request, StepPlan
 
 __all__ = ["StepEntry", "LLM", "RequestOutput", "Trace", "Model", "ModelRunner", "BlockPoolExhausted",
-           "Emission", "Scheduler", "Sequence", "SeqState", "StepPlan"]
+           "Emission", "Scheduler", "Phase", "Portion", "Request", "StepPlan"]

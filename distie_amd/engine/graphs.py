@@ -7,8 +7,9 @@ own fixed device buffers that the graph reads (tokens, positions, tables, slots)
 logits; rows added to fill the bucket write to the sink page; a bucket is captured the first
 time it is used, after one ordinary run with the same buffers (so that scratch memory has
 its size and the first result is right), and replayed from then on. If capture or replay
-fails, graphs are dropped for good and the step runs the ordinary way, which writes the same
-cache slots again.
+fails, the graphs and the memory pool they share are dropped, the step runs the ordinary way
+(which writes the same cache slots again), and so do the next decode steps; later a capture is
+tried again, and after a few failures captured steps stay off. Failures are counted and logged.
 
 The step's metadata reaches the device with one copy from pinned host memory before the
 replay; nothing inside the graph depends on a Python number.
@@ -85,6 +86,9 @@ class _Bucket:
 class DecodeGraphs:
     FIRST_CONTEXT = 1024        # the shortest class of context length
 
+    RETRY_AFTER_STEPS = 512     # after a failure, steps run uncaptured for so long before a capture is tried again
+    MAX_FAILURES = 3            # ... and after so many failures for good
+
     def __init__(self, runner, max_batch: int) -> None:
         self.runner = runner
         self.buckets = decode_buckets(max_batch)
@@ -92,8 +96,14 @@ class DecodeGraphs:
         self.max_batch = max_batch
         self._made: Dict[int, _Bucket] = {}
         self._pool = None
-        self.failed = False
         self.replays = 0
+        self.failures = 0           # captures or replays that raised
+        self._resting = 0           # decode steps still to run uncaptured after a failure
+
+    @property
+    def failed(self) -> bool:
+        """Captured steps are switched off, for now or for good."""
+        return self._resting > 0 or self.failures >= self.MAX_FAILURES
 
     @property
     def captured(self) -> List[int]:
@@ -105,20 +115,26 @@ class DecodeGraphs:
         """(batch size, context class) of every graph."""
         return sorted((size, limit) for size, b in self._made.items() for limit in b.graphs)
 
+    def drop(self) -> None:
+        """Forget every graph *and* the memory pool they were captured into. The two go together: graphs
+        that are destroyed while their pool lives on leave the allocator with blocks that belong to no
+        graph, and the next capture into that pool ends in its internal assertion
+        (`use_count > 0`)."""
+        self._made.clear()
+        self._pool = None
+
     def try_run(self, entries: Sequence[StepEntry], feed: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Logits [wanted, vocab] if this step went through a graph, None if it must run the
-        ordinary way (not a pure decode step, too many rows, or graphs have failed)."""
-        if self.failed or len(entries) > self.max_batch or any(len(e.tokens) != 1 for e in entries):
+        ordinary way (not a pure decode step, too many rows, or captured steps are switched off).
+        What is wrong with the entries themselves (a token id out of range, pages not reserved) raises
+        as it does in an ordinary step and switches nothing off."""
+        if len(entries) > self.max_batch or any(len(e.tokens) != 1 for e in entries):
             return None
-        try:
-            return self._run(entries, feed)
-        except Exception:  # noqa: BLE001 - the ordinary path rewrites the same slots
-            _log.exception("captured decode step failed; all steps run uncaptured from now on")
-            self.failed = True
-            self._made.clear()
+        if self.failures >= self.MAX_FAILURES:
             return None
-
-    def _run(self, entries: Sequence[StepEntry], feed: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+        if self._resting > 0:
+            self._resting -= 1
+            return None
         runner = self.runner
         size = bucket_for(self.buckets, len(entries))
         bucket = self._made.get(size)
@@ -126,6 +142,21 @@ class DecodeGraphs:
             bucket = self._made[size] = _Bucket(size, runner.builder, runner.ops.device)
         bucket.copied.synchronize()                      # the previous copy out of the pinned buffer is done
         max_kv = runner.builder.fill(bucket.host_np, entries, pad_requests=size - len(entries), want_all=True)[5]
+        try:
+            return self._run(bucket, entries, feed, max_kv)
+        except Exception:  # noqa: BLE001 - the ordinary path rewrites the same slots
+            self.failures += 1
+            self._resting = self.RETRY_AFTER_STEPS
+            self.drop()
+            _log.exception("captured decode step failed (failure %d of %d allowed): graphs and their memory pool "
+                           "are dropped, steps run uncaptured %s", self.failures, self.MAX_FAILURES,
+                           "from now on" if self.failures >= self.MAX_FAILURES
+                           else f"for the next {self.RETRY_AFTER_STEPS} decode steps")
+            return None
+
+    def _run(self, bucket: _Bucket, entries: Sequence[StepEntry], feed: Optional[torch.Tensor],
+             max_kv: int) -> Optional[torch.Tensor]:
+        runner = self.runner
         bucket.dev.copy_(bucket.host, non_blocking=True)
         bucket.copied.record()
         if feed is not None and feed.shape[0]:

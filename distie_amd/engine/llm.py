@@ -24,12 +24,12 @@ import torch
 
 from ..cache.manager import CacheManager
 from ..config import EngineConfig, config_from_dict, load_model_config
-from ..sampling import Sampler, SamplingParams
+from ..sampling import Sampler, SamplingParams, derive_seed
 from ..weights import load_into, random_into
 from .batch import StepEntry
 from .model import Model
 from .runner import ModelRunner
-from .scheduler import Emission, Scheduler, Sequence, SeqState, StepPlan
+from .scheduler import Emission, Phase, Request, Scheduler, StepPlan
 from .stats import StepStats
 
 _log = logging.getLogger(__name__)
@@ -51,6 +51,7 @@ class RequestOutput:
     preemptions: int = 0
     time_to_first_token_ms: float = 0.0
     total_latency_ms: float = 0.0
+    arrival_time: float = 0.0                # time.perf_counter() at add_request
 
 
 @dataclass(frozen=True)
@@ -68,8 +69,11 @@ class LLM:
                  **options) -> None:
         """`model`: a folder with config.json and model.safetensors. Without it, `config` (a typed
         configuration or the dict of a config.json) and `random_weights=True` make a model with
-        random weights on the device. `options` are fields of `EngineConfig`. `ops` is the kernel
+        random weights on the device (drawn from `seed`, which is also the engine's seed for sampling
+        unless `options` or `engine` name another). `options` are fields of `EngineConfig`. `ops` is the kernel
         surface; by default the HIP kernels, which need the GPU."""
+        if engine is None:
+            options.setdefault("seed", seed)          # one seed for random weights and for the requests' draws
         self.engine_config = engine or EngineConfig(**options)
         self.dtype = TORCH_DTYPES[self.engine_config.dtype]
         if ops is None:
@@ -98,15 +102,14 @@ class LLM:
         self.runner = ModelRunner(self.model, self.cache, ops, self.dtype, self.max_model_len)
         self.scheduler = Scheduler(self.cache, ec.max_seqs, ec.token_budget, self.max_model_len)
         self.sampler = Sampler(ops)
-        self.stats = StepStats(ec.step_stats) if ec.step_stats else None
+        self.stats = StepStats(ec.step_stats, device_events=ops.device.type == "cuda") if ec.step_stats else None
         self.eos_ids = tuple(spec.eos_token_ids)
         self._counter = itertools.count()
-        self._ahead = None            # (plan, logits) of a step that is launched and not yet completed
+        self._ahead = None            # (plan, logits, events) of a step that is launched and not yet completed
         self._picked = None           # pinned host buffer for the sampled ids
         self._ahead_failed = None     # (plan, error) of a step planned ahead whose launch raised
         self.steps_ahead = 0          # steps launched before the tokens of the step before were known
-        self._outputs: Dict[Hashable, RequestOutput] = {}
-        self._started: Dict[Hashable, float] = {}
+        self._outputs: Dict[Hashable, RequestOutput] = {}     # until `generate`, `stream` or `take_output` hands them out
         if ec.use_graphs and hasattr(ops, "graphs_supported") and ops.graphs_supported():
             from .graphs import DecodeGraphs
 
@@ -149,27 +152,46 @@ class LLM:
     def add_request(self, prompt_ids: Seq[int], params: Optional[SamplingParams] = None,
                     request_id: Optional[Hashable] = None) -> Hashable:
         params = params or SamplingParams()
+        arrival = next(self._counter)
         if request_id is None:
-            request_id = f"req-{next(self._counter)}"
+            request_id = f"req-{arrival}"
         prompt = [int(t) for t in prompt_ids]
         vocab = self.model.spec.vocab_size
         if any(t < 0 or t >= vocab for t in prompt):
             raise ValueError(f"token id outside 0..{vocab - 1}")
         eos = (params.eos_id,) if params.eos_id is not None else self.eos_ids
-        seq = Sequence(request_id=request_id, prompt_ids=prompt, params=params, eos_ids=tuple(eos))
-        self.scheduler.submit(seq)
-        self._outputs[request_id] = RequestOutput(request_id, prompt)
-        self._started[request_id] = time.perf_counter()
+        # A request without a seed of its own draws from a stream that belongs to it alone: derived from the
+        # engine's seed and the request's place in the order of arrival, so that two requests never share
+        # their random numbers (the reference draws from one global generator:
+        # worker/src/inference/model_runner.py:122-130) and a rerun of the same arrivals repeats.
+        seed = params.seed if params.seed is not None else derive_seed(self.engine_config.seed, arrival)
+        request = Request(request_id=request_id, prompt_ids=prompt, params=params, eos_ids=tuple(eos), seed=seed)
+        self.scheduler.submit(request)
+        self._outputs[request_id] = RequestOutput(request_id, prompt, arrival_time=time.perf_counter())
         return request_id
 
     def abort(self, request_id) -> None:
         self.scheduler.abort(request_id)
         out = self._outputs.get(request_id)
         if out is not None and not out.finished:
-            out.finished, out.finish_reason = True, "abort"
+            self._close(out, "abort")
+
+    def take_output(self, request_id) -> RequestOutput:
+        """The record of a request, which the engine then forgets. `generate` and `stream` do this for their
+        own requests; who drives `add_request` and `run_step` takes the records of finished requests here."""
+        return self._outputs.pop(request_id)
 
     def has_work(self) -> bool:
         return self.scheduler.has_work()
+
+    @staticmethod
+    def _close(out: RequestOutput, reason: str, error: Optional[str] = None) -> None:
+        out.finished, out.finish_reason, out.error = True, reason, error
+        out.total_latency_ms = (time.perf_counter() - out.arrival_time) * 1e3
+
+    def _fail(self, plan: StepPlan, exc: BaseException) -> None:
+        for request in self.scheduler.fail(plan, exc):
+            self._close(self._outputs[request.request_id], "error", repr(exc))
 
     def run_step(self) -> List[Emission]:
         """One turn of the loop: schedule, step, sample, complete.
@@ -179,72 +201,85 @@ class LLM:
         on the device; the host then waits for this step's tokens while the next step runs, and the
         next turn starts with that step already launched."""
         t0 = time.perf_counter()
-        plan, logits = None, None
+        plan, logits, timing = None, None, None
         if self._ahead is not None:
-            plan, logits = self._ahead
+            plan, logits, timing = self._ahead
             self._ahead = None
-            if not any(it.seq.state is SeqState.RUNNING for it in plan.items):
+            if not any(p.request.phase is Phase.SEATED for p in plan.portions):
                 plan, logits = None, None        # every request of it has ended meanwhile: nothing to take from it
         launched = plan is not None
         if plan is None:
             plan = self.scheduler.schedule()
-            if not plan.items:
+            if not plan.portions:
                 if self.scheduler.num_waiting and not self.scheduler.num_running:
                     raise RuntimeError("the scheduler cannot place the waiting requests: cache too small")
                 return []
         t1 = time.perf_counter()
         try:
             if not launched:
-                logits = self.runner.step(self._entries(plan), reserve=False)
+                logits, timing = self._launch(plan, None)
             t2 = time.perf_counter()
-            sampling = [it for it in plan.items if it.samples]
-            picks: List[Optional[int]] = [None] * len(plan.items)
+            sampling = [p for p in plan.portions if p.samples]
+            drawn: List[Optional[int]] = [None] * len(plan.portions)
             if sampling:
-                seeds = [it.seq.params.seed if it.seq.params.seed is not None else self.engine_config.seed
-                         for it in sampling]
                 chosen = self.sampler.sample_device(
-                    logits, [it.seq.params.temperature for it in sampling], seeds,
-                    [len(it.seq.output_ids) for it in sampling])
+                    logits, [p.request.params.temperature for p in sampling], [p.request.seed for p in sampling],
+                    [len(p.request.output_ids) for p in sampling])
                 fetch = self._to_host(chosen)
                 if self.engine_config.lookahead:
                     self._launch_ahead(plan, chosen)
                 tokens = iter(fetch())
-                picks = [next(tokens) if it.samples else None for it in plan.items]
+                drawn = [next(tokens) if p.samples else None for p in plan.portions]
         except Exception as exc:  # noqa: BLE001 - every request of the step learns of it
-            _log.exception("step failed; its %d requests end with the error", len(plan.items))
-            self._ahead = None
-            for seq in self.scheduler.fail(plan, exc):
-                out = self._outputs[seq.request_id]
-                out.finished, out.finish_reason, out.error = True, "error", repr(exc)
+            _log.exception("step failed; its %d requests end with the error", len(plan.portions))
+            self._fail(plan, exc)
+            self._drop_ahead()
             return []
-        emissions = self.scheduler.complete(plan, picks)
+        emissions = self.scheduler.complete(plan, drawn)
         if self._ahead_failed is not None:
             failed_plan, exc = self._ahead_failed
             self._ahead_failed = None
-            for seq in self.scheduler.fail(failed_plan, exc):
-                out = self._outputs[seq.request_id]
-                out.finished, out.finish_reason, out.error = True, "error", repr(exc)
+            self._fail(failed_plan, exc)
         now = time.perf_counter()
         for e in emissions:
-            out = self._outputs[e.seq.request_id]
+            out = self._outputs[e.request.request_id]
             if out.finished:
                 continue                         # aborted meanwhile
             if not out.token_ids:
-                out.time_to_first_token_ms = (now - self._started[e.seq.request_id]) * 1e3
+                out.time_to_first_token_ms = (now - out.arrival_time) * 1e3
             out.token_ids.append(e.token_id)
-            out.preemptions = e.seq.preemptions
+            out.preemptions = e.request.preemptions
             if e.finished:
-                out.finished, out.finish_reason = True, e.seq.finish_reason
-                out.total_latency_ms = (now - self._started[e.seq.request_id]) * 1e3
+                self._close(out, e.request.finish_reason)
         if self.stats is not None:
-            self.stats.record("decode" if plan.is_decode else "prefill", len(plan.items), plan.num_tokens,
-                              sched=(t1 - t0) * 1e3, gpu=(t2 - t1) * 1e3, emit=(now - t2) * 1e3)
+            # `launch` is the host's time inside the step function when this turn launched the step (0 when it
+            # was launched a turn earlier, behind the step before); `device` is the step's own time on the GPU,
+            # between two events, read when the step after has been queued, so that nothing waits for it
+            self.stats.record("decode" if plan.is_decode else "prefill", len(plan.portions), plan.num_tokens,
+                              timing, sched=(t1 - t0) * 1e3, launch=(t2 - t1) * 1e3, emit=(now - t2) * 1e3)
         return emissions
 
-    @staticmethod
-    def _entries(plan: StepPlan) -> List[StepEntry]:
-        return [StepEntry(it.seq.request_id, it.token_ids, [len(it.token_ids) - 1] if it.samples else [])
-                for it in plan.items]
+    def _launch(self, plan: StepPlan, feed):
+        """-> (logits, the step's pair of events or None)"""
+        entries = [StepEntry(p.request.request_id, p.token_ids, [len(p.token_ids) - 1] if p.samples else [])
+                   for p in plan.portions]
+        timing = self.stats.events() if self.stats is not None else None
+        if timing is not None:
+            timing[0].record()
+        logits = self.runner.step(entries, reserve=False, feed=feed)
+        if timing is not None:
+            timing[1].record()
+        return logits, timing
+
+    def _drop_ahead(self) -> None:
+        """The step in flight failed with a step already launched behind it. That step's results are worth
+        nothing, but it has advanced the cache's counts of its requests: those of them that are still
+        seated (requests that it seated itself) go back to the queue and start over."""
+        if self._ahead is None:
+            return
+        ahead_plan = self._ahead[0]
+        self._ahead = None
+        self.scheduler.requeue(p.request for p in ahead_plan.portions)
 
     def _to_host(self, chosen: torch.Tensor):
         """Start the copy of the sampled ids to the host; the returned function waits for it."""
@@ -270,8 +305,8 @@ class LLM:
             return
         try:
             sampled_row = {}
-            for i, it in enumerate(plan.items):
-                if it.samples:
+            for i, p in enumerate(plan.portions):
+                if p.samples:
                     sampled_row[i] = len(sampled_row)
             rows = [sampled_row[i] for i in ahead.feeds]
             feed = chosen
@@ -280,18 +315,24 @@ class LLM:
             elif rows != list(range(chosen.shape[0])):
                 index = self.ops.upload(np.asarray(rows, dtype=np.int32))
                 feed = self.ops.gather_rows(chosen.view(-1, 1), index).view(-1)
-            self._ahead = (ahead, self.runner.step(self._entries(ahead), reserve=False, feed=feed))
+            self._ahead = (ahead,) + self._launch(ahead, feed)
             self.steps_ahead += 1
         except Exception as exc:  # noqa: BLE001 - its requests learn of it once the running step is completed
-            _log.exception("the step planned ahead failed; its %d requests end with the error", len(ahead.items))
+            _log.exception("the step planned ahead failed; its %d requests end with the error", len(ahead.portions))
             self._ahead = None
             self._ahead_failed = (ahead, exc)
 
     def stream(self, prompts: Seq[Seq[int]], params=None) -> Iterator[Emission]:
         """Yield (request, token, finished) as tokens are produced."""
-        self._submit_all(prompts, params)
+        mine = set(self._submit_all(prompts, params))
         while self.scheduler.has_work():
-            yield from self.run_step()
+            for emission in self.run_step():
+                yield emission
+            for rid in [r for r in mine if self._outputs[r].finished]:
+                mine.discard(rid)
+                del self._outputs[rid]
+        for rid in mine:
+            self._outputs.pop(rid, None)
 
     def generate(self, prompts: Seq[Seq[int]], params=None) -> List[RequestOutput]:
         """Token ids in, `RequestOutput`s out, in the order of the prompts. `params`: one
@@ -312,35 +353,36 @@ class LLM:
 
     # ------------------------------------------------------------ trace
     def trace(self, prompt_ids: Seq[int], max_new_tokens: int, forced_ids: Optional[Seq[int]] = None) -> Trace:
-        """One request through the step function: the whole prompt, then one token a step.
-        Free-running feeds back the greedy pick and stops after an end-of-sequence token;
-        teacher-forced feeds `forced_ids`. Last-position logits of every step are kept
+        """One request through the step function: the whole prompt in one step, then a token a step,
+        keeping the logits at the last position of every step. Without `forced_ids` each step is fed
+        the greedy pick of the one before and the run ends after an end-of-sequence token; with them,
+        step t is fed `forced_ids[t - 1]` whatever was picked, so that the logits can be compared with
+        those of another implementation that saw the same tokens
         (worker/src/inference/torch_engine.py:295-338)."""
-        if not prompt_ids:
-            raise ValueError("prompt_ids must be non-empty")
+        prompt = [int(t) for t in prompt_ids]
+        forced = None if forced_ids is None else [int(t) for t in forced_ids]
+        if len(prompt) == 0:
+            raise ValueError("a trace needs at least one prompt token")
         if max_new_tokens < 1:
-            raise ValueError("max_new_tokens must be >= 1")
-        if forced_ids is not None and len(forced_ids) < max_new_tokens:
-            raise ValueError("forced_ids shorter than max_new_tokens")
-        rid = f"trace-{next(self._counter)}"
-        picks: List[int] = []
-        rows: List[torch.Tensor] = []
-        current = [int(t) for t in prompt_ids]
+            raise ValueError("a trace needs max_new_tokens >= 1")
+        if forced is not None and len(forced) < max_new_tokens:
+            raise ValueError(f"{len(forced)} forced ids for {max_new_tokens} steps")
+        name = f"trace-{next(self._counter)}"
+        kept = torch.empty((max_new_tokens, self.model.spec.vocab_size), dtype=torch.float32)
+        chosen: List[int] = []
+        feed = prompt
         try:
-            for step in range(max_new_tokens):
-                logits = self.runner.step([StepEntry(rid, current, [len(current) - 1])])
-                pick = int(self.ops.argmax(logits)[0])
-                picks.append(pick)
-                rows.append(logits[0].float().cpu())
-                if forced_ids is None:
-                    if pick in self.eos_ids:
-                        break
-                    current = [pick]
-                else:
-                    current = [int(forced_ids[step])]
+            while len(chosen) < max_new_tokens:
+                row = self.runner.step([StepEntry(name, feed, [len(feed) - 1])])
+                greedy = int(self.ops.argmax(row)[0])
+                kept[len(chosen)].copy_(row[0])
+                chosen.append(greedy)
+                if forced is None and greedy in self.eos_ids:
+                    break
+                feed = [greedy if forced is None else forced[len(chosen) - 1]]
         finally:
-            self.runner.finish(rid)
-        return Trace(token_ids=picks, logits=torch.stack(rows))
+            self.runner.finish(name)
+        return Trace(token_ids=chosen, logits=kept[:len(chosen)].clone())
 
     def close(self) -> None:
         self.runner.graphs = None

@@ -1,24 +1,23 @@
-"""Continuous batching: which requests run in the next step, and with which tokens.
+"""Continuous batching: which requests run in the next step, and with which of their tokens.
 
-Bookkeeping only, no tensors. Every step (the order is the reference's,
-worker/src/inference/scheduler.py:141-148):
+Book-keeping only, no tensors. The cache manager owns pages and slots; the scheduler owns the
+*queue* of requests that wait and the *seats* of those that run, and decides, step by step:
 
-1. requests that were aborted are dropped and what they hold is given back;
-2. running requests get their next tokens: one for a request that decodes, the next
-   portion for a prompt that is not yet through. If the pages for them are not there,
-   the newest running request is preempted (its pages and slot go back, it waits at the
-   front of the queue and later recomputes its prompt and the tokens it has produced;
-   it never emits a token twice) until they are, or until the needy request itself
-   was the newest (scheduler.py:182-194, 213-225);
-3. waiting requests are admitted first come first served while there is a seat
-   (`max_seqs`), budget, a state slot and pages for the portion they would run now.
+1. requests that were cancelled leave, and what they hold goes back;
+2. every seated request gets its next *portion*: one token if it decodes, else as much of its
+   prompt as the step's token budget has left. If the pages for a portion are not there, the request
+   seated last gives way (its pages and slot go back, it returns to the head of the queue and later
+   recomputes its prompt and the tokens it has produced; it never emits a token twice), again and
+   again until the pages are there or the needy request itself was the one seated last;
+3. queued requests are seated first come first served while there is a seat (`max_seqs`), budget,
+   a state slot, and pages for everything that is known of them.
 
-Different from the reference: a prompt may be cut. All tokens of a step together stay
-within `token_budget`; decoding requests come first, then prompts in flight, then new
-admissions, and a prompt gets as many tokens as the budget has left (the reference
-never cuts a prompt, so its budget only gates admission: scheduler.py:196-211). Only a
-portion that reaches the end of what is known of the request asks for logits and
-produces a token.
+The order of these three and the policy of giving way are the reference's
+(worker/src/inference/scheduler.py:141-148, 182-225). Different from it: a prompt may be cut. All
+tokens of a step together stay within `token_budget`; decoding requests come first, then prompts in
+flight, then new arrivals, and a prompt gets as many tokens as the budget has left (the reference
+never cuts a prompt, so its budget only gates admission: scheduler.py:196-211). Only a portion that
+reaches the end of what is known of the request asks for logits and produces a token.
 """
 
 from __future__ import annotations
@@ -27,7 +26,7 @@ import enum
 import logging
 from collections import deque
 from dataclasses import dataclass, field
-from typing import Deque, Dict, Hashable, List, Optional, Sequence as Seq, Set
+from typing import Deque, Dict, Hashable, Iterable, List, Optional, Sequence as Seq, Tuple
 
 from ..cache.block_pool import OutOfBlocks
 from ..cache.manager import CacheManager, pages_needed
@@ -40,24 +39,26 @@ class BlockPoolExhausted(OutOfBlocks):
     """A request can never fit the cache (the reference's name: worker/src/inference/engine.py:23)."""
 
 
-class SeqState(enum.Enum):
-    WAITING = "waiting"
-    RUNNING = "running"
-    FINISHED = "finished"
+class Phase(enum.Enum):
+    QUEUED = "queued"       # waits for a seat (new, or gave way and will recompute)
+    SEATED = "seated"       # holds a state slot and pages; takes part in steps
+    ENDED = "ended"         # length reached, end of sequence, cancelled, or failed
 
 
 @dataclass(eq=False)
-class Sequence:
+class Request:
     request_id: Hashable
     prompt_ids: List[int]
     params: SamplingParams = field(default_factory=SamplingParams)
     eos_ids: Seq[int] = ()
+    seed: int = 0                         # of this request's draws, fixed when it was submitted
     output_ids: List[int] = field(default_factory=list)
-    num_computed: int = 0                 # tokens whose keys and values are in the cache
-    state: SeqState = SeqState.WAITING
+    num_computed: int = 0                 # tokens whose keys and values are in the cache, as far as completed steps go
+    phase: Phase = Phase.QUEUED
     preemptions: int = 0
-    finish_reason: Optional[str] = None
+    finish_reason: Optional[str] = None   # "stop" | "length" | "abort" | "error"
     error: Optional[BaseException] = None
+    cancelled: bool = False
 
     @property
     def max_new_tokens(self) -> int:
@@ -65,49 +66,83 @@ class Sequence:
 
     @property
     def num_tokens(self) -> int:
+        """Prompt and produced tokens: all that is known of the request."""
         return len(self.prompt_ids) + len(self.output_ids)
 
     def tokens(self, begin: int, end: int) -> List[int]:
-        n = len(self.prompt_ids)
-        if end <= n:
-            return self.prompt_ids[begin:end]
-        if begin >= n:
-            return self.output_ids[begin - n:end - n]
-        return self.prompt_ids[begin:] + self.output_ids[:end - n]
+        split = len(self.prompt_ids)
+        head = self.prompt_ids[begin:end] if begin < split else []
+        tail = self.output_ids[max(begin - split, 0):end - split] if end > split else []
+        return head + tail
 
 
 @dataclass(frozen=True)
-class ScheduledSeq:
-    seq: Sequence
+class Portion:
+    """A request's share of one step: `token_ids` are its tokens `begin .. begin + len - 1`."""
+
+    request: Request
     token_ids: List[int]
-    past_len: int
-    samples: bool          # this portion ends where the request's known tokens end
+    begin: int
+    samples: bool          # the portion ends where the request's known tokens end: a token is drawn after it
+
+    @property
+    def end(self) -> int:
+        return self.begin + len(self.token_ids)
 
 
 @dataclass(frozen=True)
 class StepPlan:
-    items: tuple
-    # For a step planned ahead (`Scheduler.schedule_ahead`): item i continues the request of item
-    # `feeds[i]` of the step before, whose sampled token is not known to the host yet.
-    feeds: Optional[tuple] = None
+    portions: Tuple[Portion, ...]
+    # For a step planned ahead (`Scheduler.schedule_ahead`): portion i continues the request of portion
+    # `feeds[i]` of the step before, whose drawn token is not known to the host yet.
+    feeds: Optional[Tuple[int, ...]] = None
 
     @property
     def num_tokens(self) -> int:
-        return sum(len(item.token_ids) for item in self.items)
+        return sum(len(p.token_ids) for p in self.portions)
 
     @property
     def is_decode(self) -> bool:
-        return all(len(item.token_ids) == 1 for item in self.items)
+        return all(len(p.token_ids) == 1 for p in self.portions)
 
 
 @dataclass(frozen=True)
 class Emission:
-    seq: Sequence
+    request: Request
     token_id: int
     finished: bool
 
 
+class _Draft:
+    """A step while it is planned: the budget that is left, and the portions chosen so far."""
+
+    def __init__(self, budget: int) -> None:
+        self.left = budget
+        self.portions: List[Portion] = []
+        self.feeds: List[int] = []
+
+    def put(self, request: Request, begin: int, count: int) -> None:
+        """The request's known tokens begin .. begin + count - 1."""
+        self.portions.append(Portion(request, request.tokens(begin, begin + count), begin,
+                                     samples=begin + count == request.num_tokens))
+        self.left -= count
+
+    def put_pending(self, request: Request, begin: int, stand_in: int, place: int) -> None:
+        """One token that is not known yet: the one drawn after portion `place` of the step before."""
+        self.portions.append(Portion(request, [stand_in], begin, samples=True))
+        self.feeds.append(place)
+        self.left -= 1
+
+    def withdraw(self, request: Request) -> None:
+        """A request that gives way may already have its portion in the draft."""
+        kept = [p for p in self.portions if p.request is not request]
+        self.left += sum(len(p.token_ids) for p in self.portions) - sum(len(p.token_ids) for p in kept)
+        self.portions = kept
+
+
 class Scheduler:
+    PENDING = 0        # stands in a step planned ahead for the token that the step before still draws
+
     def __init__(self, cache: CacheManager, max_seqs: int = 32, token_budget: int = 2048,
                  max_model_len: Optional[int] = None) -> None:
         if max_seqs < 1 or token_budget < 1:
@@ -116,235 +151,214 @@ class Scheduler:
         self.max_seqs = min(int(max_seqs), cache.num_slots)
         self.token_budget = int(token_budget)
         self.max_model_len = max_model_len
-        self._waiting: Deque[Sequence] = deque()
-        self._running: List[Sequence] = []
-        self._aborted: Set[Hashable] = set()
-        self._ids: Dict[Hashable, Sequence] = {}
+        self._queue: Deque[Request] = deque()
+        self._seated: List[Request] = []            # in the order in which they were seated
+        self._known: Dict[Hashable, Request] = {}
+        self._to_cancel: List[Request] = []
 
     # ------------------------------------------------------------- queries
     @property
     def num_waiting(self) -> int:
-        return len(self._waiting)
+        return len(self._queue)
 
     @property
     def num_running(self) -> int:
-        return len(self._running)
+        return len(self._seated)
 
     def has_work(self) -> bool:
-        return bool(self._waiting or self._running or self._aborted)
+        return bool(self._queue) or bool(self._seated) or bool(self._to_cancel)
 
-    # ------------------------------------------------------------- requests
-    def submit(self, seq: Sequence) -> None:
-        if not seq.prompt_ids:
+    def request(self, request_id) -> Request:
+        return self._known[request_id]
+
+    def queued(self) -> List[Request]:
+        return list(self._queue)
+
+    # ------------------------------------------------------------- arrivals and cancellations
+    def submit(self, request: Request) -> None:
+        """Refuses a request that could never run: empty, a duplicate, longer than the model allows,
+        or larger than the whole cache in its worst case (scheduler.py:118-134)."""
+        if len(request.prompt_ids) == 0:
             raise ValueError("prompt_ids must be non-empty")
-        if seq.max_new_tokens < 1:
+        if request.max_new_tokens < 1:
             raise ValueError("max_new_tokens must be >= 1")
-        if seq.request_id in self._ids:
-            raise ValueError(f"duplicate request_id {seq.request_id}")
-        total = len(seq.prompt_ids) + seq.max_new_tokens
-        if self.max_model_len is not None and total > self.max_model_len:
-            raise ValueError(f"request {seq.request_id}: prompt + max_new_tokens = {total} exceeds "
+        if request.request_id in self._known:
+            raise ValueError(f"duplicate request_id {request.request_id}")
+        longest = len(request.prompt_ids) + request.max_new_tokens
+        if self.max_model_len is not None and longest > self.max_model_len:
+            raise ValueError(f"request {request.request_id}: prompt + max_new_tokens = {longest} exceeds "
                              f"the model length {self.max_model_len}")
-        # worst case the request holds every page it will ever need at once (scheduler.py:125-131)
-        need = pages_needed(total, self.cache.block_size)
-        if need > self.cache.num_blocks:
-            raise BlockPoolExhausted(f"out of KV blocks: request needs {need} pages, pool has {self.cache.num_blocks}")
-        seq.state = SeqState.WAITING
-        self._waiting.append(seq)
-        self._ids[seq.request_id] = seq
+        pages = pages_needed(longest, self.cache.block_size)
+        if pages > self.cache.num_blocks:
+            raise BlockPoolExhausted(f"out of KV blocks: request needs {pages} pages, pool has {self.cache.num_blocks}")
+        request.phase = Phase.QUEUED
+        self._known[request.request_id] = request
+        self._queue.append(request)
 
     def abort(self, request_id) -> None:
-        """Takes effect at the next schedule(); safe while a step is in flight."""
-        if request_id in self._ids:
-            self._aborted.add(request_id)
+        """Marks the request; it leaves when the next step is planned, so this is safe while a step
+        with the request is in flight (its token is then dropped by `complete`)."""
+        request = self._known.get(request_id)
+        if request is not None and not request.cancelled:
+            request.cancelled = True
+            self._to_cancel.append(request)
 
-    # ------------------------------------------------------------- one step
+    # ------------------------------------------------------------- leaving a seat, one way or another
+    def _leave(self, request: Request, reason: Optional[str]) -> None:
+        """Out of queue or seat; pages and slot back. `reason` None: the request gives way and will be
+        recomputed (back to the head of the queue); else it has ended for that reason."""
+        if request.phase is Phase.SEATED:
+            self._seated.remove(request)
+            if request.request_id in self.cache:
+                self.cache.release(request.request_id)
+        elif request.phase is Phase.QUEUED and reason is not None:
+            self._queue.remove(request)
+        if reason is None:
+            request.num_computed = 0
+            request.phase = Phase.QUEUED
+            self._queue.appendleft(request)
+            return
+        request.phase = Phase.ENDED
+        request.finish_reason = reason
+        self._known.pop(request.request_id, None)
+
+    def _drop_cancelled(self) -> None:
+        for request in self._to_cancel:
+            if request.phase is not Phase.ENDED:
+                self._leave(request, "abort")
+                _log.info("request %s cancelled", request.request_id)
+        self._to_cancel = []
+
+    def give_way(self, request: Request) -> None:
+        """Preemption by recompute."""
+        self._leave(request, None)
+        request.preemptions += 1
+        _log.info("request %s gives way with %d tokens (time %d)", request.request_id, request.num_tokens,
+                  request.preemptions)
+
+    def requeue(self, requests: Iterable[Request]) -> None:
+        """Seated requests whose cached tokens can no longer be trusted (a step that held them was
+        dropped): back to the queue as if they had never run, in their old order, ahead of all others."""
+        for request in reversed(list(requests)):
+            if request.phase is Phase.SEATED:
+                self._leave(request, None)
+
+    # ------------------------------------------------------------- planning a step
+    def _seat_arrivals(self, draft: _Draft) -> None:
+        while self._queue and len(self._seated) < self.max_seqs and draft.left > 0:
+            request = self._queue[0]
+            # seated by the pages of everything known of it (scheduler.py:196-211), though only the pages
+            # of the portion that runs now are taken
+            if self.cache.slots.num_free < 1 or not self.cache.can_reserve(request.request_id, request.num_tokens):
+                return
+            count = min(request.num_tokens, draft.left)
+            self._queue.popleft()
+            self.cache.add(request.request_id)
+            self.cache.reserve(request.request_id, count)
+            request.num_computed = 0
+            request.phase = Phase.SEATED
+            self._seated.append(request)
+            draft.put(request, 0, count)
+
     def schedule(self) -> StepPlan:
-        self._reap_aborted()
-        budget = self.token_budget
-        preempted = False
-        items: List[ScheduledSeq] = []
-        # decoding requests first, then prompts in flight; within each, oldest first
-        order = sorted(range(len(self._running)),
-                       key=lambda i: (self._running[i].num_tokens - self._running[i].num_computed > 1, i))
-        for seq in [self._running[i] for i in order]:
-            if seq.state is not SeqState.RUNNING:
-                continue            # preempted while an older request was served
-            pending = seq.num_tokens - seq.num_computed
-            n = min(pending, budget)
-            if n < 1:
+        self._drop_cancelled()
+        draft = _Draft(self.token_budget)
+        someone_gave_way = False
+        decoding = [r for r in self._seated if r.num_tokens - r.num_computed == 1]
+        in_prompt = [r for r in self._seated if r.num_tokens - r.num_computed != 1]
+        for request in decoding + in_prompt:
+            if request.phase is not Phase.SEATED:
+                continue                                  # gave way to an older request a moment ago
+            count = min(request.num_tokens - request.num_computed, draft.left)
+            if count < 1:
                 continue
-            while seq.state is SeqState.RUNNING and not self.cache.can_reserve(seq.request_id, n):
-                victim = self._running[-1]
-                # the victim may already have its tokens in this step's plan: take them out again
-                budget += sum(len(it.token_ids) for it in items if it.seq is victim)
-                items = [it for it in items if it.seq is not victim]
-                self._preempt(victim)
-                preempted = True
-            if seq.state is not SeqState.RUNNING:
-                continue
-            self.cache.reserve(seq.request_id, n)
-            items.append(self._item(seq, n))
-            budget -= n
-        # no admission in a step that had to preempt: the victim would come straight back
-        while not preempted and self._waiting and len(self._running) < self.max_seqs and budget > 0:
-            seq = self._waiting[0]
-            n = min(seq.num_tokens, budget)
-            # admit by the pages of everything known of the request (scheduler.py:196-211), though
-            # only the pages of the portion that runs now are taken
-            if self.cache.slots.num_free < 1 or not self.cache.can_reserve(seq.request_id, seq.num_tokens):
-                break
-            self._waiting.popleft()
-            self.cache.add(seq.request_id)
-            self.cache.reserve(seq.request_id, n)
-            seq.num_computed = 0
-            seq.state = SeqState.RUNNING
-            self._running.append(seq)
-            items.append(self._item(seq, n))
-            budget -= n
-        return StepPlan(items=tuple(items))
-
-    PENDING = 0        # stands in a planned-ahead item for the token that the step before is still sampling
+            while request.phase is Phase.SEATED and not self.cache.can_reserve(request.request_id, count):
+                last = self._seated[-1]
+                draft.withdraw(last)
+                self.give_way(last)
+                someone_gave_way = True
+            if request.phase is Phase.SEATED:
+                self.cache.reserve(request.request_id, count)
+                draft.put(request, request.num_computed, count)
+        if not someone_gave_way:          # else whoever gave way would come straight back
+            self._seat_arrivals(draft)
+        return StepPlan(tuple(draft.portions))
 
     def schedule_ahead(self, plan: StepPlan) -> Optional[StepPlan]:
         """The step after `plan` (launched, not yet completed), planned before `plan`'s tokens are
         known, so that it can be launched while the host still waits for them; None where that is not
-        plain. Every running request must be in `plan`. The step after then holds, in this order:
+        plain. Every seated request must be in `plan`. The step after then holds, in this order:
         the requests of `plan` that sample, with the pending token as their one token (`feeds` names
         their places in `plan`; those that reach their length with the pending token are left out);
-        the next portions of prompts that `plan` has not finished; and waiting requests for which a
+        the next portions of prompts that `plan` has not finished; and queued requests for which a
         seat, a state slot and pages are free now (the seat of a request that ends with the pending
-        token is free one step later). Nobody is preempted for it: if a page is missing the answer is
-        None and the plain schedule decides who gives way. A request that turns out to have ended
-        with the pending token (end of sequence, abort) has a row of the next step computed for
-        nothing; `complete` skips it."""
-        self._reap_aborted()
-        if not plan.items or len(plan.items) != len(self._running):
+        token is free one step later). Nobody gives way for it: if a page is missing the answer is
+        None and the plain schedule decides. A request that turns out to have ended with the pending
+        token (end of sequence, cancelled) has a row of the next step computed for nothing;
+        `complete` skips it."""
+        self._drop_cancelled()
+        if len(plan.portions) == 0 or len(plan.portions) != len(self._seated):
             return None
-        if any(item.seq.state is not SeqState.RUNNING for item in plan.items):
+        if any(p.request.phase is not Phase.SEATED for p in plan.portions):
             return None
-        budget = self.token_budget
-        items: List[ScheduledSeq] = []
-        feeds: List[int] = []
-        # called after `plan` was launched and before it is completed: its tokens are the pending ones
-        for i, item in enumerate(plan.items):
-            if not item.samples:
-                continue
-            if len(item.seq.output_ids) + 1 >= item.seq.max_new_tokens:
-                continue                                  # ends with the pending token, whatever it is
-            if budget < 1 or not self.cache.can_reserve(item.seq.request_id, 1):
-                # pages run out: the plain schedule decides who gives way. What was taken so far stays
-                # with requests that need it for their next token anyway.
+        draft = _Draft(self.token_budget)
+        for place, portion in enumerate(plan.portions):
+            request = portion.request
+            if not portion.samples or len(request.output_ids) + 1 >= request.max_new_tokens:
+                continue                  # no token pending, or it is the request's last, whatever it is
+            if draft.left < 1 or not self.cache.can_reserve(request.request_id, 1):
+                # what was taken so far stays with requests that need it for their next token anyway
                 return None
-            self.cache.reserve(item.seq.request_id, 1)
-            items.append(ScheduledSeq(seq=item.seq, token_ids=[self.PENDING],
-                                      past_len=item.past_len + len(item.token_ids), samples=True))
-            feeds.append(i)
-            budget -= 1
-        for item in plan.items:
-            if item.samples:
+            self.cache.reserve(request.request_id, 1)
+            draft.put_pending(request, portion.end, self.PENDING, place)
+        for portion in plan.portions:
+            if portion.samples:
                 continue
-            seq = item.seq
-            begin = item.past_len + len(item.token_ids)
-            n = min(seq.num_tokens - begin, budget)
-            if n < 1:
-                return None                               # every running request is in a step, or the step is not plain
-            if not self.cache.can_reserve(seq.request_id, n):
+            request = portion.request
+            count = min(request.num_tokens - portion.end, draft.left)
+            if count < 1 or not self.cache.can_reserve(request.request_id, count):
                 return None
-            self.cache.reserve(seq.request_id, n)
-            items.append(ScheduledSeq(seq=seq, token_ids=seq.tokens(begin, begin + n), past_len=begin,
-                                      samples=begin + n == seq.num_tokens))
-            budget -= n
-        while self._waiting and len(self._running) < self.max_seqs and budget > 0:
-            seq = self._waiting[0]
-            n = min(seq.num_tokens, budget)
-            if self.cache.slots.num_free < 1 or not self.cache.can_reserve(seq.request_id, seq.num_tokens):
-                break
-            self._waiting.popleft()
-            self.cache.add(seq.request_id)
-            self.cache.reserve(seq.request_id, n)
-            seq.num_computed = 0
-            seq.state = SeqState.RUNNING
-            self._running.append(seq)
-            items.append(self._item(seq, n))
-            budget -= n
-        if not items:
+            self.cache.reserve(request.request_id, count)
+            draft.put(request, portion.end, count)
+        self._seat_arrivals(draft)
+        if not draft.portions:
             return None
-        return StepPlan(items=tuple(items), feeds=tuple(feeds))
+        return StepPlan(tuple(draft.portions), feeds=tuple(draft.feeds))
 
-    def _item(self, seq: Sequence, n: int) -> ScheduledSeq:
-        begin = seq.num_computed
-        return ScheduledSeq(seq=seq, token_ids=seq.tokens(begin, begin + n), past_len=begin,
-                            samples=begin + n == seq.num_tokens)
-
-    def complete(self, plan: StepPlan, next_ids: Seq[Optional[int]]) -> List[Emission]:
-        """`next_ids[i]` is the token sampled for `plan.items[i]` (ignored where the item does
-        not sample). The cache's own counts were advanced by the step function."""
-        if len(next_ids) != len(plan.items):
-            raise ValueError("one entry per scheduled sequence is required")
-        out: List[Emission] = []
-        for item, token in zip(plan.items, next_ids):
-            seq = item.seq
-            if seq.request_id in self._aborted or seq.state is not SeqState.RUNNING:
+    # ------------------------------------------------------------- after a step
+    def complete(self, plan: StepPlan, drawn: Seq[Optional[int]]) -> List[Emission]:
+        """`drawn[i]` is the token drawn after portion i (ignored where the portion does not sample).
+        The cache's own counts were advanced by the step function."""
+        if len(drawn) != len(plan.portions):
+            raise ValueError("one entry per portion of the plan is required")
+        emitted: List[Emission] = []
+        for portion, token in zip(plan.portions, drawn):
+            request = portion.request
+            if request.cancelled or request.phase is not Phase.SEATED:
                 continue
-            seq.num_computed = item.past_len + len(item.token_ids)
-            if not item.samples:
+            request.num_computed = portion.end
+            if not portion.samples:
                 continue
             token = int(token)
-            seq.output_ids.append(token)
-            hit_eos = (not seq.params.ignore_eos) and token in seq.eos_ids
-            finished = hit_eos or len(seq.output_ids) >= seq.max_new_tokens
-            if finished:
-                seq.finish_reason = "stop" if hit_eos else "length"
-                self._finish(seq)
-            out.append(Emission(seq=seq, token_id=token, finished=finished))
-        return out
+            request.output_ids.append(token)
+            reason = None
+            if token in request.eos_ids and not request.params.ignore_eos:
+                reason = "stop"
+            elif len(request.output_ids) >= request.max_new_tokens:
+                reason = "length"
+            if reason is not None:
+                self._leave(request, reason)
+            emitted.append(Emission(request, token, reason is not None))
+        return emitted
 
-    def fail(self, plan: StepPlan, error: BaseException) -> List[Sequence]:
-        """A step raised: every request in it is over, with the error, and what it holds goes
-        back (worker/src/inference/batch_loop.py:135-147)."""
-        failed = []
-        for item in plan.items:
-            seq = item.seq
-            if seq.state is SeqState.RUNNING:
-                seq.error = error
-                seq.finish_reason = "error"
-                self._finish(seq)
-                failed.append(seq)
-        return failed
-
-    # ------------------------------------------------------------- internals
-    def _reap_aborted(self) -> None:
-        for request_id in list(self._aborted):
-            seq = self._ids.pop(request_id, None)
-            if seq is None:
-                continue
-            if seq.state is SeqState.WAITING:
-                self._waiting.remove(seq)
-            elif seq.state is SeqState.RUNNING:
-                self._running.remove(seq)
-                self._release(seq)
-            seq.state = SeqState.FINISHED
-            seq.finish_reason = "abort"
-            _log.info("sequence aborted request_id=%s", request_id)
-        self._aborted.clear()
-
-    def _preempt(self, seq: Sequence) -> None:
-        self._running.remove(seq)
-        self._release(seq)
-        seq.num_computed = 0
-        seq.state = SeqState.WAITING
-        seq.preemptions += 1
-        self._waiting.appendleft(seq)
-        _log.info("sequence preempted request_id=%s tokens=%s preemptions=%s",
-                  seq.request_id, seq.num_tokens, seq.preemptions)
-
-    def _finish(self, seq: Sequence) -> None:
-        self._running.remove(seq)
-        self._release(seq)
-        seq.state = SeqState.FINISHED
-        self._ids.pop(seq.request_id, None)
-
-    def _release(self, seq: Sequence) -> None:
-        if seq.request_id in self.cache:
-            self.cache.release(seq.request_id)
+    def fail(self, plan: StepPlan, error: BaseException) -> List[Request]:
+        """A step raised: every request in it is over, with the error, and what it holds goes back
+        (worker/src/inference/batch_loop.py:135-147)."""
+        ended = []
+        for portion in plan.portions:
+            request = portion.request
+            if request.phase is Phase.SEATED:
+                request.error = error
+                self._leave(request, "error")
+                ended.append(request)
+        return ended

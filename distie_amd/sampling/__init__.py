@@ -1,3 +1,3 @@
-from .sampler import Sampler, SamplingParams, uniform_of
+from .sampler import Sampler, SamplingParams, derive_seed, uniform_of
 
-__all__ = ["Sampler", "SamplingParams", "uniform_of"]
+__all__ = ["Sampler", "SamplingParams", "derive_seed", "uniform_of"]

@@ -30,6 +30,15 @@ def uniform_of(seed: int, counter: int) -> float:
     return (z >> 40) / 16777216.0
 
 
+def derive_seed(engine_seed: int, arrival: int) -> int:
+    """The seed of the `arrival`-th request of an engine that was not given one: a splitmix64 step of
+    the two, so that neighbouring arrivals get unrelated streams."""
+    z = ((engine_seed & _MASK) ^ ((arrival * 0x9E3779B97F4A7C15 + 0x632BE59BD9B4E019) & _MASK)) & _MASK
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _MASK
+    return z ^ (z >> 31)
+
+
 @dataclass(frozen=True)
 class SamplingParams:
     """`max_new_tokens` and `temperature` are the reference's `max_tokens` and
@@ -38,7 +47,7 @@ class SamplingParams:
 
     max_new_tokens: int = 16
     temperature: float = 0.0
-    seed: Optional[int] = None
+    seed: Optional[int] = None        # None: a stream of the request's own, derived from the engine's seed
     eos_id: Optional[int] = None      # None: the model's own end-of-sequence ids
     ignore_eos: bool = False
 

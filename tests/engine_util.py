@@ -88,3 +88,49 @@ def check_logits(got, weights, cfg, ids, dtype, folder=None):
     rms = diff.pow(2).mean().sqrt().item()
     assert err < scale / 16, f"max error {err} vs oracle, largest logit {scale}"
     assert rms < scale / 64, f"rms error {rms} vs oracle, largest logit {scale}"
+
+
+def plain_uniform(seed, counter):
+    """The uniform number of a request's `counter`-th draw, written out independently of the product's
+    `uniform_of`: the state seed * G + counter * C + K goes through the output function of splitmix64
+    (xor-shift 30, multiply, xor-shift 27, multiply, xor-shift 31); the top 24 bits are the number."""
+    import numpy as np
+
+    with np.errstate(over="ignore"):
+        u = np.uint64
+        z = u(seed & (2 ** 64 - 1)) * u(0x9E3779B97F4A7C15) + u(counter & (2 ** 64 - 1)) * u(0xD1B54A32D192ED03) \
+            + u(0x94D049BB133111EB)
+        z = (z ^ (z >> u(30))) * u(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> u(27))) * u(0x94D049BB133111EB)
+        z = z ^ (z >> u(31))
+    return float(int(z) >> 40) / float(1 << 24)
+
+
+def check_generation(weights, cfg, prompt, token_ids, temperature=0.0, seed=0, tol=1e-4):
+    """Every produced token is the plain implementation's choice given the tokens before it: the
+    argmax of its float64 logits, or for a temperature the first index whose cumulative softmax weight
+    exceeds the request's `n`-th uniform number. The engine's float32 logits differ from the oracle's
+    by up to `tol`, so a draw within that distance of an interval's end may land in the neighbouring
+    interval, and of two logits within `tol` either may win. -> how many tokens were such near misses."""
+    ids = list(prompt)
+    near = 0
+    for n, token in enumerate(token_ids):
+        logits = plain.forward(weights, cfg, ids, torch.float64)[-1]
+        if temperature <= 0:
+            best = int(logits.argmax())
+            if token != best:
+                assert logits[token] >= logits[best] - tol, f"token {n}: {token} is not the greedy pick {best}"
+                near += 1
+        else:
+            w = torch.exp((logits - logits.max()) / temperature)
+            c = torch.cumsum(w, 0) / w.sum()
+            u = plain_uniform(seed, n)
+            want = int((c > u).nonzero()[0])
+            if token != want:
+                below = float(c[token - 1]) if token else 0.0
+                slack = 4 * tol / temperature
+                assert w[token] > 0 and below - slack <= u <= float(c[token]) + slack, \
+                    f"token {n}: {token} drawn, the plain draw is {want} (u = {u})"
+                near += 1
+        ids.append(int(token))
+    return near

@@ -8,7 +8,7 @@ import torch
 
 import plain_qwen2 as plain
 from distie_amd import LLM, SamplingParams
-from engine_util import make_model_dir, oracle, random_ids
+from engine_util import check_generation, make_model_dir, oracle, plain_uniform, random_ids
 from torch_ops import TorchOps
 
 
@@ -193,3 +193,103 @@ def test_abort_and_arrival_while_a_step_is_ahead(tiny):
     assert llm._outputs[c].token_ids == plain_greedy(weights, cfg, late_prompt, 6)
     llm.cache.check()
     assert llm.cache.free_pages() == [64, 64] and llm.cache.slots.num_free == llm.cache.num_slots
+
+
+def test_the_uniform_numbers_are_splitmix64():
+    """The generator is pinned from outside: the output function of splitmix64 turns the state
+    0x9E3779B97F4A7C15 (its first state from seed 0) into 0xE220A8397B1DCDAF, the published first value
+    of that generator. The seed that makes (seed * G + K) equal that state reaches it through the kernel's
+    own arithmetic; the independent copy of the tests agrees everywhere else."""
+    from distie_amd.sampling import derive_seed, uniform_of
+
+    G, K, M = 0x9E3779B97F4A7C15, 0x94D049BB133111EB, 1 << 64
+    seed = ((G - K) * pow(G, -1, M)) % M
+    assert uniform_of(seed, 0) == (0xE220A8397B1DCDAF >> 40) / 2 ** 24
+    for s_, n in ((0, 0), (1, 0), (0, 1), (5, 17), (2 ** 63 + 11, 2 ** 40), (2 ** 64 - 1, 3)):
+        assert uniform_of(s_, n) == plain_uniform(s_, n)
+    seeds = [derive_seed(0, i) for i in range(100)] + [derive_seed(1, i) for i in range(100)]
+    assert len(set(seeds)) == 200 and all(0 <= s_ < M for s_ in seeds)
+
+
+def test_sampled_tokens_are_the_plain_draws_token_by_token(tiny):
+    """Greedy and temperature requests mixed in one batch, prompts in portions: every token is
+    argmax / the inverse of the cumulative sum at the request's own n-th uniform number, given the
+    tokens before it, whatever else runs beside it."""
+    cfg, folder, weights = tiny
+    prompts = [random_ids(cfg, n, 90 + n) for n in (1, 9, 23, 40)]
+    params = [SamplingParams(max_new_tokens=12, temperature=0.7, seed=11), SamplingParams(max_new_tokens=12),
+              SamplingParams(max_new_tokens=12, temperature=0.7, seed=12), SamplingParams(max_new_tokens=12)]
+    for options in ({"token_budget": 7}, {"token_budget": 7, "lookahead": False}, {"num_blocks": 9}):
+        outs = engine(folder, **options).generate(prompts, params)
+        for prompt, sp, out in zip(prompts, params, outs):
+            assert len(out.token_ids) == 12
+            assert check_generation(weights, cfg, prompt, out.token_ids, sp.temperature, sp.seed or 0, tol=1e-6) == 0
+
+
+def test_requests_without_a_seed_draw_from_streams_of_their_own(tiny):
+    cfg, folder, _ = tiny
+    prompt = random_ids(cfg, 6, 1)
+    params = SamplingParams(max_new_tokens=8, temperature=1.5)
+    llm = engine(folder)
+    first = [o.token_ids for o in llm.generate([prompt] * 3, params)]
+    assert len({tuple(t) for t in first}) == 3                     # three samples of one prompt differ
+    later = [o.token_ids for o in llm.generate([prompt] * 3, params)]
+    assert later != first                                          # and so do later ones of the same engine
+    assert [o.token_ids for o in engine(folder).generate([prompt] * 3, params)] == first     # a rerun repeats
+    assert [o.token_ids for o in engine(folder, seed=1).generate([prompt] * 3, params)] != first
+    # an explicit seed is taken as it is: the same stream for every request that names it
+    fixed = SamplingParams(max_new_tokens=8, temperature=1.5, seed=4)
+    same = [o.token_ids for o in engine(folder).generate([prompt] * 2, fixed)]
+    assert same[0] == same[1]
+
+
+def test_a_step_that_fails_while_the_next_one_is_ahead(tiny):
+    """The step in flight fails after the step behind it was launched, and that step had seated a new
+    request: the failed step's requests end with the error, the new request starts over and still gets
+    the plain implementation's tokens (its cached tokens of the dropped step are not trusted)."""
+    cfg, folder, weights = tiny
+    llm = engine(folder, max_seqs=2)
+    prompts = [random_ids(cfg, n, 110 + n) for n in (4, 6, 5)]
+    a = llm.add_request(prompts[0], SamplingParams(max_new_tokens=2))
+    b = llm.add_request(prompts[1], SamplingParams(max_new_tokens=10))
+    c = llm.add_request(prompts[2], SamplingParams(max_new_tokens=6))
+    real = llm._to_host
+    calls = {"n": 0}
+
+    def flaky(chosen):
+        fetch = real(chosen)
+        calls["n"] += 1
+        if calls["n"] != 3:
+            return fetch
+
+        def broken():
+            # by now the step behind this one is launched, and it has seated c
+            assert llm._ahead is not None and c in [p.request.request_id for p in llm._ahead[0].portions]
+            raise RuntimeError("injected failure while fetching")
+        return broken
+
+    llm._to_host = flaky
+    while llm.has_work():
+        llm.run_step()
+    assert calls["n"] > 3
+    outs = {r: llm.take_output(r) for r in (a, b, c)}
+    assert outs[a].finish_reason == "length" and outs[a].token_ids == plain_greedy(weights, cfg, prompts[0], 2)
+    assert outs[b].finish_reason == "error" and "injected" in outs[b].error
+    assert outs[c].finish_reason == "length" and outs[c].token_ids == plain_greedy(weights, cfg, prompts[2], 6)
+    assert not llm._outputs
+    llm.cache.check()
+    assert llm.cache.free_pages() == [64, 64] and llm.cache.slots.num_free == llm.cache.num_slots
+
+
+def test_step_stats_and_forgotten_records(tiny):
+    cfg, folder, _ = tiny
+    llm = engine(folder, step_stats=1000, token_budget=6)
+    for _ in llm.stream([random_ids(cfg, 9, 1), random_ids(cfg, 3, 2)], SamplingParams(max_new_tokens=4)):
+        pass
+    assert not llm._outputs                                        # stream hands nothing on and keeps nothing
+    summary = llm.stats.summary()
+    assert set(summary) == {"decode", "prefill"}
+    assert summary["prefill"]["tokens"] > summary["prefill"]["rows"] and summary["decode"]["tokens"] == summary["decode"]["rows"]
+    assert all(row["host"] >= row["launch"] > 0 for row in summary.values())
+    assert "device" not in summary["decode"]                       # no GPU here: host parts only
+    assert "host=" in llm.stats.format()

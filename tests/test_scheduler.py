@@ -5,7 +5,7 @@ scheduler cuts prompts (the reference never does)."""
 import pytest
 
 from distie_amd.cache import CacheManager
-from distie_amd.engine.scheduler import BlockPoolExhausted, Scheduler, Sequence, SeqState
+from distie_amd.engine.scheduler import BlockPoolExhausted, Scheduler, Request, Phase
 from distie_amd.parts import PagedKV
 from distie_amd.sampling import SamplingParams
 
@@ -19,21 +19,21 @@ def make(pages, block=4, max_seqs=32, budget=2048, window=None, slots=8, max_mod
 
 
 def seq(rid, prompt_len, max_new=8):
-    return Sequence(request_id=rid, prompt_ids=list(range(1, prompt_len + 1)),
+    return Request(request_id=rid, prompt_ids=list(range(1, prompt_len + 1)),
                     params=SamplingParams(max_new_tokens=max_new), eos_ids=(EOS,))
 
 
 def run(sched, cache, tokens):
     """schedule, pretend the step ran (the step function advances the cache's counts), complete"""
     plan = sched.schedule()
-    for item in plan.items:
-        cache.commit(item.seq.request_id, len(item.token_ids))
-    picks = [tokens if isinstance(tokens, int) else tokens[i] for i in range(len(plan.items))]
+    for item in plan.portions:
+        cache.commit(item.request.request_id, len(item.token_ids))
+    picks = [tokens if isinstance(tokens, int) else tokens[i] for i in range(len(plan.portions))]
     return plan, sched.complete(plan, picks)
 
 
 def names(plan):
-    return [i.seq.request_id for i in plan.items]
+    return [i.request.request_id for i in plan.portions]
 
 
 def test_fifo_and_prefill_then_decode():
@@ -43,15 +43,15 @@ def test_fifo_and_prefill_then_decode():
     sched.submit(b)
     plan = sched.schedule()
     assert names(plan) == ["a", "b"]
-    assert [len(i.token_ids) for i in plan.items] == [5, 2]
-    assert [i.past_len for i in plan.items] == [0, 0]
-    assert all(i.samples for i in plan.items)
+    assert [len(i.token_ids) for i in plan.portions] == [5, 2]
+    assert [i.begin for i in plan.portions] == [0, 0]
+    assert all(i.samples for i in plan.portions)
     assert len(cache.request("a").tables[0]) == 2
-    for i in plan.items:
-        cache.commit(i.seq.request_id, len(i.token_ids))
+    for i in plan.portions:
+        cache.commit(i.request.request_id, len(i.token_ids))
     sched.complete(plan, [7, 8])
     plan = sched.schedule()
-    assert [(i.token_ids, i.past_len) for i in plan.items] == [([7], 5), ([8], 2)]
+    assert [(i.token_ids, i.begin) for i in plan.portions] == [([7], 5), ([8], 2)]
     assert plan.is_decode
 
 
@@ -61,11 +61,11 @@ def test_max_seqs_and_token_budget_cut_prompts():
         sched.submit(seq(rid, 4))
     plan, _ = run(sched, cache, 7)
     # a whole, b's first two tokens: the budget of 6 is filled, b does not sample yet
-    assert [(i.seq.request_id, i.token_ids, i.samples) for i in plan.items] == [("a", [1, 2, 3, 4], True), ("b", [1, 2], False)]
-    assert sched._ids["b"].output_ids == []
+    assert [(i.request.request_id, i.token_ids, i.samples) for i in plan.portions] == [("a", [1, 2, 3, 4], True), ("b", [1, 2], False)]
+    assert sched.request("b").output_ids == []
     plan, _ = run(sched, cache, 7)
     # decoding first, then the prompt in flight
-    assert [(i.seq.request_id, i.token_ids, i.past_len, i.samples) for i in plan.items] == \
+    assert [(i.request.request_id, i.token_ids, i.begin, i.samples) for i in plan.portions] == \
         [("a", [7], 4, True), ("b", [3, 4], 2, True)]
     plan, _ = run(sched, cache, 7)
     assert names(plan) == ["a", "b"] and sched.num_waiting == 1      # max_seqs keeps c waiting
@@ -77,7 +77,7 @@ def test_long_prompt_is_cut_under_the_budget():
     sizes = []
     for _ in range(3):
         plan, out = run(sched, cache, 7)
-        sizes.append((plan.num_tokens, plan.items[0].past_len, plan.items[0].samples))
+        sizes.append((plan.num_tokens, plan.portions[0].begin, plan.portions[0].samples))
     assert sizes == [(4, 0, False), (4, 4, False), (2, 8, True)]
     assert out[0].token_id == 7
     assert all(p.num_tokens <= 4 for p in [plan])
@@ -91,7 +91,7 @@ def test_every_step_stays_within_the_budget_and_decodes_come_first():
     for _ in range(6):
         plan, _ = run(sched, cache, 7)
         assert plan.num_tokens <= 8
-        assert plan.items[0].seq.request_id == "a" and len(plan.items[0].token_ids) == 1
+        assert plan.portions[0].request.request_id == "a" and len(plan.portions[0].token_ids) == 1
 
 
 def test_waits_for_blocks():
@@ -102,7 +102,7 @@ def test_waits_for_blocks():
     assert names(plan) == ["a"] and cache.free_pages() == [0]
     cache.commit("a", 7)
     emitted = sched.complete(plan, [7])
-    assert emitted[0].finished and emitted[0].seq.finish_reason == "length"
+    assert emitted[0].finished and emitted[0].request.finish_reason == "length"
     assert names(sched.schedule()) == ["b"]
 
 
@@ -121,7 +121,7 @@ def test_rejects_duplicate_and_empty():
     with pytest.raises(ValueError):
         sched.submit(seq("a", 2))
     with pytest.raises(ValueError):
-        sched.submit(Sequence(request_id="b", prompt_ids=[]))
+        sched.submit(Request(request_id="b", prompt_ids=[]))
 
 
 def test_eos_and_cap_free_blocks():
@@ -129,7 +129,7 @@ def test_eos_and_cap_free_blocks():
     sched.submit(seq("a", 2, max_new=5))
     sched.submit(seq("b", 2, max_new=1))
     plan, emitted = run(sched, cache, [EOS, 3])
-    assert [(e.seq.request_id, e.finished, e.seq.finish_reason) for e in emitted] == \
+    assert [(e.request.request_id, e.finished, e.request.finish_reason) for e in emitted] == \
         [("a", True, "stop"), ("b", True, "length")]
     assert cache.free_pages() == [4] and cache.slots.num_free == 8
     assert not sched.has_work()
@@ -137,7 +137,7 @@ def test_eos_and_cap_free_blocks():
 
 def test_ignore_eos():
     sched, cache = make(4)
-    s = Sequence("a", [1, 2], SamplingParams(max_new_tokens=3, ignore_eos=True), eos_ids=(EOS,))
+    s = Request("a", [1, 2], SamplingParams(max_new_tokens=3, ignore_eos=True), eos_ids=(EOS,))
     sched.submit(s)
     _, emitted = run(sched, cache, EOS)
     assert not emitted[0].finished
@@ -153,7 +153,7 @@ def test_newest_is_preempted_and_recomputed_without_reemitting():
     plan = sched.schedule()
     # a needs a second page; the pool is empty, so b (newest) is preempted
     assert names(plan) == ["a"]
-    assert b.state is SeqState.WAITING and "b" not in cache
+    assert b.phase is Phase.QUEUED and "b" not in cache
     assert b.output_ids == [20, 21] and b.preemptions == 1 and b.num_computed == 0
     cache.commit("a", 1)
     assert [e.token_id for e in sched.complete(plan, [12])] == [12]
@@ -167,10 +167,10 @@ def test_recompute_prefills_prompt_plus_output():
     sched.submit(b)
     run(sched, cache, [10, 20])
     plan, _ = run(sched, cache, [11, 21])     # a finishes on the cap and frees its pages
-    assert len(plan.items) == 2 and cache.free_pages() == [2]
-    sched._preempt(b)
-    item = sched.schedule().items[0]
-    assert (item.seq.request_id, item.token_ids, item.past_len, item.samples) == ("b", [1, 2, 3, 20, 21], 0, True)
+    assert len(plan.portions) == 2 and cache.free_pages() == [2]
+    sched.give_way(b)
+    item = sched.schedule().portions[0]
+    assert (item.request.request_id, item.token_ids, item.begin, item.samples) == ("b", [1, 2, 3, 20, 21], 0, True)
 
 
 def test_queue_front_after_preemption_and_no_readmission_in_that_step():
@@ -182,7 +182,7 @@ def test_queue_front_after_preemption_and_no_readmission_in_that_step():
     sched.submit(seq("c", 1, max_new=4))
     plan = sched.schedule()
     assert names(plan) == ["a"]
-    assert [s.request_id for s in sched._waiting] == ["b", "c"]
+    assert [s.request_id for s in sched.queued()] == ["b", "c"]
 
 
 def test_needy_request_preempts_itself_when_it_is_the_newest():
@@ -193,7 +193,7 @@ def test_needy_request_preempts_itself_when_it_is_the_newest():
     run(sched, cache, 5)                      # one page each, one page free
     plan = sched.schedule()
     # both need a second page: a (older) takes the free one, b is the newest and goes itself
-    assert names(plan) == ["a"] and sched._waiting[0] is b and b.preemptions == 1
+    assert names(plan) == ["a"] and sched.queued()[0] is b and b.preemptions == 1
     assert cache.free_pages() == [1]
     cache.check()
 
@@ -205,7 +205,7 @@ def test_abort_running_frees_on_next_schedule():
     sched.abort("a")
     cache.commit("a", 2)
     assert sched.complete(plan, [5]) == []        # aborted in flight: nothing emitted
-    assert sched.schedule().items == ()
+    assert sched.schedule().portions == ()
     assert cache.free_pages() == [4] and not sched.has_work()
 
 
@@ -243,20 +243,20 @@ def test_the_step_after_is_planned_ahead_only_when_that_is_plain():
     sched.submit(a)
     sched.submit(b)
     plan = sched.schedule()
-    for item in plan.items:
-        cache.commit(item.seq.request_id, len(item.token_ids))
+    for item in plan.portions:
+        cache.commit(item.request.request_id, len(item.token_ids))
     # both decode from here on, nothing waits: the next step can be planned before the tokens are known
     ahead = sched.schedule_ahead(plan)
     assert names(ahead) == ["a", "b"] and ahead.feeds == (0, 1)
-    assert [(i.token_ids, i.past_len, i.samples) for i in ahead.items] == [([sched.PENDING], 3, True), ([sched.PENDING], 2, True)]
+    assert [(i.token_ids, i.begin, i.samples) for i in ahead.portions] == [([sched.PENDING], 3, True), ([sched.PENDING], 2, True)]
     sched.complete(plan, [7, 8])
-    for item in ahead.items:
-        cache.commit(item.seq.request_id, 1)
+    for item in ahead.portions:
+        cache.commit(item.request.request_id, 1)
     # a reaches its length with the token that is pending now: it is not in the step after
     after = sched.schedule_ahead(ahead)
     assert names(after) == ["b"] and after.feeds == (1,)
     out = sched.complete(ahead, [5, 6])
-    assert [(e.seq.request_id, e.finished) for e in out] == [("a", True), ("b", False)]
+    assert [(e.request.request_id, e.finished) for e in out] == [("a", True), ("b", False)]
     cache.commit("b", 1)
     # b ends with an end-of-sequence token: its row of the step after was computed for nothing
     again = sched.schedule_ahead(after)
@@ -269,15 +269,15 @@ def test_the_step_after_is_planned_ahead_only_when_that_is_plain():
     # a request that waits is admitted by the step planned ahead if a seat, a slot and its pages are free now
     sched.submit(seq("d", 2))
     plan = sched.schedule()
-    for item in plan.items:
-        cache.commit(item.seq.request_id, len(item.token_ids))
+    for item in plan.portions:
+        cache.commit(item.request.request_id, len(item.token_ids))
     sched.submit(c)
     ahead = sched.schedule_ahead(plan)
     assert names(ahead) == ["d", "c"] and ahead.feeds == (0,)
-    assert [(i.token_ids, i.past_len, i.samples) for i in ahead.items] == [([sched.PENDING], 2, True), (list(range(1, 10)), 0, True)]
+    assert [(i.token_ids, i.begin, i.samples) for i in ahead.portions] == [([sched.PENDING], 2, True), (list(range(1, 10)), 0, True)]
     sched.complete(plan, [1])
-    for item in ahead.items:
-        cache.commit(item.seq.request_id, len(item.token_ids))
+    for item in ahead.portions:
+        cache.commit(item.request.request_id, len(item.token_ids))
     sched.complete(ahead, [2, 3])
     assert c.output_ids == [3] and c.num_computed == 9
     # a prompt in portions goes on in the step planned ahead; a waiting request without pages stays out of it
@@ -286,15 +286,15 @@ def test_the_step_after_is_planned_ahead_only_when_that_is_plain():
     small.submit(e)
     small.submit(f)
     plan = small.schedule()
-    assert [(i.seq.request_id, i.token_ids, i.samples) for i in plan.items] == [("e", [1, 2, 3, 4], False)]   # f: no pages
-    for item in plan.items:
-        cache2.commit(item.seq.request_id, len(item.token_ids))
+    assert [(i.request.request_id, i.token_ids, i.samples) for i in plan.portions] == [("e", [1, 2, 3, 4], False)]   # f: no pages
+    for item in plan.portions:
+        cache2.commit(item.request.request_id, len(item.token_ids))
     ahead = small.schedule_ahead(plan)
-    assert [(i.seq.request_id, i.token_ids, i.past_len, i.samples) for i in ahead.items] == [("e", [5, 6, 7], 4, True)]
+    assert [(i.request.request_id, i.token_ids, i.begin, i.samples) for i in ahead.portions] == [("e", [5, 6, 7], 4, True)]
     assert ahead.feeds == () and small.num_waiting == 1
     small.complete(plan, [None])
-    for item in ahead.items:
-        cache2.commit(item.seq.request_id, len(item.token_ids))
+    for item in ahead.portions:
+        cache2.commit(item.request.request_id, len(item.token_ids))
     after = small.schedule_ahead(ahead)
     assert names(after) == ["e"] and after.feeds == (0,)
     small.complete(ahead, [1])
@@ -304,8 +304,8 @@ def test_the_step_after_is_planned_ahead_only_when_that_is_plain():
     tight.submit(seq("k", 3, max_new=1))
     plan = tight.schedule()
     assert names(plan) == ["j", "k"]
-    for item in plan.items:
-        cache4.commit(item.seq.request_id, len(item.token_ids))
+    for item in plan.portions:
+        cache4.commit(item.request.request_id, len(item.token_ids))
     assert tight.schedule_ahead(plan) is None             # j needs a second page, none is free
     tight.complete(plan, [1, 2])
     # a request waits and those that go on fill every seat: the step after is planned without it; the seat of a
@@ -315,13 +315,13 @@ def test_the_step_after_is_planned_ahead_only_when_that_is_plain():
         two.submit(s_)
     plan = two.schedule()
     assert names(plan) == ["g", "h"]
-    for item in plan.items:
-        cache3.commit(item.seq.request_id, len(item.token_ids))
+    for item in plan.portions:
+        cache3.commit(item.request.request_id, len(item.token_ids))
     ahead = two.schedule_ahead(plan)
     assert names(ahead) == ["g", "h"]
     two.complete(plan, [1, 2])
-    for item in ahead.items:
-        cache3.commit(item.seq.request_id, 1)
+    for item in ahead.portions:
+        cache3.commit(item.request.request_id, 1)
     after = two.schedule_ahead(ahead)
     assert names(after) == ["h"] and after.feeds == (1,)      # g ends with the pending token; its seat is still taken
     two.complete(ahead, [3, 4])

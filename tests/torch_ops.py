@@ -101,7 +101,7 @@ class TorchOps(Ops):
 def plain_sample(logits, temperature, seeds, counters):
     """argmax where t <= 0; else the first index whose cumulative softmax weight (float64)
     exceeds u * total, u from the request's (seed, counter)."""
-    from distie_amd.sampling import uniform_of
+    from engine_util import plain_uniform as uniform_of
 
     out = []
     for row, t, seed, counter in zip(logits.double().cpu(), temperature.tolist(), seeds.tolist(), counters.tolist()):
