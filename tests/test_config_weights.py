@@ -166,3 +166,62 @@ def test_random_weights_mode_writes_a_model_folder(tmp_path):
     # the plain implementation reads the folder too
     logits = plain.forward(wa, plain.read_config(a), [1, 2, 3])
     assert logits.shape == (3, 323)
+
+
+def _write_sharded(folder, cfg, weights, pieces=3):
+    """A folder whose tensors are spread over several files, named by `model.safetensors.index.json`."""
+    from safetensors.torch import save_file
+
+    folder.mkdir(parents=True, exist_ok=True)
+    (folder / "config.json").write_text(json.dumps(cfg))
+    names = list(weights)
+    weight_map = {}
+    for i in range(pieces):
+        file = f"model-{i + 1:05d}-of-{pieces:05d}.safetensors"
+        mine = names[i::pieces]                       # interleaved: a layer's tensors lie in different files
+        save_file({n: weights[n].contiguous() for n in mine}, str(folder / file))
+        weight_map.update({n: file for n in mine})
+    (folder / "model.safetensors.index.json").write_text(json.dumps({"metadata": {}, "weight_map": weight_map}))
+
+
+def test_sharded_folder_loads_as_the_single_file_does(tmp_path):
+    cfg = plain.TINY_B
+    weights = plain.random_weights(cfg, 3, std=0.1)
+    plain.write_model_dir(tmp_path / "one", cfg, weights)
+    _write_sharded(tmp_path / "many", cfg, weights)
+    single, sharded = (Model(load_model_config(tmp_path / name).model_spec()) for name in ("one", "many"))
+    load_into(single, tmp_path / "one", "cpu", torch.float32)
+    load_into(sharded, tmp_path / "many", "cpu", torch.float32)
+    assert torch.equal(single.embedding, sharded.embedding) and torch.equal(single.head, sharded.head)
+    for a, b in zip(single.blocks, sharded.blocks):
+        assert torch.equal(a.mixer.qkv_weight, b.mixer.qkv_weight) and torch.equal(a.mixer.qkv_bias_t, b.mixer.qkv_bias_t)
+        assert torch.equal(a.feed_forward.gate_up_weight, b.feed_forward.gate_up_weight)
+        assert torch.equal(a.feed_forward_norm.weight, b.feed_forward_norm.weight)
+    # a tensor that the index names but no file holds, and one that no file of the index holds at all
+    broken = dict(weights)
+    del broken["model.layers.2.mlp.down_proj.weight"]
+    _write_sharded(tmp_path / "broken", cfg, broken)
+    index = json.loads((tmp_path / "broken" / "model.safetensors.index.json").read_text())
+    files = sorted(set(index["weight_map"].values()))
+    holder = index["weight_map"]["model.norm.weight"]
+    index["weight_map"]["model.norm.weight"] = [f for f in files if f != holder][0]
+    (tmp_path / "broken" / "model.safetensors.index.json").write_text(json.dumps(index))
+    model = Model(load_model_config(tmp_path / "broken").model_spec())
+    with pytest.raises(WeightsError) as info:
+        load_into(model, tmp_path / "broken", "cpu", torch.float32)
+    assert set(info.value.missing) == {"model.layers.2.mlp.down_proj.weight", "model.norm.weight"}
+
+
+def test_a_half_precision_file(tmp_path):
+    """fp16 is not a precision of the engine: a bfloat16 engine keeps such tensors in bfloat16, a float32
+    engine in float32, each converted from the stored values."""
+    cfg = plain.TINY_A
+    weights = plain.random_weights(cfg, 4, std=0.1, dtype=torch.float16)
+    plain.write_model_dir(tmp_path / "m", cfg, weights)
+    for engine_dtype in (torch.bfloat16, torch.float32):
+        model = Model(load_model_config(tmp_path / "m").model_spec())
+        load_into(model, tmp_path / "m", "cpu", engine_dtype)
+        assert model.embedding.dtype == engine_dtype and model.blocks[1].feed_forward.down_weight.dtype == engine_dtype
+        assert torch.equal(model.embedding, weights["model.embed_tokens.weight"].to(engine_dtype))
+        assert torch.equal(model.blocks[1].feed_forward.down_weight,
+                           weights["model.layers.1.mlp.down_proj.weight"].to(engine_dtype))

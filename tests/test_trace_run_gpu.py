@@ -83,8 +83,6 @@ def test_replay_mixed_trace(tmp_path, name, dtype):
         rows = [begin + w for begin, want, _ in pieces for w in want]
         stacked = torch.cat([l for _, _, l in pieces])
         # compare at the rows that were asked for
-        class _Sel:
-            pass
         diff = (stacked - want_all[rows]).abs().max().item()
         scale = want_all.abs().max().item()
         assert diff < (1e-4 if dtype == "float32" else scale / 16), (r, diff)
