@@ -1,5 +1,5 @@
 from .block_pool import BlockPool, OutOfBlocks
-from .manager import GONE, CacheGroup, CacheManager, LayerCache, RequestCache, pages_needed
+from .manager import GONE, CacheGroup, CacheManager, CacheView, LayerCache, RequestCache, pages_needed
 
-__all__ = ["BlockPool", "OutOfBlocks", "GONE", "CacheGroup", "CacheManager", "LayerCache",
+__all__ = ["BlockPool", "OutOfBlocks", "GONE", "CacheGroup", "CacheManager", "CacheView", "LayerCache",
            "RequestCache", "pages_needed"]

@@ -1,13 +1,13 @@
 """The cache manager: pages of keys and values with a block table for each request, and
 slots for per-request state of fixed size.
 
-Layers are put into *groups* by what their mixer keeps (`PagedKV(kv_heads, head_dim,
-window)`): layers that keep every key form one group, layers that keep a window of the
-same length another. Every group has pages of its own: its own id pool, its own slabs
-`k, v : [layers of the group, pages + 1, kv_heads, block_size, head_dim]` (the last page
-is a sink that is never handed out: padding rows of a captured decode step write there,
-as in worker/src/inference/torch_engine.py:439-446) and, for each request, its own block
-table. A table is addressed by position: entry i holds the page of positions
+A mixer declares what it keeps (`PagedTensors`: tensors per page and a window, or `FixedState`:
+tensors per request); the manager allocates what is declared and knows nothing of what the tensors
+mean. Mixers are put into *groups* by their declaration: attention layers that keep every key form one
+group, those that keep a window of the same length another. Every group has pages of its own: its own
+id pool, for each declared tensor a slab `[mixers of the group, pages + 1, *shape of a page]` (the last
+page is a sink that is never handed out: padding rows of a captured decode step write there, as in
+worker/src/inference/torch_engine.py:439-446) and, for each request, its own block table. A table is addressed by position: entry i holds the page of positions
 i*block_size .. (i+1)*block_size - 1, or -1 once a window has passed that page and it
 was given back. Pages are handed out when a step needs them (`reserve`), given back when
 a request ends (`release`), is preempted (`reset`), or a window has passed them
@@ -16,9 +16,12 @@ a request ends (`release`), is preempted (`reset`), or a window has passed them
 The reference has one group and Python lists of ids on each sequence
 (worker/src/inference/kv_cache.py:61-103, worker/src/inference/scheduler.py:50).
 
-Slots: every live request owns one slot id. Layers whose mixer declares `FixedState`
-get a float32 slab `[slots + 1, *shape]` each; a request's row is zeroed when the slot is
-taken. The model of this engine has no such layer, the slots exist all the same.
+Slots: every live request owns one slot id. A mixer that declares `FixedState` gets, for each
+tensor it names, a slab `[slots + 1, *shape]`; a request's rows are zeroed when the slot is
+taken. The model of this engine has no such mixer, the slots exist all the same.
+
+A layer may hold several mixers (its block says which, by name): `requirements[l]` maps the name of
+each mixer of layer l to its declaration, and `layer(l)[name]` is that mixer's view.
 """
 
 from __future__ import annotations
@@ -28,7 +31,7 @@ from typing import Dict, Hashable, List, Optional, Sequence
 
 import torch
 
-from ..parts.base import FixedState, PagedKV
+from ..parts.base import FixedState, PagedTensors
 from .block_pool import BlockPool, OutOfBlocks
 
 GONE = -1
@@ -43,23 +46,39 @@ def pages_needed(token_count: int, block_size: int) -> int:
     return (token_count + block_size - 1) // block_size
 
 
-@dataclass
-class LayerCache:
-    """What a mixer gets: its group's index and its own layer's slabs (or its state slab)."""
+class CacheView:
+    """What one mixer gets: the tensors it declared, by name (`view["k"]`): for paged tensors its own
+    layer's slab `[pages + 1, *page shape]` and the index of its group (whose block table and slots of the
+    step are `meta.groups[group]`); for fixed state `[slots + 1, *shape]` (rows by `meta.state_slots`)."""
 
-    group: int = -1
-    k: Optional[torch.Tensor] = None
-    v: Optional[torch.Tensor] = None
-    state: Optional[torch.Tensor] = None
+    def __init__(self, group: int = -1, tensors: Optional[Dict[str, torch.Tensor]] = None) -> None:
+        self.group = group
+        self.tensors = tensors or {}
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        return self.tensors[name]
+
+
+class LayerCache:
+    """The views of one layer's mixers, by the mixer's name in its block."""
+
+    def __init__(self) -> None:
+        self.views: Dict[str, CacheView] = {}
+
+    def __getitem__(self, name: str) -> CacheView:
+        return self.views[name]
 
 
 @dataclass
 class CacheGroup:
-    requirement: PagedKV
-    layers: List[int]
+    requirement: PagedTensors
+    members: List[tuple]                  # (layer, mixer name) of every mixer that shares these pages
     pool: BlockPool
-    k: Optional[torch.Tensor] = None      # [layers, pages + 1, KH, P, D]
-    v: Optional[torch.Tensor] = None      # [layers, pages + 1, KH, D, P]
+    tensors: Dict[str, torch.Tensor] = field(default_factory=dict)    # name -> [members, pages + 1, *page shape]
+
+    @property
+    def layers(self) -> List[int]:
+        return [layer for layer, _ in self.members]
 
     @property
     def sink_page(self) -> int:
@@ -76,8 +95,9 @@ class RequestCache:
 class CacheManager:
     def __init__(self, requirements: Sequence, block_size: int, num_blocks: int, num_slots: int,
                  device=None, dtype=torch.float32, allocate: bool = True) -> None:
-        """`requirements[l]` is what layer l's mixer keeps: PagedKV, FixedState or None.
-        `allocate=False` makes the book-keeping without the slabs (for tests of decisions)."""
+        """`requirements[l]`: what the mixers of layer l keep, `{mixer name: PagedTensors | FixedState |
+        None}` (a bare declaration stands for `{"mixer": declaration}`). `dtype`: of paged tensors that
+        name none. `allocate=False` makes the book-keeping without the slabs (for tests of decisions)."""
         if block_size < 1 or num_blocks < 1 or num_slots < 1:
             raise ValueError("block_size, num_blocks and num_slots must be >= 1")
         self.block_size = int(block_size)
@@ -86,50 +106,55 @@ class CacheManager:
         self.device = device
         self.dtype = dtype
         self.groups: List[CacheGroup] = []
-        self._layer_view: Dict[int, LayerCache] = {}
-        self._state_layers: Dict[int, torch.Tensor] = {}
-        by_need: Dict[PagedKV, CacheGroup] = {}
-        for layer, need in enumerate(requirements):
-            if isinstance(need, PagedKV):
-                if need not in by_need:
-                    by_need[need] = CacheGroup(need, [], BlockPool(self.num_blocks))
-                    self.groups.append(by_need[need])
-                by_need[need].layers.append(layer)
-            elif isinstance(need, FixedState):
-                slab = torch.zeros((self.num_slots + 1, *need.shape), dtype=torch.float32, device=device) \
-                    if allocate else None
-                self._state_layers[layer] = slab
-                self._layer_view[layer] = LayerCache(state=slab)
-            elif need is None:
-                self._layer_view[layer] = LayerCache()
-            else:
-                raise TypeError(f"layer {layer}: unknown cache requirement {need!r}")
+        self._layers: List[LayerCache] = []
+        self._state_slabs: List[torch.Tensor] = []
+        by_need: Dict[PagedTensors, CacheGroup] = {}
+        for layer, needs in enumerate(requirements):
+            if not isinstance(needs, dict):
+                needs = {"mixer": needs}
+            views = LayerCache()
+            self._layers.append(views)
+            for name, need in needs.items():
+                if isinstance(need, PagedTensors):
+                    if need not in by_need:
+                        by_need[need] = CacheGroup(need, [], BlockPool(self.num_blocks))
+                        self.groups.append(by_need[need])
+                    by_need[need].members.append((layer, name))
+                elif isinstance(need, FixedState):
+                    slabs = {}
+                    for decl in need.tensors:
+                        if allocate:
+                            slabs[decl.name] = torch.zeros((self.num_slots + 1, *decl.shape),
+                                                           dtype=decl.dtype or torch.float32, device=device)
+                            self._state_slabs.append(slabs[decl.name])
+                    views.views[name] = CacheView(tensors=slabs)
+                elif need is None:
+                    views.views[name] = CacheView()
+                else:
+                    raise TypeError(f"layer {layer}, {name}: unknown cache requirement {need!r}")
         for index, group in enumerate(self.groups):
             need = group.requirement
             if allocate:
-                lead = (len(group.layers), self.num_blocks + 1, need.num_kv_heads)
-                group.k = torch.zeros(lead + (self.block_size, need.head_dim), dtype=dtype, device=device)
-                group.v = torch.zeros(lead + (need.head_dim, self.block_size), dtype=dtype, device=device)
-            for i, layer in enumerate(group.layers):
-                self._layer_view[layer] = LayerCache(
-                    group=index, k=group.k[i] if allocate else None, v=group.v[i] if allocate else None)
+                for decl in need.tensors:
+                    shape = (len(group.members), self.num_blocks + 1) + need.page_shape(decl, self.block_size)
+                    group.tensors[decl.name] = torch.zeros(shape, dtype=decl.dtype or dtype, device=device)
+            for i, (layer, name) in enumerate(group.members):
+                self._layers[layer].views[name] = CacheView(
+                    group=index, tensors={n: slab[i] for n, slab in group.tensors.items()})
         self.slots = BlockPool(self.num_slots)
         self._requests: Dict[Hashable, RequestCache] = {}
 
     # ---------------------------------------------------------------- views
     def layer(self, layer: int) -> LayerCache:
-        return self._layer_view[layer]
+        return self._layers[layer]
 
     @property
     def sink_slot(self) -> int:
         return self.num_slots
 
     def bytes(self) -> int:
-        total = 0
-        for group in self.groups:
-            if group.k is not None:
-                total += 2 * group.k.numel() * group.k.element_size()
-        return total
+        slabs = [t for group in self.groups for t in group.tensors.values()] + self._state_slabs
+        return sum(t.numel() * t.element_size() for t in slabs)
 
     # ------------------------------------------------------------- requests
     def __contains__(self, request_id) -> bool:
@@ -149,9 +174,8 @@ class CacheManager:
             (slot,) = self.slots.allocate(1)
         except OutOfBlocks as exc:
             raise OutOfBlocks(f"no free state slot (all {self.num_slots} in use)") from exc
-        for slab in self._state_layers.values():
-            if slab is not None:
-                slab[slot].zero_()
+        for slab in self._state_slabs:
+            slab[slot].zero_()
         entry = RequestCache(slot=slot, tables=[[] for _ in self.groups])
         self._requests[request_id] = entry
         return entry
@@ -240,9 +264,8 @@ class CacheManager:
         """Preemption by recompute: every page back, nothing cached, the slot's state zeroed."""
         entry = self._requests[request_id]
         self._give_back_pages(entry)
-        for slab in self._state_layers.values():
-            if slab is not None:
-                slab[entry.slot].zero_()
+        for slab in self._state_slabs:
+            slab[entry.slot].zero_()
 
     def release(self, request_id) -> None:
         """The request is over: pages and slot back."""

@@ -37,13 +37,12 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """A layer = an arrangement (`block`) of a mixer, a feed-forward and their norms."""
+    """A layer = an arrangement (`block`) and the parts it arranges, under the names that the block's
+    class gives them (the pre-norm block of this package: `mixer`, `feed_forward`, `mixer_norm`,
+    `feed_forward_norm`; another block may arrange four norms, two mixers, or no feed-forward)."""
 
     block: PartSpec
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    parts: Mapping[str, PartSpec] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)
@@ -256,9 +255,8 @@ class Qwen2Config:
         for l in range(self.num_hidden_layers):
             base = f"model.layers.{l}."
             norm = {"eps": self.rms_norm_eps, "size": self.hidden_size}
-            layers.append(LayerSpec(
-                block=PartSpec("prenorm_residual"),
-                mixer=PartSpec("attention", base + "self_attn.", {
+            layers.append(LayerSpec(PartSpec("prenorm_residual"), {
+                "mixer": PartSpec("attention", base + "self_attn.", {
                     "hidden_size": self.hidden_size,
                     "num_heads": self.num_attention_heads,
                     "num_kv_heads": self.num_key_value_heads,
@@ -269,13 +267,13 @@ class Qwen2Config:
                     "scale": self.head_dim ** -0.5,
                     "position": PartSpec("rope", "", {"dim": self.head_dim, "theta": self.rope_theta}),
                 }),
-                feed_forward=PartSpec("swiglu", base + "mlp.", {
+                "feed_forward": PartSpec("swiglu", base + "mlp.", {
                     "hidden_size": self.hidden_size,
                     "intermediate_size": self.intermediate_size,
                 }),
-                mixer_norm=PartSpec("rmsnorm", base + "input_layernorm.", norm),
-                feed_forward_norm=PartSpec("rmsnorm", base + "post_attention_layernorm.", norm),
-            ))
+                "mixer_norm": PartSpec("rmsnorm", base + "input_layernorm.", norm),
+                "feed_forward_norm": PartSpec("rmsnorm", base + "post_attention_layernorm.", norm),
+            }))
         return ModelSpec(
             architecture=self.architecture,
             vocab_size=self.vocab_size,
@@ -288,6 +286,6 @@ class Qwen2Config:
             final_norm=PartSpec("rmsnorm", "model.norm.", {"eps": self.rms_norm_eps, "size": self.hidden_size}),
             head=PartSpec("lm_head", "lm_head.", {
                 "vocab_size": self.vocab_size, "hidden_size": self.hidden_size,
-                "tied": self.tie_word_embeddings}),
+                "tied_to": "model.embed_tokens.weight" if self.tie_word_embeddings else None}),
             eos_token_ids=self.eos_token_ids,
         )

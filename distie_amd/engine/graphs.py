@@ -14,12 +14,11 @@ tried again, and after a few failures captured steps stay off. Failures are coun
 The step's metadata reaches the device with one copy from pinned host memory before the
 replay; nothing inside the graph depends on a Python number.
 
-One number of the step is frozen into a graph all the same: the longest context it is made for,
-from which decode attention derives how many runs of keys a request may be cut into and where a
-wave first looks for its pages. A graph made for the model's limit would suit a 2,000-token
-context badly, so a bucket keeps one graph per class of context length (1,024, 1,536, 2,048,
-3,072, ... up to the limit), each captured when a step first needs it; a step replays the graph
-of the smallest class that holds its longest request.
+One number of the step is frozen into a graph all the same: the longest context it is made for
+(`BatchMeta.max_kv`). Which lengths deserve a graph of their own is the parts' business
+(`Part.capture_context`; attention answers with classes of length, since it cuts the keys into runs
+by that number): a bucket keeps one graph per answer of the model, each captured when a step first
+needs it.
 """
 
 from __future__ import annotations
@@ -55,21 +54,6 @@ def bucket_for(buckets: Sequence[int], rows: int) -> int:
     return buckets[bisect.bisect_left(buckets, rows)]
 
 
-def context_classes(limit: int, first: int = 1024) -> Tuple[int, ...]:
-    """(4096) -> 1024, 1536, 2048, 3072, 4096; (700) -> 700: steps of a factor 1.5 or 1.33, so a
-    graph's runs of keys are at most that much longer than the step's own would be."""
-    if limit < 1 or first < 1:
-        raise ValueError("context lengths must be >= 1")
-    out = {limit}
-    c = first
-    while c < limit:
-        out.add(c)
-        if c + c // 2 < limit and c >= 2:
-            out.add(c + c // 2)
-        c *= 2
-    return tuple(sorted(out))
-
-
 class _Bucket:
     def __init__(self, size: int, builder, device) -> None:
         self.size = size
@@ -84,15 +68,12 @@ class _Bucket:
 
 
 class DecodeGraphs:
-    FIRST_CONTEXT = 1024        # the shortest class of context length
-
     RETRY_AFTER_STEPS = 512     # after a failure, steps run uncaptured for so long before a capture is tried again
     MAX_FAILURES = 3            # ... and after so many failures for good
 
     def __init__(self, runner, max_batch: int) -> None:
         self.runner = runner
         self.buckets = decode_buckets(max_batch)
-        self.contexts = context_classes(runner.max_model_len, self.FIRST_CONTEXT)
         self.max_batch = max_batch
         self._made: Dict[int, _Bucket] = {}
         self._pool = None
@@ -161,7 +142,9 @@ class DecodeGraphs:
         bucket.copied.record()
         if feed is not None and feed.shape[0]:
             bucket.dev[:feed.shape[0]].copy_(feed)       # the token ids lead the packed buffer
-        limit = self.contexts[bisect.bisect_left(self.contexts, max_kv)]
+        limit = runner.model.capture_context(max_kv, runner.max_model_len)
+        if limit < max_kv:
+            raise RuntimeError(f"a part asks for a captured step made for {limit} tokens to serve {max_kv}")
         made = bucket.graphs.get(limit)
         if made is None:
             logits = self._capture(bucket, limit)

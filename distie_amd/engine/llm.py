@@ -111,9 +111,13 @@ class LLM:
         self.steps_ahead = 0          # steps launched before the tokens of the step before were known
         self._outputs: Dict[Hashable, RequestOutput] = {}     # until `generate`, `stream` or `take_output` hands them out
         if ec.use_graphs and hasattr(ops, "graphs_supported") and ops.graphs_supported():
-            from .graphs import DecodeGraphs
+            if self.model.capturable:
+                from .graphs import DecodeGraphs
 
-            self.runner.graphs = DecodeGraphs(self.runner, ec.max_seqs)
+                self.runner.graphs = DecodeGraphs(self.runner, ec.max_seqs)
+            else:
+                names = sorted({type(p).__name__ for p in self.model.parts() if not p.capturable})
+                _log.info("decode steps are not captured: %s cannot be recorded into a graph", ", ".join(names))
         if ec.tune_products and hasattr(ops, "tune_library_products"):
             self._tune_products()
         _log.info("engine ready: %s dtype=%s pages=%d x %d tokens, %d cache groups, %.1f MiB cache",

@@ -1,9 +1,9 @@
 """A model put together from parts, as a `ModelSpec` describes it.
 
-`Model` knows no architecture: it builds the embedding, one block per `LayerSpec`, the
-final norm and the head from the registries of parts, asks each part for the tensors it
-wants, and runs the blocks in the order the spec gives (an order may name a layer twice,
-or let a layer use another layer's cache). It computes only through the kernel surface.
+`Model` knows no architecture and no part: it builds the embedding, one block per `LayerSpec` (the
+block builds the parts it arranges), the final norm and the head from the registries of parts, asks
+every part for the tensors it wants, and runs the blocks in the order the spec gives (an order may name
+a layer twice, or let a layer use another layer's cache). It computes only through the parts.
 
 The flow of one step is the reference's `forward_batch`
 (worker/src/inference/qwen2/model.py:369-380): embed, blocks, select the rows whose
@@ -23,42 +23,59 @@ from ..parts import ParamSpec, ResidualStream, StepContext, build_part
 class Model:
     def __init__(self, spec: ModelSpec) -> None:
         self.spec = spec
-        self.blocks = []
-        for layer in spec.layers:
-            mixer = build_part("mixer", layer.mixer)
-            feed_forward = build_part("feed_forward", layer.feed_forward)
-            mixer_norm = build_part("norm", layer.mixer_norm)
-            feed_forward_norm = build_part("norm", layer.feed_forward_norm)
-            self.blocks.append(build_part("block", layer.block, mixer, feed_forward, mixer_norm, feed_forward_norm))
+        self.embed = build_part("embedding", spec.embedding)
+        self.blocks = [build_part("block", layer.block, layer.parts) for layer in spec.layers]
         self.final_norm = build_part("norm", spec.final_norm)
         self.position = build_part("position", spec.position) if spec.position is not None else None
-        self.tied_head = bool(spec.head.get("tied", False))
-        self.embedding: Optional[torch.Tensor] = None
-        self.head: Optional[torch.Tensor] = None
+        self.lm_head = build_part("head", spec.head)
         for call in spec.order:
             if not 0 <= call.layer < len(self.blocks) or not 0 <= call.cache_layer < len(self.blocks):
                 raise ValueError(f"run order names layer {call.layer} / cache of {call.cache_layer}, "
                                  f"the model has {len(self.blocks)} layers")
 
     # ------------------------------------------------------------ tensors
-    def _parts(self):
-        """(part, its spec) for every part that owns tensors."""
+    def parts(self):
+        """Every part of the model, in the order in which their tensors are declared."""
+        yield from self.embed.parts()
         for block in self.blocks:
-            for part in (block.mixer_norm, block.mixer, block.feed_forward_norm, block.feed_forward, block):
-                yield part
-        yield self.final_norm
+            yield from block.parts()
+        yield from self.final_norm.parts()
         if self.position is not None:
-            yield self.position
+            yield from self.position.parts()
+        yield from self.lm_head.parts()
+
+    @property
+    def embedding(self) -> Optional[torch.Tensor]:
+        return getattr(self.embed, "weight", None)
+
+    @property
+    def head(self) -> Optional[torch.Tensor]:
+        return getattr(self.lm_head, "weight", None)
+
+    @property
+    def capturable(self) -> bool:
+        """Every part can be recorded into a device graph."""
+        return all(part.capturable for part in self.parts())
+
+    def capture_context(self, longest: int, limit: int) -> int:
+        """The context length a captured step should be made for to serve a step whose longest request
+        holds `longest` tokens: the largest of the parts' answers, `limit` if no part cares."""
+        answers = [a for a in (part.capture_context(longest, limit) for part in self.parts()) if a is not None]
+        return max(answers) if answers else limit
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         """Checkpoint name -> shape, in a fixed order (embedding, layers, final norm, head)."""
-        s = self.spec
-        out = {s.embedding.prefix + "weight": ParamSpec((s.vocab_size, s.hidden_size))}
-        for part in self._parts():
+        out: Dict[str, ParamSpec] = {}
+        for part in self.parts():
             for local, spec in part.param_specs().items():
-                out[part.spec.prefix + local] = spec
-        if not self.tied_head:
-            out[s.head.prefix + "weight"] = ParamSpec((s.vocab_size, s.hidden_size))
+                name = part.spec.prefix + local
+                if name in out and out[name] != spec:
+                    raise ValueError(f"two parts declare {name} with different shapes")
+                out[name] = spec
+        for part in self.parts():
+            for local, name in part.shared_specs().items():
+                if name not in out:
+                    raise ValueError(f"{part.spec.kind} wants to share {name}, which no part declares")
         return out
 
     @classmethod
@@ -66,39 +83,42 @@ class Model:
         return cls(spec).param_specs()
 
     def ignorable_names(self) -> List[str]:
-        """Tensors a file may hold that the model does not use: the head's copy when it is
-        tied to the embedding."""
-        return [self.spec.head.prefix + "weight"] if self.tied_head else []
+        """Tensors a file may hold that the model does not use (the head's copy when it is tied to the
+        embedding)."""
+        return [part.spec.prefix + local for part in self.parts() for local in part.optional_names()]
 
     def load_tensors(self, fetch: Callable[[str], torch.Tensor]) -> None:
-        """`fetch(name)` gives each declared tensor, on the device, in the kept dtype."""
-        s = self.spec
-        self.embedding = fetch(s.embedding.prefix + "weight").contiguous()
-        for part in self._parts():
-            names = part.param_specs()
-            if names:
-                part.load({local: fetch(part.spec.prefix + local) for local in names})
-        # tied: one buffer (worker/src/inference/qwen2/model.py:302-303)
-        self.head = self.embedding if self.tied_head else fetch(s.head.prefix + "weight").contiguous()
+        """`fetch(name)` gives each declared tensor, on the device, in the kept dtype. A tensor that two
+        parts use is fetched once: both hold the same object."""
+        fetched: Dict[str, torch.Tensor] = {}
+
+        def get(name: str) -> torch.Tensor:
+            if name not in fetched:
+                fetched[name] = fetch(name).contiguous()
+            return fetched[name]
+
+        for part in self.parts():
+            wanted = {local: part.spec.prefix + local for local in part.param_specs()}
+            wanted.update(part.shared_specs())
+            if wanted:
+                part.load({local: get(name) for local, name in wanted.items()})
 
     def prepare(self, ops) -> None:
         """Once after loading, with the kernel surface the model will run on."""
-        for part in self._parts():
+        for part in self.parts():
             part.prepare(ops)
-        ops.prepare_linear(self.head)
 
     def cache_requirements(self) -> list:
-        return [block.mixer.cache_requirement() for block in self.blocks]
+        """Per layer: what each mixer of the layer's block keeps, by the mixer's name in the block."""
+        return [block.cache_requirements() for block in self.blocks]
 
     def weight_bytes(self) -> int:
         seen, total = set(), 0
-        tensors = [self.embedding, self.head]
-        for part in self._parts():
-            tensors += [v for v in vars(part).values() if isinstance(v, torch.Tensor)]
-        for t in tensors:
-            if t is not None and t.data_ptr() not in seen:
-                seen.add(t.data_ptr())
-                total += t.numel() * t.element_size()
+        for part in self.parts():
+            for t in vars(part).values():
+                if isinstance(t, torch.Tensor) and t.data_ptr() not in seen:
+                    seen.add(t.data_ptr())
+                    total += t.numel() * t.element_size()
         return total
 
     # ------------------------------------------------------------ the step
@@ -107,22 +127,20 @@ class Model:
         """ids int32 [T] -> float32 logits [R, vocab] at `want_rows` (int32 [R]); None if no
         row is wanted (the step then only fills the cache). `every_row`: `want_rows` names every row
         in order (a captured decode step), so nothing needs to be gathered."""
-        stream = ResidualStream(ops.embed(ids, self.embedding))
+        stream = ResidualStream(self.embed.forward(ops, ids, meta))
         if self.position is not None:
             self.position.on_embedding(ops, stream.hidden, meta)
         ctx = StepContext(meta, act_dtype)
         for call in self.spec.order:
-            view = cache.layer(call.cache_layer)
-            ctx.state = view.state
-            self.blocks[call.layer].forward(ops, stream, ctx, view, call.writes_cache)
+            self.blocks[call.layer].forward(ops, stream, ctx, cache.layer(call.cache_layer), call.writes_cache)
         if want_rows is None:
             return None
         if every_row:
             normed = self.final_norm.of_stream(ops, stream, act_dtype)
-            return ops.linear_f32out(normed, self.head)
+            return self.lm_head.forward(ops, normed)
         hidden = ops.gather_rows(stream.hidden, want_rows)
         if stream.pending is not None:
             normed = self.final_norm.add_apply(ops, hidden, ops.gather_rows(stream.pending, want_rows), act_dtype)
         else:
             normed = self.final_norm.apply(ops, hidden, act_dtype)
-        return ops.linear_f32out(normed, self.head)
+        return self.lm_head.forward(ops, normed)

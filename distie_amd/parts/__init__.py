@@ -1,6 +1,8 @@
-from . import attention, block, feed_forward, norm, position  # noqa: F401  (registration)
-from .base import (Block, FeedForward, FixedState, Mixer, Norm, PagedKV, ParamSpec, Part,
-                   PositionEncoding, ResidualStream, StepContext, build_part, register_part)
+from . import attention, block, embedding, feed_forward, norm, position  # noqa: F401  (registration)
+from .attention import PagedKV
+from .base import (PAGE, Block, Embedding, FeedForward, FixedState, Head, Mixer, Norm, PagedTensors, ParamSpec, Part,
+                   PositionEncoding, ResidualStream, StepContext, TensorDecl, build_part, register_part)
 
-__all__ = ["Block", "FeedForward", "FixedState", "Mixer", "Norm", "PagedKV", "ParamSpec", "Part",
-           "PositionEncoding", "ResidualStream", "StepContext", "build_part", "register_part"]
+__all__ = ["PAGE", "Block", "Embedding", "FeedForward", "FixedState", "Head", "Mixer", "Norm", "PagedKV", "PagedTensors",
+           "ParamSpec", "Part", "PositionEncoding", "ResidualStream", "StepContext", "TensorDecl", "build_part",
+           "register_part"]

@@ -12,13 +12,41 @@ The three projections are one matrix product: their weights are stacked at load.
 
 from __future__ import annotations
 
+import bisect
+from typing import Optional, Tuple
+
 import torch
 
 from ..config.model_config import PartSpec
-from .base import Mixer, PagedKV, ParamSpec, build_part, register_part
+from .base import PAGE, Mixer, PagedTensors, ParamSpec, TensorDecl, build_part, register_part
+
+
+def PagedKV(num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> PagedTensors:
+    """What attention keeps for every token, in the layout its kernels read: keys as
+    `[kv_heads, page, head_dim]` per page, values transposed inside a page, `[kv_heads, head_dim, page]`,
+    so that the key index is contiguous for the matrix cores."""
+    return PagedTensors((TensorDecl("k", (num_kv_heads, PAGE, head_dim)),
+                         TensorDecl("v", (num_kv_heads, head_dim, PAGE))), window)
+
+
+def context_classes(limit: int, first: int = 1024) -> Tuple[int, ...]:
+    """(4096) -> 1024, 1536, 2048, 3072, 4096; (700) -> 700: steps of a factor 1.5 or 1.33, so a
+    captured step's runs of keys are at most that much longer than the step's own would be."""
+    if limit < 1 or first < 1:
+        raise ValueError("context lengths must be >= 1")
+    out = {limit}
+    c = first
+    while c < limit:
+        out.add(c)
+        if c + c // 2 < limit and c >= 2:
+            out.add(c + c // 2)
+        c *= 2
+    return tuple(sorted(out))
 
 
 class Attention(Mixer):
+    FIRST_CONTEXT = 1024        # the shortest class of context length that captured steps are made for
+
     def __init__(self, spec: PartSpec) -> None:
         super().__init__(spec)
         p = spec.params
@@ -69,11 +97,20 @@ class Attention(Mixer):
         ops.prepare_linear(self.qkv_weight, rotary=(self.num_heads, self.num_kv_heads, self.head_dim))
         ops.prepare_linear(self.out_weight)
 
+    def capture_context(self, longest: int, limit: int):
+        """Decode attention cuts the keys into runs by the longest context of the step, and that number is
+        frozen into a captured step: a graph made for the model's limit would suit a 2,000-token context
+        badly. So captured steps are made per class of context length (1,024, 1,536, 2,048, 3,072, ... the
+        limit), and a step uses the smallest class that holds its longest request."""
+        classes = context_classes(limit, self.FIRST_CONTEXT)
+        return classes[min(bisect.bisect_left(classes, longest), len(classes) - 1)]
+
     def forward(self, ops, x, ctx, cache, writes_cache: bool):
-        qkv = ops.linear_rope_kv_write(x, self.qkv_weight, self.qkv_bias_t, ctx.meta, cache.group, cache.k, cache.v,
+        k_cache, v_cache = cache["k"], cache["v"]
+        qkv = ops.linear_rope_kv_write(x, self.qkv_weight, self.qkv_bias_t, ctx.meta, cache.group, k_cache, v_cache,
                                        self.position.rotary(), self.num_heads, self.num_kv_heads, self.head_dim,
                                        writes_cache)
-        mixed = ops.paged_attention(qkv, ctx.meta, cache.group, cache.k, cache.v, self.num_heads,
+        mixed = ops.paged_attention(qkv, ctx.meta, cache.group, k_cache, v_cache, self.num_heads,
                                     self.num_kv_heads, self.head_dim, self.scale, self.window)
         return ops.linear(mixed, self.out_weight, self.out_bias_t)
 

@@ -8,9 +8,11 @@ from .base import Block, ResidualStream, StepContext, register_part
 
 
 class PreNormResidual(Block):
+    CHILDREN = {"mixer_norm": "norm", "mixer": "mixer", "feed_forward_norm": "norm", "feed_forward": "feed_forward"}
+
     def forward(self, ops, stream: ResidualStream, ctx: StepContext, cache, writes_cache: bool) -> None:
         normed = self.mixer_norm.of_stream(ops, stream, ctx.act_dtype)
-        stream.pending = self.mixer.forward(ops, normed, ctx, cache, writes_cache)
+        stream.pending = self.mixer.forward(ops, normed, ctx, cache["mixer"], writes_cache)
         normed = self.feed_forward_norm.of_stream(ops, stream, ctx.act_dtype)
         stream.pending = self.feed_forward.forward(ops, normed, ctx)
 

@@ -64,7 +64,7 @@ def test_pool_threads():
 
 
 def manager(block=4, pages=12, slots=4, window=6):
-    needs = [PagedKV(2, 16), PagedKV(2, 16, window), PagedKV(2, 16), None, FixedState((3,))]
+    needs = [PagedKV(2, 16), PagedKV(2, 16, window), PagedKV(2, 16), None, FixedState.of((3,))]
     return CacheManager(needs, block, pages, slots, allocate=False)
 
 
@@ -72,7 +72,7 @@ def test_groups_by_need():
     m = manager()
     assert len(m.groups) == 2
     assert m.groups[0].layers == [0, 2] and m.groups[1].layers == [1]
-    assert m.layer(0).group == 0 and m.layer(1).group == 1 and m.layer(3).group == -1
+    assert m.layer(0)["mixer"].group == 0 and m.layer(1)["mixer"].group == 1 and m.layer(3)["mixer"].group == -1
 
 
 def test_reserve_commit_release_and_window():

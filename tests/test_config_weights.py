@@ -59,9 +59,9 @@ def test_registry():
 
 def test_model_spec_has_no_size_in_code():
     spec = config_from_dict(plain.TINY_B).model_spec()
-    assert [l.mixer.params["window"] for l in spec.layers] == [None, 8, 8]
-    assert spec.layers[0].mixer.params["scale"] == 32 ** -0.5
-    assert spec.layers[2].mixer.prefix == "model.layers.2.self_attn."
+    assert [l.parts["mixer"].params["window"] for l in spec.layers] == [None, 8, 8]
+    assert spec.layers[0].parts["mixer"].params["scale"] == 32 ** -0.5
+    assert spec.layers[2].parts["mixer"].prefix == "model.layers.2.self_attn."
     assert [c.layer for c in spec.order] == [0, 1, 2]
     names = Model.declare(spec)
     assert set(names) == set(plain.tensor_shapes(plain.TINY_B))

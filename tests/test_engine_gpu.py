@@ -79,8 +79,8 @@ def test_mixed_with_page_reuse(setup, ops):
     runner = build_runner(folder, ops, dtype, block_size=block, num_blocks=pages, num_slots=4)
     # poison the cache: stale contents must never be read
     for group in runner.cache.groups:
-        group.k.fill_(float("nan"))
-        group.v.fill_(float("nan"))
+        for slab in group.tensors.values():
+            slab.fill_(float("nan"))
     reqs = {f"r{i}": random_ids(cfg, n, 10 + i) for i, n in enumerate(lengths)}
     got = {r: [] for r in reqs}
     at = {r: 0 for r in reqs}

@@ -138,7 +138,7 @@ def test_a_corrupted_cache_fails_the_comparison(tmp_path, name, block, dtype):
         def damage(runner):
             page = runner.cache.request("a").tables[group][position // block]
             assert page >= 0
-            runner.cache.groups[group].k[0, page, :, position % block, :] = 0
+            runner.cache.groups[group].tensors["k"][0, page, :, position % block, :] = 0
         return damage
 
     def exchange_last_two(group):

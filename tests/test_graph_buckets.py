@@ -2,7 +2,8 @@
 
 import pytest
 
-from distie_amd.engine.graphs import bucket_for, context_classes, decode_buckets
+from distie_amd.engine.graphs import bucket_for, decode_buckets
+from distie_amd.parts.attention import context_classes
 
 
 def test_decode_buckets():

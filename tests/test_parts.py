@@ -15,7 +15,7 @@ from distie_amd.config import LayerCall, LayerSpec, ModelSpec, PartSpec, registe
 from distie_amd.engine.batch import BatchBuilder, StepEntry
 from distie_amd.engine.model import Model
 from distie_amd.engine.runner import ModelRunner
-from distie_amd.parts import (FixedState, Mixer, PagedKV, ParamSpec, ResidualStream, StepContext, build_part,
+from distie_amd.parts import (FeedForward, FixedState, Mixer, PagedKV, PagedTensors, ParamSpec, ResidualStream, StepContext, build_part,
                               register_part)
 from torch_ops import TorchOps
 
@@ -101,7 +101,7 @@ def test_attention_part(ops, heads, kv_heads, dim, window, bias):
     lengths = [9, 1, 14]
     cache, meta = context(ops, [part.cache_requirement()], lengths)
     x = rnd(sum(lengths), hidden, seed=5)
-    got = dense(ops, part.forward(ops, x.to(ops.device), StepContext(meta, torch.float32), cache.layer(0), True)).cpu()
+    got = dense(ops, part.forward(ops, x.to(ops.device), StepContext(meta, torch.float32), cache.layer(0)["mixer"], True)).cpu()
     cfg = {"num_attention_heads": heads, "num_key_value_heads": kv_heads, "head_dim": dim, "hidden_size": hidden,
            "rope_theta": 1e4}
     named = {"a." + k: v.double() for k, v in w.items()}
@@ -126,24 +126,24 @@ def test_prenorm_block(ops):
 
     register_part("mixer", "test_twice", Twice)
 
-    class Half:
-        spec = PartSpec("half")
-
-        def param_specs(self):
-            return {}
-
+    class Half(FeedForward):
         def forward(self, ops, x, ctx):
             calls.append("ffn")
             return x * 0.5
 
-    norm = lambda: build_part("norm", PartSpec("rmsnorm", "", {"size": 8, "eps": 1e-6}))
-    n1, n2 = norm(), norm()
-    for n in (n1, n2):
+    register_part("feed_forward", "test_half", Half)
+    norm = PartSpec("rmsnorm", "", {"size": 8, "eps": 1e-6})
+    block = build_part("block", PartSpec("prenorm_residual"), {
+        "mixer": PartSpec("test_twice"), "feed_forward": PartSpec("test_half"), "mixer_norm": norm, "feed_forward_norm": norm})
+    assert [type(p).__name__ for p in block.parts()] == ["RMSNorm", "Twice", "RMSNorm", "Half", "PreNormResidual"]
+    for n in (block.mixer_norm, block.feed_forward_norm):
         n.load({"weight": torch.ones(8, device=ops.device)})
-    block = build_part("block", PartSpec("prenorm_residual"), build_part("mixer", PartSpec("test_twice")), Half(), n1, n2)
+    with pytest.raises(ValueError, match="missing \\['feed_forward_norm'\\], not known to it \\['third_norm'\\]"):
+        build_part("block", PartSpec("prenorm_residual"), {
+            "mixer": PartSpec("test_twice"), "feed_forward": PartSpec("test_half"), "mixer_norm": norm, "third_norm": norm})
     x = rnd(3, 8, seed=1)
     stream = ResidualStream(x.clone().to(ops.device))
-    block.forward(ops, stream, StepContext(None, torch.float32), None, True)
+    block.forward(ops, stream, StepContext(None, torch.float32), {"mixer": None}, True)
     rms = lambda t: plain.rms_norm(t, torch.ones(8), 1e-6)
     h1 = x + 2 * rms(x)
     assert calls == ["mixer", "ffn"]
@@ -162,7 +162,7 @@ class DecayMixer(Mixer):
         self.weight = None
 
     def cache_requirement(self):
-        return FixedState((self.size,))
+        return FixedState.of((self.size,))
 
     def param_specs(self):
         return {"mix.weight": ParamSpec((self.size, self.size))}
@@ -177,12 +177,12 @@ class DecayMixer(Mixer):
         slots = meta.state_slots.tolist()
         cu = meta.cu_q.tolist()
         for b in range(meta.num_requests):          # tokens of a request in order; the state carries over
-            s = cache.state[slots[b]]
+            s = cache["state"][slots[b]]
             for t in range(cu[b], cu[b + 1]):
                 s = self.decay * s + u[t]
                 out[t] = s
             if writes_cache:
-                cache.state[slots[b]] = s
+                cache["state"][slots[b]] = s
         return out.to(x.dtype)
 
 
@@ -209,10 +209,13 @@ class ToyConfig:
         layers = []
         for l, mixer in enumerate([attention("l0.attn."), PartSpec("test_decay", "l1.", {"hidden_size": self.hidden, "decay": self.decay}),
                                    attention("l2.attn.")]):
-            layers.append(LayerSpec(PartSpec("prenorm_residual"), mixer, ffn(f"l{l}.ffn."), norm(f"l{l}.n1."), norm(f"l{l}.n2.")))
+            layers.append(LayerSpec(PartSpec("prenorm_residual"), {
+                "mixer": mixer, "feed_forward": ffn(f"l{l}.ffn."), "mixer_norm": norm(f"l{l}.n1."),
+                "feed_forward_norm": norm(f"l{l}.n2.")}))
         order = (LayerCall(0), LayerCall(1), LayerCall(2), LayerCall(2, cache_of=0))
-        return ModelSpec("ToyForCausalLM", self.vocab, self.hidden, 256, PartSpec("token_embedding", "emb."), layers, order,
-                         norm("final."), PartSpec("lm_head", "head.", {"tied": True}))
+        sizes = {"vocab_size": self.vocab, "hidden_size": self.hidden}
+        return ModelSpec("ToyForCausalLM", self.vocab, self.hidden, 256, PartSpec("token_embedding", "emb.", sizes), layers,
+                         order, norm("final."), PartSpec("lm_head", "head.", dict(sizes, tied_to="emb.weight")))
 
 
 def toy_plain(weights, cfg, ids):
@@ -278,7 +281,8 @@ def test_toy_architecture_with_a_state_mixer_is_registered_built_and_stepped(ops
                for n, s in specs.items()}
     model.load_tensors(lambda name: weights[name].to(ops.device))
     needs = model.cache_requirements()
-    assert isinstance(needs[1], FixedState) and isinstance(needs[0], PagedKV)
+    assert isinstance(needs[1]["mixer"], FixedState) and needs[0] == {"mixer": PagedKV(1, 16)} and \
+        isinstance(needs[0]["mixer"], PagedTensors)
     cache = CacheManager(needs, 4, 32, 4, device=ops.device, dtype=torch.float32)
     runner = ModelRunner(model, cache, ops, torch.float32, 256)
     a = torch.randint(0, 70, (23,), generator=gen).tolist()
@@ -316,7 +320,7 @@ def test_toy_architecture_with_a_state_mixer_is_registered_built_and_stepped(ops
 # and in one layer a routed feed-forward (the best of three experts of different widths, scaled by its
 # router weight) beside a dense one in the other: chosen layer by layer by the configuration
 # ---------------------------------------------------------------------------------------------
-from distie_amd.parts import FeedForward, PositionEncoding   # noqa: E402
+from distie_amd.parts import PositionEncoding   # noqa: E402
 
 
 class LearnedPositions(PositionEncoding):
@@ -393,10 +397,12 @@ class RoutedToyConfig:
                                                         "head_dim": h // self.heads, "qkv_bias": False})     # no position inside
         feed_forward = [PartSpec("swiglu", "l0.ffn.", {"hidden_size": h, "intermediate_size": 3 * h}),
                         PartSpec("test_best_of_experts", "l1.moe.", {"hidden_size": h, "expert_sizes": self.expert_sizes})]
-        layers = [LayerSpec(PartSpec("prenorm_residual"), attention(f"l{l}.attn."), feed_forward[l], norm(f"l{l}.n1."),
-                            norm(f"l{l}.n2.")) for l in range(2)]
-        return ModelSpec("RoutedToyForCausalLM", self.vocab, h, self.max_positions, PartSpec("token_embedding", "emb."),
-                         layers, (LayerCall(0), LayerCall(1)), norm("final."), PartSpec("lm_head", "head.", {"tied": False}),
+        layers = [LayerSpec(PartSpec("prenorm_residual"), {
+            "mixer": attention(f"l{l}.attn."), "feed_forward": feed_forward[l], "mixer_norm": norm(f"l{l}.n1."),
+            "feed_forward_norm": norm(f"l{l}.n2.")}) for l in range(2)]
+        sizes = {"vocab_size": self.vocab, "hidden_size": h}
+        return ModelSpec("RoutedToyForCausalLM", self.vocab, h, self.max_positions, PartSpec("token_embedding", "emb.", sizes),
+                         layers, (LayerCall(0), LayerCall(1)), norm("final."), PartSpec("lm_head", "head.", sizes),
                          position=PartSpec("test_learned_positions", "pos.", {"max_positions": self.max_positions,
                                                                               "hidden_size": h}))
 
@@ -499,11 +505,13 @@ class CentredNorm(Norm):
 
 
 class PostNormResidual(Block):
+    CHILDREN = {"mixer": "mixer", "mixer_norm": "norm", "feed_forward": "feed_forward", "feed_forward_norm": "norm"}
+
     def forward(self, ops, stream, ctx, cache, writes_cache):
         if stream.pending is not None:                   # what the layer before left to be added
             stream.hidden += dense(ops, stream.pending).float()
             stream.pending = None
-        y = self.mixer.forward(ops, stream.hidden.to(ctx.act_dtype), ctx, cache, writes_cache)
+        y = self.mixer.forward(ops, stream.hidden.to(ctx.act_dtype), ctx, cache["mixer"], writes_cache)
         stream.hidden = self.mixer_norm.apply(ops, stream.hidden + dense(ops, y).float(), torch.float32)
         y = self.feed_forward.forward(ops, stream.hidden.to(ctx.act_dtype), ctx)
         stream.hidden = self.feed_forward_norm.apply(ops, stream.hidden + dense(ops, y).float(), torch.float32)
@@ -525,11 +533,15 @@ class PostNormToyConfig:
             "hidden_size": h, "num_heads": self.heads, "num_kv_heads": 1, "head_dim": d, "qkv_bias": False,
             "position": PartSpec("rope", "", {"dim": d, "theta": 300.0})})
         ffn = lambda p: PartSpec("swiglu", p, {"hidden_size": h, "intermediate_size": 2 * h + 8})
-        layers = [LayerSpec(PartSpec("test_postnorm_residual"), attention("l0.attn."), ffn("l0.ffn."), centred("l0.n1."),
-                            centred("l0.n2.")),
-                  LayerSpec(PartSpec("prenorm_residual"), attention("l1.attn."), ffn("l1.ffn."), rms("l1.n1."), rms("l1.n2."))]
-        return ModelSpec("PostNormToyForCausalLM", self.vocab, h, 128, PartSpec("token_embedding", "emb."), layers,
-                         (LayerCall(0), LayerCall(1)), centred("final."), PartSpec("lm_head", "head.", {"tied": False}))
+        named = lambda mixer, feed_forward, n1, n2: {"mixer": mixer, "feed_forward": feed_forward, "mixer_norm": n1,
+                                                    "feed_forward_norm": n2}
+        layers = [LayerSpec(PartSpec("test_postnorm_residual"),
+                            named(attention("l0.attn."), ffn("l0.ffn."), centred("l0.n1."), centred("l0.n2."))),
+                  LayerSpec(PartSpec("prenorm_residual"),
+                            named(attention("l1.attn."), ffn("l1.ffn."), rms("l1.n1."), rms("l1.n2.")))]
+        sizes = {"vocab_size": self.vocab, "hidden_size": h}
+        return ModelSpec("PostNormToyForCausalLM", self.vocab, h, 128, PartSpec("token_embedding", "emb.", sizes), layers,
+                         (LayerCall(0), LayerCall(1)), centred("final."), PartSpec("lm_head", "head.", sizes))
 
 
 def postnorm_toy_plain(weights, cfg, ids, norm_first=False):
@@ -600,3 +612,219 @@ def test_toy_architecture_with_a_norm_and_an_arrangement_of_its_own(ops):
     runner.finish("a")
     runner.finish("b")
     cache.check()
+
+
+# ---------------------------------------------------------------------------------------------
+# a fourth toy architecture: embeddings scaled by a constant and a head with a bias and capped logits;
+# layer 0 arranged as a sandwich (a norm before and after each sub-layer: four norms) around a mixer that
+# keeps one latent vector per token, and the token's position beside it as an integer, instead of keys and
+# values; layer 1 is the package's pre-norm attention layer, so two kinds of pages live side by side. The
+# latent mixer reads numbers back to the host and therefore says that it cannot be captured.
+# ---------------------------------------------------------------------------------------------
+from distie_amd.parts import PAGE, Embedding, Head, TensorDecl   # noqa: E402
+
+
+class ScaledEmbedding(Embedding):
+    def __init__(self, spec):
+        super().__init__(spec)
+        self.shape = (int(spec.params["vocab_size"]), int(spec.params["hidden_size"]))
+        self.scale = float(spec.params["scale"])
+        self.weight = None
+
+    def param_specs(self):
+        return {"weight": ParamSpec(self.shape)}
+
+    def load(self, tensors):
+        self.weight = tensors["weight"]
+
+    def forward(self, ops, ids, meta):
+        return ops.embed(ids, self.weight) * self.scale
+
+
+class CappedBiasedHead(Head):
+    def __init__(self, spec):
+        super().__init__(spec)
+        self.shape = (int(spec.params["vocab_size"]), int(spec.params["hidden_size"]))
+        self.cap = float(spec.params["cap"])
+        self.weight = self.bias = None
+
+    def param_specs(self):
+        return {"weight": ParamSpec(self.shape), "bias": ParamSpec(self.shape[:1])}
+
+    def load(self, tensors):
+        self.weight, self.bias = tensors["weight"], tensors["bias"].float()
+
+    def forward(self, ops, normed):
+        return self.cap * torch.tanh((ops.linear_f32out(normed, self.weight) + self.bias) / self.cap)
+
+
+class SandwichBlock(Block):
+    CHILDREN = {"before_mixer": "norm", "mixer": "mixer", "after_mixer": "norm",
+                "before_feed_forward": "norm", "feed_forward": "feed_forward", "after_feed_forward": "norm"}
+
+    def forward(self, ops, stream, ctx, cache, writes_cache):
+        y = self.mixer.forward(ops, self.before_mixer.of_stream(ops, stream, ctx.act_dtype), ctx, cache["mixer"], writes_cache)
+        stream.hidden += self.after_mixer.apply(ops, dense(ops, y).float(), torch.float32)
+        y = self.feed_forward.forward(ops, self.before_feed_forward.apply(ops, stream.hidden, ctx.act_dtype), ctx)
+        stream.hidden += self.after_feed_forward.apply(ops, dense(ops, y).float(), torch.float32)
+
+
+class LatentMixer(Mixer):
+    """c_t = x_t D is all that is kept of token t; y_t = softmax_j<=t(q_t . c_j / sqrt(R) - slope (t - j)) c_j U."""
+
+    capturable = False
+
+    def __init__(self, spec):
+        super().__init__(spec)
+        self.hidden, self.rank, self.slope = int(spec.params["hidden_size"]), int(spec.params["rank"]), float(spec.params["slope"])
+        self.down = self.query = self.up = None
+
+    def cache_requirement(self):
+        return PagedTensors((TensorDecl("latent", (PAGE, self.rank), torch.float32),
+                             TensorDecl("stamp", (PAGE,), torch.int32)))
+
+    def param_specs(self):
+        return {"down.weight": ParamSpec((self.rank, self.hidden)), "query.weight": ParamSpec((self.rank, self.hidden)),
+                "up.weight": ParamSpec((self.hidden, self.rank))}
+
+    def load(self, tensors):
+        self.down, self.query, self.up = (tensors[f"{n}.weight"].float() for n in ("down", "query", "up"))
+
+    def forward(self, ops, x, ctx, cache, writes_cache):
+        meta = ctx.meta
+        latent, stamp = cache["latent"], cache["stamp"]
+        assert latent.dtype == torch.float32 and stamp.dtype == torch.int32
+        P = latent.shape[1]
+        c = x.float() @ self.down.T
+        q = x.float() @ self.query.T
+        slots = meta.groups[cache.group].slots.long()
+        if writes_cache:
+            latent[slots // P, slots % P] = c
+            stamp[slots // P, slots % P] = meta.positions
+        table = meta.groups[cache.group].block_table.long()
+        out = torch.empty(x.shape[0], self.hidden, dtype=torch.float32, device=x.device)
+        cu, positions = meta.cu_q.tolist(), meta.positions.tolist()          # the host waits here: not capturable
+        for b in range(meta.num_requests):
+            for t in range(cu[b], cu[b + 1]):
+                keys = torch.arange(positions[t] + 1, device=x.device)
+                pages = table[b, keys // P]
+                assert bool((pages >= 0).all()) and torch.equal(stamp[pages, keys % P].long(), keys), "a wrong page was read"
+                kept = latent[pages, keys % P]
+                scores = kept @ q[t] / self.rank ** 0.5 - self.slope * (positions[t] - keys).float()
+                out[t] = (torch.softmax(scores, 0) @ kept) @ self.up.T
+        return out.to(x.dtype)
+
+
+class SandwichToyConfig:
+    def __init__(self, data):
+        self.hidden, self.vocab, self.rank, self.cap, self.slope = (data[k] for k in ("hidden", "vocab", "rank", "cap", "slope"))
+
+    @classmethod
+    def from_dict(cls, data):
+        return cls(data)
+
+    def model_spec(self):
+        h = self.hidden
+        norm = lambda p: PartSpec("rmsnorm", p, {"size": h, "eps": 1e-5})
+        ffn = lambda p: PartSpec("swiglu", p, {"hidden_size": h, "intermediate_size": 3 * h})
+        sandwich = LayerSpec(PartSpec("test_sandwich"), {
+            "before_mixer": norm("l0.n1."), "after_mixer": norm("l0.n2."), "before_feed_forward": norm("l0.n3."),
+            "after_feed_forward": norm("l0.n4."), "feed_forward": ffn("l0.ffn."),
+            "mixer": PartSpec("test_latent", "l0.mix.", {"hidden_size": h, "rank": self.rank, "slope": self.slope})})
+        usual = LayerSpec(PartSpec("prenorm_residual"), {
+            "mixer_norm": norm("l1.n1."), "feed_forward_norm": norm("l1.n2."), "feed_forward": ffn("l1.ffn."),
+            "mixer": PartSpec("attention", "l1.attn.", {"hidden_size": h, "num_heads": 2, "num_kv_heads": 2, "head_dim": h // 2,
+                                                        "qkv_bias": False,
+                                                        "position": PartSpec("rope", "", {"dim": h // 2, "theta": 50.0})})})
+        sizes = {"vocab_size": self.vocab, "hidden_size": h}
+        return ModelSpec("SandwichToyForCausalLM", self.vocab, h, 128,
+                         PartSpec("test_scaled_embedding", "emb.", dict(sizes, scale=h ** 0.5)), (sandwich, usual),
+                         (LayerCall(0), LayerCall(1)), norm("final."),
+                         PartSpec("test_capped_head", "head.", dict(sizes, cap=self.cap)))
+
+
+def sandwich_toy_plain(weights, cfg, ids, scaled=True):
+    """float64, whole sequence, no cache. `scaled=False` leaves the embeddings unscaled (the mistake that the
+    test must tell from the right model)."""
+    w = {k: v.double() for k, v in weights.items()}
+    n, h = len(ids), cfg.hidden
+    rms = lambda t, p: plain.rms_norm(t, w[p + "weight"], 1e-5)
+    ffn = lambda t, p: plain.swiglu(t, w[p + "gate_proj.weight"], w[p + "up_proj.weight"], w[p + "down_proj.weight"])
+    x = w["emb.weight"][torch.tensor(ids)] * (h ** 0.5 if scaled else 1.0)
+    t = rms(x, "l0.n1.")
+    c, q = t @ w["l0.mix.down.weight"].T, t @ w["l0.mix.query.weight"].T
+    place = torch.arange(n, dtype=torch.float64)
+    scores = q @ c.T / cfg.rank ** 0.5 - cfg.slope * (place[:, None] - place[None, :])
+    scores = scores.masked_fill(place[None, :] > place[:, None], float("-inf"))
+    x = x + rms((torch.softmax(scores, -1) @ c) @ w["l0.mix.up.weight"].T, "l0.n2.")
+    x = x + rms(ffn(rms(x, "l0.n3."), "l0.ffn."), "l0.n4.")
+    named = dict(w)
+    for name in "qkv":
+        named[f"l1.attn.{name}_proj.bias"] = torch.zeros(h, dtype=torch.float64)
+    att_cfg = {"num_attention_heads": 2, "num_key_value_heads": 2, "head_dim": h // 2, "rope_theta": 50.0}
+    x = x + plain.self_attention(rms(x, "l1.n1."), named, "l1.attn.", torch.arange(n), att_cfg, None)
+    x = x + ffn(rms(x, "l1.n2."), "l1.ffn.")
+    return cfg.cap * torch.tanh((rms(x, "final.") @ w["head.weight"].T + w["head.bias"]) / cfg.cap)
+
+
+def test_toy_architecture_with_four_norms_a_latent_cache_and_ends_of_its_own(ops):
+    register_part("embedding", "test_scaled_embedding", ScaledEmbedding)
+    register_part("head", "test_capped_head", CappedBiasedHead)
+    register_part("block", "test_sandwich", SandwichBlock)
+    register_part("mixer", "test_latent", LatentMixer)
+    register_architecture("SandwichToyForCausalLM", SandwichToyConfig)
+    from distie_amd.config import config_from_dict
+
+    data = {"architectures": ["SandwichToyForCausalLM"], "hidden": 32, "vocab": 61, "rank": 12, "cap": 5.0, "slope": 0.3}
+    cfg = config_from_dict(data)
+    model = Model(cfg.model_spec())
+    specs = model.param_specs()
+    assert {"l0.n1.weight", "l0.n2.weight", "l0.n3.weight", "l0.n4.weight", "l0.mix.down.weight", "head.bias",
+            "emb.weight", "l1.attn.o_proj.weight"} <= set(specs)
+    assert not model.capturable and Model(config_from_dict(plain.TINY_A).model_spec()).capturable
+    gen = torch.Generator().manual_seed(31)
+    weights = {n: (torch.ones(s.shape) + 0.2 * torch.randn(s.shape, generator=gen) if s.init == "ones"
+                   else torch.randn(s.shape, generator=gen) * 0.2) for n, s in specs.items()}
+    model.load_tensors(lambda name: weights[name].to(ops.device))
+    needs = model.cache_requirements()
+    assert [t.name for t in needs[0]["mixer"].tensors] == ["latent", "stamp"] and needs[1] == {"mixer": PagedKV(2, 16)}
+    cache = CacheManager(needs, 4, 24, 4, device=ops.device, dtype=torch.float32)
+    assert len(cache.groups) == 2 and cache.groups[0].tensors["latent"].shape == (1, 25, 4, 12) and \
+        cache.groups[0].tensors["stamp"].dtype == torch.int32 and cache.groups[1].tensors["v"].shape == (1, 25, 2, 16, 4)
+    for group in cache.groups:                   # stale pages must not be read: poison what can be poisoned
+        for slab in group.tensors.values():
+            slab.fill_(float("nan") if slab.dtype.is_floating_point else -5)
+    runner = ModelRunner(model, cache, ops, torch.float32, 128)
+    a = torch.randint(0, 61, (23,), generator=gen).tolist()
+    b = torch.randint(0, 61, (9,), generator=gen).tolist()
+    want_a, want_b = sandwich_toy_plain(weights, cfg, a).float(), sandwich_toy_plain(weights, cfg, b).float()
+    assert (sandwich_toy_plain(weights, cfg, a, scaled=False).float() - want_a).abs().max() > 1e-2
+    assert want_a.abs().max() < 5.0 and want_a.abs().max() > 2.0          # the cap bends the logits
+    got = runner.step([StepEntry("a", a, list(range(23)))]).cpu()
+    assert (got - want_a).abs().max() < 1e-4
+    runner.finish("a")
+    rows = {"a": [], "b": []}
+    seqs = {"a": a, "b": b}
+    for step in [[("a", 0, 5)], [("a", 5, 7), ("b", 0, 3)], [("a", 7, 22), ("b", 3, 4)], [("b", 4, 9), ("a", 22, 23)]]:
+        logits = runner.step([StepEntry(r, seqs[r][lo:hi], list(range(hi - lo))) for r, lo, hi in step]).cpu()
+        at = 0
+        for r, lo, hi in step:
+            rows[r].append(logits[at:at + hi - lo])
+            at += hi - lo
+    assert (torch.cat(rows["a"]) - want_a).abs().max() < 1e-4
+    assert (torch.cat(rows["b"]) - want_b).abs().max() < 1e-4
+    runner.finish("a")
+    runner.finish("b")
+    cache.check()
+    assert cache.free_pages() == [24, 24]
+    # through the entry point: the registry finds the architecture, and a model with a part that cannot be
+    # captured runs its decode steps uncaptured, whatever the options ask for
+    from distie_amd import LLM, SamplingParams
+
+    llm = LLM(config=data, random_weights=True, seed=5, ops=ops, dtype="fp32", block_size=4, num_blocks=24, max_seqs=4,
+              use_graphs=True)
+    assert llm.runner.graphs is None
+    outs = llm.generate([a[:6], b[:3]], SamplingParams(max_new_tokens=5))
+    assert [len(o.token_ids) for o in outs] == [5, 5] and all(o.finish_reason == "length" for o in outs)
+    again = llm.generate([a[:6]], SamplingParams(max_new_tokens=5))
+    assert again[0].token_ids == outs[0].token_ids

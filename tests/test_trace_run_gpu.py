@@ -168,14 +168,14 @@ def test_captured_steps_per_class_of_context_length(tmp_path, monkeypatch):
     alone and three at a time, give the logits of the whole sequences."""
     from distie_amd import LLM
     from distie_amd.engine.batch import StepEntry
-    from distie_amd.engine.graphs import DecodeGraphs
+    from distie_amd.parts.attention import Attention
     from engine_util import check_logits
 
-    monkeypatch.setattr(DecodeGraphs, "FIRST_CONTEXT", 32)
+    monkeypatch.setattr(Attention, "FIRST_CONTEXT", 32)
     cfg = plain.TINY_C
     folder, weights = make_model_dir(tmp_path, cfg, seed=8, dtype=torch.bfloat16)
     llm = LLM(folder, dtype="bf16", block_size=16, num_blocks=40, max_seqs=4)
-    assert llm.runner.graphs.contexts[:5] == (32, 48, 64, 96, 128)
+    assert [llm.model.capture_context(n, 256) for n in (1, 33, 49, 97, 200)] == [32, 48, 64, 128, 256]
     seqs = {name: random_ids(cfg, n, 17 + n) for name, n in (("a", 150), ("b", 70), ("c", 101))}
     got = {name: [] for name in seqs}
     starts = {"a": 20, "b": 1, "c": 40}
