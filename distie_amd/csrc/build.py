@@ -34,10 +34,10 @@ HIP_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17",
              "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
 CXX_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-pthread"]
 
-OPS_SOURCES = ["elementwise.hip", "gemm.hip", "sampling.hip"]
+OPS_SOURCES = ["elementwise.hip", "gemm.hip", "decode_products.hip", "sampling.hip"]
 ATTN_SOURCES = ["attention.hip"]
 HEADERS = ["common.h"]
-OPS_HEADERS = ["no_alloc.h"]
+OPS_HEADERS = ["no_alloc.h", "packed.h"]
 
 
 class BuildError(RuntimeError):

@@ -16,6 +16,7 @@
 // 231-233, 301); bfloat16 products of many rows (prefill) are left to the library here as well.
 
 #include "common.h"
+#include "packed.h"
 #include <algorithm>
 
 // ---------------------------------------------------------------- generic
@@ -89,8 +90,6 @@ extern "C" int distie_gemm_generic(const void* x, int x_dtype, const void* w, in
 }
 
 // ---------------------------------------------------------------- skinny, bfloat16, matrix cores
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 #define SK_ROWS 16          // rows of W per wave
 #define SK_KSTEP 128        // k per wave iteration: four MFMAs of 32 k each
@@ -260,10 +259,6 @@ extern "C" int distie_gemm_skinny_bf16(const void* x, const void* w, const float
 //    [M, N] result and k and v into the paged cache.
 // In all of them lanes 0-31 of the accumulator hold rows 0-7 of the block and lanes 32-63 rows 8-15 for
 // the same tokens, so partners meet through one exchange between lane l and lane l ^ 32.
-#define PK_TILE 512         // elements of a tile
-#define PK_PLAIN 0
-#define PK_GATED 1
-#define PK_ROTARY 2
 
 __global__ __launch_bounds__(256) void pack_rows_kernel(const bf16_t* __restrict__ w, bf16_t* __restrict__ out,
                                                         const int32_t* __restrict__ row_map, int K, int64_t row_blocks,
@@ -350,20 +345,6 @@ __device__ __forceinline__ floatx4 packed_accumulate(const bf16_t* wp, const bf1
   return acc;
 }
 
-struct RotaryOut {
-  const float2* table;        // [M, D / 2] cosine and sine of each token's angles
-  const int32_t* slots;       // [M] place of each token in the cache
-  bf16_t* k_cache;            // [pages, kv_heads, block_size, D]
-  bf16_t* v_cache;            // [pages, kv_heads, D, block_size]
-  int heads, kv_heads, dim, block_size, write;
-};
-
-static __device__ __forceinline__ uint2 pack_bf16x4(const float v[4]) {
-  uint32_t h[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) h[i] = __builtin_bit_cast(uint16_t, static_cast<bf16_t>(v[i]));
-  return uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
-}
 
 // blockIdx.x: row block; blockIdx.y: slice of K (PLAIN only; slices side by side in y, bias on slice 0, as
 // gemm_skinny_kernel); blockIdx.z: a group of 16 rows of x (with more than 16 rows the weights are read once

@@ -69,7 +69,49 @@ class PartialSums:
         return self.data.shape[0]
 
 
+class PendingNorm:
+    """rmsnorm(residual) * weight, not computed yet: for steps of few rows the product that reads it computes
+    it itself, in front of its own work (`distie_decode_norm_product`); anything else sees the finished
+    tensor through `HipOps.dense`. Valid as long as the residual it was made from is unchanged."""
+
+    def __init__(self, residual: torch.Tensor, weight: torch.Tensor, eps: float, dtype: torch.dtype) -> None:
+        self.residual = residual
+        self.weight = weight
+        self.eps = float(eps)
+        self.dtype = dtype
+        self.shape = residual.shape
+        self.device = residual.device
+        self.version = getattr(residual, "_distie_version", 0)
+
+    def check(self) -> None:
+        if getattr(self.residual, "_distie_version", 0) != self.version:
+            raise KernelError("a normed value was used after the residual stream it was made from had changed")
+
+
+class PendingProduct:
+    """x W^T + bias for few rows of x, not computed yet: if the next thing that happens to it is the sum into
+    the residual stream, the product adds itself to the stream in place (`distie_decode_product_residual`) and
+    never exists as a tensor; anything else sees the finished tensor through `HipOps.dense`."""
+
+    def __init__(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> None:
+        self.x = x
+        self.weight = weight
+        self.bias = bias
+        self.dtype = x.dtype
+        self.shape = torch.Size((x.shape[0], weight.shape[0]))
+        self.device = x.device
+
+
 class HipOps(Ops):
+    # Steps of up to FUSED_MAX_ROWS rows can run their products with the norm in front and the residual sum behind
+    # folded in (six launches a layer instead of eight, no partial sums handed on). On the device that is no
+    # gain: a kernel's time here is a chain of trips to memory, and the folded-in norm or the sum across a
+    # workgroup's waves adds its trip to the product's own (measured at 8 rows, 1,536 wide: gate+up 18.7 us with
+    # the norm against 13.4 + 4.2 us apart; down 13.2 against 8.3 us in 14 slices, since 96 workgroups pull
+    # less than 1,344; q/k/v 9.0 against 5.5 + 4.2 us). Where the host bounds a step, two launches fewer a layer
+    # count: steps that are launched kernel by kernel take this path, captured steps do not.
+    FUSED_MAX_ROWS = 16
+    FUSED_IN_CAPTURED_STEPS = False
     # bfloat16 products by rows of x: up to SKINNY_MAX_ROWS the weights are streamed by one wave per block
     # of 16 weight rows, x straight from memory (above that, the library's tiles are faster);
     SKINNY_MAX_ROWS = 16
@@ -161,6 +203,10 @@ class HipOps(Ops):
         o.distie_gemm_packed_wide_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
         o.distie_gemm_packed_wide_slices.argtypes = [_I, _I]
         o.distie_gemm_packed_rotary_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
+        o.distie_decode_norm_fits.argtypes = [_I]
+        o.distie_decode_product_residual.argtypes = [_P, _P, _P, _P, _I, _I, _I, _P]
+        o.distie_decode_norm_product.argtypes = [_P, _P, _F, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P,
+                                                 _I, _I, _I, _I, _I, _P]
         o.distie_argmax.argtypes = [_P, _P, _I, _I, _P, _P, _P]
         o.distie_argmax_parts.argtypes = [_I, _I]
         o.distie_sample.argtypes = [_P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P]
@@ -237,10 +283,24 @@ class HipOps(Ops):
                                       ids.shape[0], table.shape[1], table.shape[0], self._stream()), "embed")
         return out
 
+    def _norm_later(self, residual, weight, out_dtype) -> bool:
+        """The norm of these rows can be left to the product that reads it."""
+        return (self.packed_weights and self._fused(residual.shape[0]) and out_dtype == torch.bfloat16 and
+                residual.dtype == torch.float32 and residual.dim() == 2 and
+                weight.dtype in _CODES and bool(self._ops.distie_decode_norm_fits(residual.shape[1])))
+
+    def _fused(self, rows: int) -> bool:
+        return rows <= self.FUSED_MAX_ROWS and (self.FUSED_IN_CAPTURED_STEPS or not self.captured)
+
     def rmsnorm(self, x, weight, eps, out_dtype):
         self._own(x, weight)
         if x.dtype != torch.float32:
             raise KernelError("rmsnorm reads the float32 residual stream")
+        if self._norm_later(x, weight, out_dtype):
+            return PendingNorm(x, weight, eps, out_dtype)
+        return self._rmsnorm_now(x, weight, eps, out_dtype)
+
+    def _rmsnorm_now(self, x, weight, eps, out_dtype):
         out = torch.empty(x.shape, dtype=out_dtype, device=self.device)
         _check(self._ops.distie_rmsnorm(x.data_ptr(), None, _F32, 1, weight.data_ptr(), _code(weight),
                                         out.data_ptr(), _CODES[out_dtype], x.shape[0], x.shape[1], eps,
@@ -248,7 +308,15 @@ class HipOps(Ops):
         return out
 
     def add_rmsnorm(self, residual, delta, weight, eps, out_dtype):
+        if isinstance(delta, PendingProduct):
+            self._own(residual, weight)
+            if residual.dtype != torch.float32 or residual.shape != delta.shape:
+                raise KernelError("add_rmsnorm: residual must be float32 and shaped like delta")
+            # the product adds itself to the stream; what is left is the norm of the stream
+            self._product_into_residual(delta, residual)
+            return self.rmsnorm(residual, weight, eps, out_dtype)
         slices = 1
+        delta = self.dense(delta) if isinstance(delta, PendingNorm) else delta
         if isinstance(delta, PartialSums):
             slices, delta = delta.slices, delta.data
         self._own(residual, delta, weight)
@@ -258,10 +326,29 @@ class HipOps(Ops):
         _check(self._ops.distie_rmsnorm(residual.data_ptr(), delta.data_ptr(), _code(delta), slices,
                                         weight.data_ptr(), _code(weight), out.data_ptr(), _CODES[out_dtype],
                                         residual.shape[0], residual.shape[1], eps, self._stream()), "add_rmsnorm")
+        residual._distie_version = getattr(residual, "_distie_version", 0) + 1
         return out
 
+    def _product_into_residual(self, product: PendingProduct, residual: torch.Tensor) -> None:
+        x, weight, bias = product.x, product.weight, product.bias
+        packed = getattr(weight, "_distie_packed")
+        M, K = x.shape
+        N = weight.shape[0]
+        if packed.numel() != self._packed_elements(N, K, False):
+            raise KernelError("linear: the packed copy does not belong to this weight")
+        _check(self._ops.distie_decode_product_residual(
+            x.data_ptr(), packed.data_ptr(), bias.data_ptr() if bias is not None else None, residual.data_ptr(),
+            M, N, K, self._stream()), "decode_product_residual")
+        residual._distie_version = getattr(residual, "_distie_version", 0) + 1
+
     def dense(self, x):
-        """The finished sum of a `PartialSums`; any other tensor as it is."""
+        """The finished tensor of a value that an operation here returned in a form of its own (partial sums,
+        a norm or a product that was left for later); any other tensor as it is."""
+        if isinstance(x, PendingNorm):
+            x.check()
+            return self._rmsnorm_now(x.residual, x.weight, x.eps, x.dtype)
+        if isinstance(x, PendingProduct):
+            return self._linear(x.x, x.weight, x.bias, x.dtype, lazy=False)
         if not isinstance(x, PartialSums):
             return x
         out = torch.empty(tuple(x.shape), dtype=x.dtype, device=self.device)
@@ -324,8 +411,36 @@ class HipOps(Ops):
         # the copy lives and dies with the weight
         setattr(weight, name, (packed, tuple(rotary)) if name == "_distie_rotary" else packed)
 
+    def _norm_product(self, x: PendingNorm, packed, bias, out, mode, N, rotary=None):
+        """`out` = the product of rmsnorm(x.residual) with the weight whose packed copy is `packed`, the norm
+        computed inside the product."""
+        x.check()
+        M, K = x.shape
+        table = slots = k_cache = v_cache = None
+        heads = kv_heads = dim = block_size = write = 0
+        if rotary is not None:
+            table, slots, k_cache, v_cache, heads, kv_heads, dim, block_size, write = rotary
+        ptr = lambda t: t.data_ptr() if t is not None else None
+        norm_weight = x.weight
+        if norm_weight.dtype != torch.float32:
+            # the kernel takes the norm's weights in float32 (a bfloat16 value is one exactly); kept on the tensor
+            norm_weight = getattr(x.weight, "_distie_f32", None)
+            if norm_weight is None:
+                norm_weight = x.weight._distie_f32 = x.weight.float()
+        _check(self._ops.distie_decode_norm_product(
+            x.residual.data_ptr(), norm_weight.data_ptr(), x.eps, packed.data_ptr(), ptr(bias),
+            out.data_ptr(), mode, M, N, K, ptr(table), ptr(slots), ptr(k_cache), ptr(v_cache), heads, kv_heads, dim,
+            block_size, write, self._stream()), "decode_norm_product")
+        return out
+
     def linear_silu_mul(self, x, gate_up_weight):
         packed = getattr(gate_up_weight, "_distie_gated", None)
+        if isinstance(x, PendingNorm) and packed is not None and gate_up_weight.shape[1] == x.shape[1]:
+            N, K = gate_up_weight.shape
+            if packed.numel() != self._packed_elements(N, K, True):
+                raise KernelError("linear_silu_mul: the packed copy does not belong to this weight")
+            out = torch.empty((x.shape[0], N // 2), dtype=torch.bfloat16, device=self.device)
+            return self._norm_product(x, packed, None, out, 1, N)
         x = self.dense(x)
         if packed is None or x.dtype != torch.bfloat16 or x.shape[0] > self._packed_rows():
             return self.silu_mul(self.linear(x, gate_up_weight))
@@ -349,6 +464,27 @@ class HipOps(Ops):
     def linear_rope_kv_write(self, x, weight, bias, meta, group, k_cache, v_cache, inv_freq, num_heads, num_kv_heads,
                              head_dim, write):
         held = getattr(weight, "_distie_rotary", None)
+        if isinstance(x, PendingNorm) and held is not None and held[1] == (num_heads, num_kv_heads, head_dim) and \
+                inv_freq is not None and 2 * inv_freq.shape[0] == head_dim and k_cache.dtype == torch.bfloat16 and \
+                weight.shape[1] == x.shape[1]:
+            packed = held[0]
+            slots = meta.groups[group].slots
+            self._own(bias, k_cache, v_cache, inv_freq, slots)
+            M, K = x.shape
+            N = weight.shape[0]
+            if N != (num_heads + 2 * num_kv_heads) * head_dim:
+                raise KernelError(f"linear: weight is {list(weight.shape)} for {num_heads} + 2 x {num_kv_heads} heads")
+            if bias is not None and (bias.dtype != torch.float32 or bias.shape[0] != N):
+                raise KernelError("linear: bias must be float32 [N]")
+            if packed.numel() != self._packed_elements(N, K, False):
+                raise KernelError("linear_rope_kv_write: the packed copy does not belong to this weight")
+            self._check_cache(k_cache, v_cache, num_kv_heads, meta.block_size, head_dim)
+            if M != meta.num_tokens or slots.shape[0] != M:
+                raise KernelError("linear_rope_kv_write: rows do not match the batch")
+            table = self._rope_table(meta, inv_freq)
+            out = torch.empty((M, N), dtype=torch.bfloat16, device=self.device)
+            return self._norm_product(x, packed, bias, out, 2, N, rotary=(
+                table, slots, k_cache, v_cache, num_heads, num_kv_heads, head_dim, meta.block_size, 1 if write else 0))
         x = self.dense(x)
         fused = held is not None and held[1] == (num_heads, num_kv_heads, head_dim) and \
             x.dtype == torch.bfloat16 and x.shape[0] <= self._packed_rows() and \
@@ -401,7 +537,16 @@ class HipOps(Ops):
             meta.scratch[key] = table
         return table
 
-    def _linear(self, x, weight, bias, out_dtype, partial_ok=False):
+    def _linear(self, x, weight, bias, out_dtype, partial_ok=False, lazy=False):
+        packed = getattr(weight, "_distie_packed", None)
+        if isinstance(x, PendingNorm) and out_dtype == torch.float32 and bias is None and packed is not None and \
+                weight.shape[1] == x.shape[1] and weight.dtype == torch.bfloat16:
+            # the head behind the final norm
+            N, K = weight.shape
+            if packed.numel() != self._packed_elements(N, K, False):
+                raise KernelError("linear: the packed copy does not belong to this weight")
+            out = torch.empty((x.shape[0], N), dtype=torch.float32, device=self.device)
+            return self._norm_product(x, packed, None, out, 0, N)
         x = self.dense(x)
         self._own(x, weight, bias)
         M, K = x.shape
@@ -411,7 +556,9 @@ class HipOps(Ops):
         if bias is not None and (bias.dtype != torch.float32 or bias.shape[0] != N):
             raise KernelError("linear: bias must be float32 [N]")
         both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-        packed = getattr(weight, "_distie_packed", None) if both_bf16 else None
+        packed = packed if both_bf16 else None
+        if lazy and packed is not None and self._fused(M) and K % 8 == 0 and out_dtype == torch.bfloat16:
+            return PendingProduct(x, weight, bias)
         if packed is not None and self.SKINNY_MAX_ROWS < M <= self._packed_rows() and K % 8 == 0 and \
                 N * K > self.ROW_GROUPS_MAX_ELEMENTS:
             if packed.numel() != self._packed_elements(N, K, False):
@@ -469,13 +616,15 @@ class HipOps(Ops):
 
     def linear(self, x, weight, bias=None):
         """May return `PartialSums` (see there)."""
-        return self._linear(x, weight, bias, x.dtype, partial_ok=True)
+        return self._linear(x, weight, bias, x.dtype, partial_ok=True, lazy=True)
 
     def linear_f32out(self, x, weight):
         return self._linear(x, weight, None, torch.float32)
 
     def rope_kv_write(self, qkv, meta: BatchMeta, group, k_cache, v_cache, inv_freq, num_heads, num_kv_heads,
                       head_dim, write):
+        if isinstance(qkv, (PendingNorm, PendingProduct)):
+            qkv = self.dense(qkv)
         slices, source = 1, qkv
         if isinstance(qkv, PartialSums):
             slices, source = qkv.slices, qkv.data
@@ -587,6 +736,8 @@ class HipOps(Ops):
         return plan
 
     def silu_mul(self, gate_up):
+        if isinstance(gate_up, (PendingNorm, PendingProduct)):
+            gate_up = self.dense(gate_up)
         slices, source, dtype = 1, gate_up, gate_up.dtype
         if isinstance(gate_up, PartialSums):
             slices, source = gate_up.slices, gate_up.data

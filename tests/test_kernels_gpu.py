@@ -50,12 +50,12 @@ def test_rmsnorm_and_fused_add(ops, dtype, rows, width):
     w = rand(width, dtype=dtype, seed=2)
     eps = 1e-5
     want = x.double() * torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True) + eps) * w.double()
-    got = ops.rmsnorm(x, w, eps, dtype)
+    got = ops.dense(ops.rmsnorm(x, w, eps, dtype))          # (few rows in bfloat16 are normed when they are read)
     assert got.dtype == dtype
     close(got, want, dtype, scale=want.abs().max().item())
     delta = rand(rows, width, dtype=dtype, seed=3)
     res = x.clone()
-    got = ops.add_rmsnorm(res, delta, w, eps, dtype)
+    got = ops.dense(ops.add_rmsnorm(res, delta, w, eps, dtype))
     s = x.double() + delta.double()
     assert torch.allclose(res.double(), s, atol=1e-6)
     want = s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + eps) * w.double()
@@ -116,7 +116,7 @@ def test_gemm_skinny_bf16(ops, M, N, K):
 def test_gemm_packed_bf16(ops, M, N, K):
     """The same products through the weight's packed copy (what `prepare_linear` leaves): rows and
     k that do not fill a tile, one slice and several, with and without a bias."""
-    from distie_amd.kernels.hip_ops import PartialSums
+    from distie_amd.kernels.hip_ops import PartialSums, PendingProduct
 
     x, w, b = rand(M, K, dtype=torch.bfloat16, seed=1), rand(N, K, dtype=torch.bfloat16, seed=2), rand(N, seed=3)
     natural = ops.dense(ops.linear(x, w, b)).float()
@@ -133,7 +133,11 @@ def test_gemm_packed_bf16(ops, M, N, K):
         for limit, two_pass in routes:
             ops.ROW_GROUPS_MAX_ELEMENTS, ops.TWO_PASS_MAX_ELEMENTS = limit, two_pass
             part = ops.linear(x, w, b)
-            if M <= 16 or limit > 0:
+            if M <= 16:
+                # few rows: the product waits for its reader (the residual sum takes it in; see the test of
+                # the decode products); any other reader sees it through `dense`, computed the usual way
+                assert isinstance(part, PendingProduct)
+            elif limit > 0:
                 assert isinstance(part, PartialSums) == (K >= 768)
             got = ops.dense(part)
             assert got.dtype == torch.bfloat16
@@ -244,6 +248,88 @@ def test_linear_rope_kv_write_fused(ops, M, heads, kv_heads, dim, K, P, with_bia
     k3, v3 = k2.clone(), v2.clone()
     unfused = ops.linear_rope_kv_write(x, w2, b, meta, 0, k3, v3, inv_freq, heads, kv_heads, dim, write)
     close(unfused, want, torch.bfloat16, scale=2 * scale)
+
+
+@pytest.mark.parametrize("M", [1, 5, 8, 9, 16])
+@pytest.mark.parametrize("C,I,heads,kv_heads,dim", [(1536, 4484, 12, 2, 128), (72, 13, 3, 1, 16), (3584, 300, 4, 4, 48),
+                                                    (4096, 88, 2, 1, 80), (264, 172, 5, 5, 32)])
+def test_decode_products_with_the_norm_in_front_and_the_residual_sum_behind(ops, M, C, I, heads, kv_heads, dim):
+    """Steps of few rows: a product that is added to the residual stream adds itself (nothing is handed on as
+    partial sums), the norm of the stream is left to the product that reads it, and that product computes it
+    in front of its own work: gate+up with the activation, q/k/v with bias, rotation and cache write, and the
+    head in float32. Each against the same operations one after the other."""
+    from distie_amd.kernels.hip_ops import KernelError, PendingNorm, PendingProduct
+
+    eps = 1e-5
+    # the product that feeds the stream: y [M, C] = a [M, I] W^T + b, added to the residual in place
+    a = rand(M, I * 8, dtype=torch.bfloat16, seed=1)
+    w_out = rand(C, I * 8, dtype=torch.bfloat16, seed=2, scale=1.0 / (I * 8) ** 0.5)
+    b_out = rand(C, seed=3)
+    ops.prepare_linear(w_out)
+    residual = rand(M, C, seed=4)
+    want_residual = residual.double() + a.double() @ w_out.double().T + b_out.double()
+    g = (1 + 0.2 * rand(C, seed=5)).to(torch.bfloat16)
+    delta = ops.linear(a, w_out, b_out)
+    assert isinstance(delta, PendingProduct) and tuple(delta.shape) == (M, C)
+    normed = ops.add_rmsnorm(residual, delta, g, eps, torch.bfloat16)
+    scale = want_residual.abs().max().item()
+    assert (residual.double() - want_residual).abs().max().item() <= 2e-5 * max(1.0, scale) * 8
+    assert isinstance(normed, PendingNorm) and tuple(normed.shape) == (M, C)
+    want_normed = want_residual * torch.rsqrt(want_residual.pow(2).mean(-1, keepdim=True) + eps) * g.double()
+    xn = ops.dense(normed)
+    assert xn.dtype == torch.bfloat16
+    close(xn, want_normed, torch.bfloat16, scale=want_normed.abs().max().item())
+    xn = xn.double()                       # what the products below see: the norm rounded to bfloat16
+    # gate + up with the activation
+    w_gu = rand(2 * I, C, dtype=torch.bfloat16, seed=6, scale=2.0 / C ** 0.5)
+    ops.prepare_linear(w_gu, gated=True)
+    gu = xn @ w_gu.double().T
+    want = gu[:, :I] / (1 + torch.exp(-gu[:, :I])) * gu[:, I:]
+    got = ops.linear_silu_mul(normed, w_gu)
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (M, I)
+    close(got, want, torch.bfloat16, scale=1.5 * want.abs().max().item())
+    # q/k/v with bias, rotation and cache write
+    P = 16
+    N = (heads + 2 * kv_heads) * dim
+    w_qkv = rand(N, C, dtype=torch.bfloat16, seed=7, scale=1.0 / C ** 0.5)
+    b_qkv = rand(N, seed=8)
+    ops.prepare_linear(w_qkv, rotary=(heads, kv_heads, dim))
+    pages = 2 * M + 2
+    gen = torch.Generator().manual_seed(M * 17 + dim)
+    slots = torch.randperm(pages * P, generator=gen)[:M].tolist()
+    positions = torch.randint(0, 5000, (M,), generator=gen).tolist()
+    meta = make_meta(positions, list(range(M)), list(range(M + 1)), [p + 1 for p in positions], [[0] * 8] * M, slots, P)
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, dim, 2, dtype=torch.float32) / dim))).cuda()
+    k1 = rand(pages, kv_heads, P, dim, dtype=torch.bfloat16, seed=9)
+    v1 = rand(pages, kv_heads, dim, P, dtype=torch.bfloat16, seed=10)
+    k2, v2 = k1.clone(), v1.clone()
+    dense = (xn @ w_qkv.double().T + b_qkv.double()).float()
+    want = TorchOps("cuda").rope_kv_write(dense.clone(), meta, 0, k2, v2, inv_freq, heads, kv_heads, dim, True)
+    got = ops.linear_rope_kv_write(normed, w_qkv, b_qkv, meta, 0, k1, v1, inv_freq, heads, kv_heads, dim, True)
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (M, N)
+    close(got, want, torch.bfloat16, scale=1.5 * want.abs().max().item())
+    close(k1, k2, torch.bfloat16, scale=1.5 * want.abs().max().item())
+    close(v1, v2, torch.bfloat16, scale=1.5 * want.abs().max().item())
+    at = torch.tensor(slots).cuda()
+    view = got.view(M, heads + 2 * kv_heads, dim)
+    assert torch.equal(k1[at // P, :, at % P], view[:, heads:heads + kv_heads])
+    assert torch.equal(v1[at // P, :, :, at % P], view[:, heads + kv_heads:])
+    # the head: float32 logits
+    V = 1001
+    w_head = rand(V, C, dtype=torch.bfloat16, seed=11, scale=1.0 / C ** 0.5)
+    ops.prepare_linear(w_head)
+    logits = ops.linear_f32out(normed, w_head)
+    assert logits.dtype == torch.float32 and tuple(logits.shape) == (M, V)
+    want = xn @ w_head.double().T
+    assert (logits.double() - want).abs().max().item() <= 2e-3 * want.abs().max().item()
+    # a norm that was left for later is of no use once its stream has moved on
+    ops.add_rmsnorm(residual, ops.linear(a, w_out, b_out), g, eps, torch.bfloat16)
+    with pytest.raises(KernelError, match="had changed"):
+        ops.linear_silu_mul(normed, w_gu)
+    # rows that the fused products do not take are normed at once
+    wide = rand(3, 4100, seed=12)
+    assert isinstance(ops.rmsnorm(wide, rand(4100, seed=13), eps, torch.bfloat16), torch.Tensor)
+    assert isinstance(ops.rmsnorm(rand(17, C, seed=14), g, eps, torch.bfloat16), torch.Tensor)
 
 
 def test_partial_sums_are_added_by_their_readers(ops):
