@@ -1,4 +1,5 @@
-// Attention over the paged cache for one head size (compile with -DDISTIE_HEAD_DIM=<multiple of 16>).
+// Attention over the paged cache for one head size (compile with -DDISTIE_HEAD_DIM=<even size up to 256>; the
+// matrix-core kernels exist for multiples of 16 only, the wave-per-token kernel for every even size).
 //
 // out[t, h] = softmax_j(q[t, h] . k[j, h / G] * scale) v[j, h / G] over the keys j that token t may see:
 // first(t) <= j <= position(t), first = 0, or position - window + 1 on a windowed layer. Keys and values
@@ -17,9 +18,10 @@
 #ifndef DISTIE_HEAD_DIM
 #error "compile with -DDISTIE_HEAD_DIM=<head size>"
 #endif
-#if DISTIE_HEAD_DIM % 16 != 0 || DISTIE_HEAD_DIM < 16 || DISTIE_HEAD_DIM > 256
-#error "head size must be a multiple of 16 between 16 and 256"
+#if DISTIE_HEAD_DIM % 2 != 0 || DISTIE_HEAD_DIM < 2 || DISTIE_HEAD_DIM > 256
+#error "head size must be even and at most 256"
 #endif
+#define DISTIE_MATRIX_CORE_ATTENTION (DISTIE_HEAD_DIM % 16 == 0)
 
 constexpr int D = DISTIE_HEAD_DIM;
 constexpr int DIMS_PER_LANE = (D + DISTIE_WAVE - 1) / DISTIE_WAVE;
@@ -32,8 +34,13 @@ __device__ __forceinline__ float dot_row(const float* q, const C* k);
 template <>
 __device__ __forceinline__ float dot_row<float>(const float* q, const float* k) {
   float s = 0.f;
+  if constexpr (D % 4 != 0) {                  // rows are not 16-byte aligned: element by element
 #pragma unroll
-  for (int d = 0; d < D; d += 4) {
+    for (int d = 0; d < D; ++d) s = fmaf(q[d], k[d], s);
+    return s;
+  }
+#pragma unroll
+  for (int d = 0; d + 4 <= D; d += 4) {
     const float4 v = *reinterpret_cast<const float4*>(k + d);
     s = fmaf(q[d], v.x, s);
     s = fmaf(q[d + 1], v.y, s);
@@ -46,8 +53,13 @@ __device__ __forceinline__ float dot_row<float>(const float* q, const float* k) 
 template <>
 __device__ __forceinline__ float dot_row<bf16_t>(const float* q, const bf16_t* k) {
   float s = 0.f;
+  if constexpr (D % 8 != 0) {
 #pragma unroll
-  for (int d = 0; d < D; d += 8) {
+    for (int d = 0; d < D; ++d) s = fmaf(q[d], to_float(k[d]), s);
+    return s;
+  }
+#pragma unroll
+  for (int d = 0; d + 8 <= D; d += 8) {
     const uint4 raw = *reinterpret_cast<const uint4*>(k + d);
     const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
@@ -59,70 +71,139 @@ __device__ __forceinline__ float dot_row<bf16_t>(const float* q, const bf16_t* k
   return s;
 }
 
-template <typename T, typename C>
-__global__ __launch_bounds__(DISTIE_WAVE) void attn_generic_kernel(
+// four consecutive values of a page's row of V^T as floats
+__device__ __forceinline__ void load4(const float* p, float v[4]) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+}
+__device__ __forceinline__ void load4(const bf16_t* p, float v[4]) {
+  const uint2 raw = *reinterpret_cast<const uint2*>(p);
+  v[0] = __uint_as_float(raw.x << 16); v[1] = __uint_as_float(raw.x & 0xffff0000u);
+  v[2] = __uint_as_float(raw.y << 16); v[3] = __uint_as_float(raw.y & 0xffff0000u);
+}
+
+// One workgroup of WAVES waves per (token, head). The keys are taken in chunks of 64 that begin at multiples of
+// 64; the chunks are dealt to the waves in turn (a token that decodes over thousands of keys then has eight
+// waves at work instead of one), every wave keeps its own running maximum, sum and output, and wave 0 puts them
+// together at the end, in wave order. In a chunk a lane owns one key for the scores; for the output it owns
+// the dimensions lane, lane + 64, ... and walks the chunk's keys: a page at a time with 16-byte loads of the
+// page's row of V^T when pages divide 64 and hold a multiple of four tokens, else key by key.
+template <typename T, typename C, int WAVES>
+__global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_generic_kernel(
     const T* __restrict__ qkv, int64_t q_stride, const C* __restrict__ k_cache, const C* __restrict__ v_cache,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_request,
     const int32_t* __restrict__ block_table, int table_width, T* __restrict__ out, int heads, int kv_heads,
     int block_size, float scale, int window) {
   __shared__ float q_s[D];
-  __shared__ float p_s[DISTIE_WAVE];
-  __shared__ int64_t at_s[DISTIE_WAVE];
-  const int lane = threadIdx.x;
+  __shared__ float p_s[WAVES][DISTIE_WAVE];
+  __shared__ int64_t base_s[WAVES][DISTIE_WAVE];
+  __shared__ float m_s[WAVES], l_s[WAVES];
+  __shared__ float acc_s[WAVES][D];
+  const int lane = threadIdx.x % DISTIE_WAVE;
+  const int wave = threadIdx.x / DISTIE_WAVE;
   const int64_t t = blockIdx.x;
   const int h = blockIdx.y;
   const int kh = h / (heads / kv_heads);
   const int q_pos = positions[t];
   const int32_t* table = block_table + static_cast<int64_t>(token_request[t]) * table_width;
   const T* q = qkv + t * q_stride + static_cast<int64_t>(h) * D;
-  for (int d = lane; d < D; d += DISTIE_WAVE) q_s[d] = to_float(q[d]);
+  for (int d = threadIdx.x; d < D; d += DISTIE_WAVE * WAVES) q_s[d] = to_float(q[d]);
   __syncthreads();
 
   const int first = window > 0 ? max(0, q_pos - window + 1) : 0;
   const int last = q_pos;   // inclusive
+  const bool by_page = block_size % 4 == 0 && DISTIE_WAVE % block_size == 0;
   float m = -INFINITY, l = 0.f;
   float acc[DIMS_PER_LANE];
 #pragma unroll
   for (int i = 0; i < DIMS_PER_LANE; ++i) acc[i] = 0.f;
 
-  for (int c = first; c <= last; c += DISTIE_WAVE) {
+  for (int c = first / DISTIE_WAVE * DISTIE_WAVE + wave * DISTIE_WAVE; c <= last; c += DISTIE_WAVE * WAVES) {
     const int key = c + lane;
-    const bool valid = key <= last;
+    const bool valid = key >= first && key <= last;
     float s = -INFINITY;
-    int64_t at = 0;
+    int64_t base = 0;
     if (valid) {
       const int page = table[key / block_size];
-      const int64_t base = (static_cast<int64_t>(page) * kv_heads + kh) * block_size * D;
-      const int offset = key % block_size;
-      at = base + offset;                      // of the value: v[base + d * block_size + offset]
-      s = dot_row<C>(q_s, k_cache + base + static_cast<int64_t>(offset) * D) * scale;
+      base = (static_cast<int64_t>(page) * kv_heads + kh) * block_size * D;
+      s = dot_row<C>(q_s, k_cache + base + static_cast<int64_t>(key % block_size) * D) * scale;
     }
     const float m_new = fmaxf(m, wave_max(s));
-    const float alpha = expf(m - m_new);          // 0 on the first chunk (m = -inf)
+    const float alpha = m_new == -INFINITY ? 0.f : expf(m - m_new);     // 0 on the first chunk with a key (m = -inf)
     const float p = valid ? expf(s - m_new) : 0.f;
     l = l * alpha + wave_sum(p);
     m = m_new;
-    __syncthreads();
-    p_s[lane] = p;
-    at_s[lane] = at;
-    __syncthreads();
-    const int n = min(DISTIE_WAVE, last - c + 1);
+    // what the lanes of this wave hand each other goes through the wave's own rows of LDS; the wave runs its
+    // LDS traffic in order, so no barrier across waves is needed, only that the compiler keeps the order
+    __builtin_amdgcn_wave_barrier();
+    p_s[wave][lane] = p;
+    base_s[wave][lane] = base;
+    __builtin_amdgcn_wave_barrier();
+    const int lo = max(first - c, 0);                                   // keys lo .. hi of the chunk count
+    const int hi = min(DISTIE_WAVE - 1, last - c);
 #pragma unroll
     for (int i = 0; i < DIMS_PER_LANE; ++i) {
       const int d = lane + i * DISTIE_WAVE;
-      if (d < D) {
-        float a = acc[i] * alpha;
-        for (int j = 0; j < n; ++j) a = fmaf(p_s[j], to_float(v_cache[at_s[j] + static_cast<int64_t>(d) * block_size]), a);
-        acc[i] = a;
+      if (d >= D) continue;
+      float a = acc[i] * alpha;
+      if (by_page) {
+        for (int j0 = lo / block_size * block_size; j0 <= hi; j0 += block_size) {
+          // the page of keys j0 .. j0 + P - 1: its address from a key of it that counts
+          const C* row = v_cache + base_s[wave][max(j0, lo)] + static_cast<int64_t>(d) * block_size;
+          for (int jj = 0; jj < block_size; jj += 4) {
+            float v[4];
+            load4(row + jj, v);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int j = j0 + jj + e;
+              if (j >= lo && j <= hi) a = fmaf(p_s[wave][j], v[e], a);    // never a value of a key that does not count
+            }
+          }
+        }
+      } else {
+        for (int j = lo; j <= hi; ++j)
+          a = fmaf(p_s[wave][j], to_float(v_cache[base_s[wave][j] + static_cast<int64_t>(d) * block_size + (c + j) % block_size]), a);
       }
+      acc[i] = a;
     }
   }
   T* o = out + (t * heads + h) * D;
-  const float inv = 1.f / l;
+  if constexpr (WAVES == 1) {
+    const float inv = 1.f / l;
 #pragma unroll
-  for (int i = 0; i < DIMS_PER_LANE; ++i) {
-    const int d = lane + i * DISTIE_WAVE;
-    if (d < D) o[d] = from_float<T>(acc[i] * inv);
+    for (int i = 0; i < DIMS_PER_LANE; ++i) {
+      const int d = lane + i * DISTIE_WAVE;
+      if (d < D) o[d] = from_float<T>(acc[i] * inv);
+    }
+  } else {
+    if (lane == 0) {
+      m_s[wave] = m;
+      l_s[wave] = l;
+    }
+#pragma unroll
+    for (int i = 0; i < DIMS_PER_LANE; ++i) {
+      const int d = lane + i * DISTIE_WAVE;
+      if (d < D) acc_s[wave][d] = acc[i];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float top = -INFINITY;
+    for (int w = 0; w < WAVES; ++w) top = fmaxf(top, m_s[w]);
+    float total = 0.f;
+    float weight[WAVES];
+    for (int w = 0; w < WAVES; ++w) {
+      weight[w] = m_s[w] == -INFINITY ? 0.f : expf(m_s[w] - top);       // a wave without keys counts nothing
+      total += l_s[w] * weight[w];
+    }
+    const float inv = 1.f / total;
+#pragma unroll
+    for (int i = 0; i < DIMS_PER_LANE; ++i) {
+      const int d = lane + i * DISTIE_WAVE;
+      if (d >= D) continue;
+      float sum = 0.f;
+      for (int w = 0; w < WAVES; ++w) sum += acc_s[w][d] * weight[w];
+      o[d] = from_float<T>(sum * inv);
+    }
   }
 }
 
@@ -137,14 +218,24 @@ extern "C" int distie_attention_generic(const void* qkv, int dtype, int64_t q_st
     return DISTIE_BAD_ARGUMENT;
   if (heads > 65535) return DISTIE_BAD_ARGUMENT;
   dim3 grid(tokens, heads);
-  DISTIE_DISPATCH(dtype, T, DISTIE_DISPATCH(cache_dtype, C,
-      attn_generic_kernel<T, C><<<grid, DISTIE_WAVE, 0, stream>>>(
-          static_cast<const T*>(qkv), q_stride, static_cast<const C*>(k_cache), static_cast<const C*>(v_cache),
-          positions, token_request, block_table, table_width, static_cast<T*>(out), heads, kv_heads, block_size,
-          scale, window)));
+  // few (token, head) pairs, as when requests decode: eight waves share each pair's keys
+  if (static_cast<int64_t>(tokens) * heads < 2048) {
+    DISTIE_DISPATCH(dtype, T, DISTIE_DISPATCH(cache_dtype, C,
+        (attn_generic_kernel<T, C, 8><<<grid, DISTIE_WAVE * 8, 0, stream>>>(
+            static_cast<const T*>(qkv), q_stride, static_cast<const C*>(k_cache), static_cast<const C*>(v_cache),
+            positions, token_request, block_table, table_width, static_cast<T*>(out), heads, kv_heads, block_size,
+            scale, window))));
+  } else {
+    DISTIE_DISPATCH(dtype, T, DISTIE_DISPATCH(cache_dtype, C,
+        (attn_generic_kernel<T, C, 1><<<grid, DISTIE_WAVE, 0, stream>>>(
+            static_cast<const T*>(qkv), q_stride, static_cast<const C*>(k_cache), static_cast<const C*>(v_cache),
+            positions, token_request, block_table, table_width, static_cast<T*>(out), heads, kv_heads, block_size,
+            scale, window))));
+  }
   return launch_status();
 }
 
+#if DISTIE_MATRIX_CORE_ATTENTION
 // ===================================================================================================
 //  Matrix-core kernels (bfloat16, pages of a multiple of 16 tokens). Both work on 16-wide blocks of
 //  "columns" against blocks of 16 keys with two products:
@@ -981,3 +1072,21 @@ extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, 
       part_o, part_ml, token_request, cu_q, static_cast<bf16_t*>(out), tokens, heads, min_q_len, splits);
   return launch_status();
 }
+
+#else   // a head size that is no multiple of 16: the wave-per-token kernel is all there is
+
+extern "C" int distie_attention_decode_columns() { return 0; }
+
+extern "C" int distie_attention_decode_bf16(const void*, int64_t, const void*, const void*, const int32_t*, const int32_t*,
+                                            const int32_t*, int, void*, void*, void*, int, int, int, int, float, int, int,
+                                            int, int, hipStream_t) {
+  return DISTIE_BAD_ARGUMENT;
+}
+
+extern "C" int distie_attention_prefill_bf16(const void*, int64_t, const void*, const void*, const int32_t*, const int32_t*,
+                                             const int32_t*, int, void*, int, int, int, int, int, float, int, int,
+                                             const int32_t*, void*, void*, int, hipStream_t) {
+  return DISTIE_BAD_ARGUMENT;
+}
+
+#endif

@@ -4,7 +4,8 @@ Three kinds of shared library, all built from the sources beside this file:
 
 * `core`  - the id pool of the cache manager (C++, host only, g++);
 * `ops`   - the HIP kernels that do not depend on the head size (hipcc, gfx950);
-* `attn_d<D>` - the attention kernels for head size D (hipcc, `-DDISTIE_HEAD_DIM=D`).
+* `attn_d<D>` - the attention kernels for head size D (hipcc, `-DDISTIE_HEAD_DIM=D`; the matrix-core
+  kernels for multiples of 16, the wave-per-token kernel for every even size).
 
 A library's file name carries a hash of its sources and flags, so a stale build is never
 loaded. Libraries live in `distie_amd/_lib/` (in-tree); if that folder cannot be written,
@@ -34,7 +35,7 @@ HIP_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17",
              "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
 CXX_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-pthread"]
 
-OPS_SOURCES = ["elementwise.hip", "gemm.hip", "decode_products.hip", "sampling.hip"]
+OPS_SOURCES = ["elementwise.hip", "gemm.hip", "gemv.hip", "decode_products.hip", "sampling.hip"]
 ATTN_SOURCES = ["attention.hip"]
 HEADERS = ["common.h"]
 OPS_HEADERS = ["no_alloc.h", "packed.h"]
@@ -68,8 +69,8 @@ def _spec(name: str):
         return list(OPS_SOURCES), _hipcc(), list(HIP_FLAGS)
     if name.startswith("attn_d"):
         dim = int(name[len("attn_d"):])
-        if dim < 16 or dim > 256 or dim % 16:
-            raise BuildError(f"attention kernels are built for head sizes 16, 32, ..., 256, not {dim}")
+        if dim < 2 or dim > 256 or dim % 2:
+            raise BuildError(f"attention kernels are built for even head sizes up to 256, not {dim}")
         return list(ATTN_SOURCES), _hipcc(), list(HIP_FLAGS) + [f"-DDISTIE_HEAD_DIM={dim}"]
     raise BuildError(f"no native library named {name}")
 
@@ -186,7 +187,7 @@ def ensure(name: str) -> Path:
     return build(name, force=False)
 
 
-DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 256)
+DEFAULT_HEAD_DIMS = (16, 32, 40, 48, 64, 80, 96, 112, 128, 256)
 
 
 def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True) -> List[Path]:

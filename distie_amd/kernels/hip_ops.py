@@ -112,6 +112,9 @@ class HipOps(Ops):
     # count: steps that are launched kernel by kernel take this path, captured steps do not.
     FUSED_MAX_ROWS = 16
     FUSED_IN_CAPTURED_STEPS = False
+    # float32 products (and products against weights kept in float32) of up to ROWS_MAX_ROWS rows stream the weights
+    # through `gemv_rows` (FMAs on the vector ALU); beyond that the tiled float32 kernel
+    ROWS_MAX_ROWS = 64
     # bfloat16 products by rows of x: up to SKINNY_MAX_ROWS the weights are streamed by one wave per block
     # of 16 weight rows, x straight from memory (above that, the library's tiles are faster);
     SKINNY_MAX_ROWS = 16
@@ -196,6 +199,7 @@ class HipOps(Ops):
         o.distie_sum_slices.argtypes = [_P, _I, _L, _P, _I, _P]
         o.distie_gather_rows.argtypes = [_P, _P, _P, _I, _L, _I, _P]
         o.distie_gemm_generic.argtypes = [_P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _P]
+        o.distie_gemv_rows.argtypes = [_P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _P]
         o.distie_gemm_skinny_slices.argtypes = [_I, _I, _I]
         o.distie_gemm_skinny_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _P]
         o.distie_pack_rows.argtypes = [_P, _P, _P, _I, _I, _P]
@@ -245,8 +249,8 @@ class HipOps(Ops):
     def attention_library(self, head_dim: int) -> ctypes.CDLL:
         lib = self._attn.get(head_dim)
         if lib is None:
-            if head_dim % 16 or not 16 <= head_dim <= 256:
-                raise KernelError(f"attention kernels take head sizes 16, 32, ..., 256, not {head_dim}")
+            if head_dim % 2 or not 2 <= head_dim <= 256:
+                raise KernelError(f"attention kernels take even head sizes up to 256, not {head_dim}")
             lib = ctypes.CDLL(str(build.ensure(f"attn_d{head_dim}")))
             lib.distie_attention_generic.argtypes = [_P, _I, _L, _P, _P, _I, _P, _P, _P, _I, _P,
                                                      _I, _I, _I, _I, _F, _I, _P]
@@ -609,6 +613,12 @@ class HipOps(Ops):
                 return y if bias is None else y + bias
             return torch.nn.functional.linear(x, weight, lib_bias)
         out = torch.empty((M, N), dtype=out_dtype, device=self.device)
+        if M <= self.ROWS_MAX_ROWS and K % 8 == 0:
+            # few rows in float32 (or against a weight kept in float32): the weights are streamed, FMAs only
+            _check(self._ops.distie_gemv_rows(
+                x.data_ptr(), _code(x), weight.data_ptr(), _code(weight), bias.data_ptr() if bias is not None else None,
+                out.data_ptr(), _CODES[out_dtype], M, N, K, self._stream()), "gemv_rows")
+            return out
         _check(self._ops.distie_gemm_generic(
             x.data_ptr(), _code(x), weight.data_ptr(), _code(weight), bias.data_ptr() if bias is not None else None,
             out.data_ptr(), _CODES[out_dtype], M, N, K, self._stream()), "gemm_generic")
@@ -661,7 +671,7 @@ class HipOps(Ops):
             raise KernelError("paged_attention: tensors do not match the batch")
         out = torch.empty((T, num_heads * head_dim), dtype=qkv.dtype, device=self.device)
         bf16 = qkv.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16
-        if bf16 and meta.block_size % 16 == 0:
+        if bf16 and meta.block_size % 16 == 0 and head_dim % 16 == 0:
             # how the step is launched, and its buffers for partial results, are the same for every layer
             # with these sizes: worked out once per step (the layers run one after the other, so they can
             # share the buffers)

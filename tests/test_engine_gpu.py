@@ -190,6 +190,7 @@ def test_layer_sizes_of_the_1_5b_model(tmp_path, ops):
 
 
 ODD_SIZES = [
+    dict(hidden_size=120, num_attention_heads=3, num_key_value_heads=1, head_dim=40, intermediate_size=96, vocab_size=77),
     dict(hidden_size=48, num_attention_heads=3, num_key_value_heads=1, head_dim=16, intermediate_size=100, vocab_size=1001),
     dict(hidden_size=336, num_attention_heads=7, num_key_value_heads=1, head_dim=48, intermediate_size=250, vocab_size=333,
          layer_types=["sliding_attention", "full_attention"], sliding_window=40),
@@ -204,7 +205,8 @@ ODD_SIZES = [
 def test_odd_sizes(tmp_path, ops, sizes, dtype_name):
     """Sizes at the edges of what the kernels take: a feed-forward width and a vocabulary that are no multiple
     of 8, seven and 66 query heads on one kv head (more than the decode kernel's columns), head sizes 16 and
-    256, a vocabulary of nine."""
+    256 and one that is no multiple of 16 (40: attention then runs on the wave-per-token kernel in both
+    precisions), a vocabulary of nine."""
     dtype = DTYPES[dtype_name]
     cfg = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 2, "rope_theta": 10000.0,
            "rms_norm_eps": 1e-5, "tie_word_embeddings": True, "max_position_embeddings": 512, "hidden_act": "silu", **sizes}

@@ -99,6 +99,38 @@ def test_gemm_generic(ops, xd, wd, M, N, K):
         close(got32, x.double() @ w.double().T, torch.float32, scale=want.abs().max().item())
 
 
+@pytest.mark.parametrize("xd,wd", [(torch.float32, torch.float32), (torch.bfloat16, torch.float32),
+                                   (torch.float32, torch.bfloat16)])
+@pytest.mark.parametrize("M", [1, 2, 3, 5, 8, 9, 17, 64, 65])
+@pytest.mark.parametrize("N,K", [(100, 72), (333, 256), (1536, 8960), (7, 8), (2050, 1536)])
+def test_products_of_few_rows_in_float32_stream_the_weights(ops, xd, wd, M, N, K):
+    """Up to 64 rows in float32 (or against a weight that is kept in float32) go through the kernel that streams
+    the weights and multiplies on the vector ALU: the same values as the tiled float32 kernel within float32
+    rounding (another order of the sums), whatever the row count, with and without a bias."""
+    x, w, b = rand(M, K, dtype=xd, seed=1), rand(N, K, dtype=wd, seed=2), rand(N, seed=3)
+    want = x.double() @ w.double().T + b.double()
+    scale = want.abs().max().item()
+    got = ops._linear(x, w, b, xd)
+    assert got.dtype == xd and tuple(got.shape) == (M, N)
+    close(got, want, xd, scale=scale)
+    tiled = torch.empty(M, N, dtype=xd, device="cuda")
+    code = {torch.float32: 0, torch.bfloat16: 1}
+    assert ops._ops.distie_gemm_generic(x.data_ptr(), code[xd], w.data_ptr(), code[wd], b.data_ptr(), tiled.data_ptr(),
+                                        code[xd], M, N, K, None) == 0
+    assert (got.float() - tiled.float()).abs().max().item() <= (2e-5 if xd == torch.float32 else 2 ** -7) * scale
+    logits = ops.linear_f32out(x, w)
+    assert logits.dtype == torch.float32
+    close(logits, x.double() @ w.double().T, torch.float32, scale=scale)
+    if M <= 64:
+        # it is this kernel that ran: its entry point gives the same bits
+        direct = torch.empty(M, N, dtype=torch.float32, device="cuda")
+        assert ops._ops.distie_gemv_rows(x.data_ptr(), code[xd], w.data_ptr(), code[wd], None, direct.data_ptr(), 0,
+                                         M, N, K, None) == 0
+        assert torch.equal(direct, logits)
+    assert ops._ops.distie_gemv_rows(x.data_ptr(), code[xd], w.data_ptr(), code[wd], None, logits.data_ptr(), 0,
+                                     65, N, K, None) == -1                     # more rows than it takes: refused
+
+
 @pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 64])
 @pytest.mark.parametrize("N,K", [(48, 128), (100, 264), (1536, 1536), (333, 8960), (2050, 72)])
 def test_gemm_skinny_bf16(ops, M, N, K):
@@ -458,7 +490,8 @@ def paged_case(heads, kv_heads, dim, P, lens, q_lens, dtype, seed=0):
 ATTENTION_SHAPES = [
     (4, 2, 16, 4, None), (3, 1, 32, 8, 8), (5, 5, 48, 16, 20), (12, 2, 128, 16, None),
     (6, 3, 64, 5, 33), (8, 1, 80, 16, None), (2, 2, 256, 32, 100), (4, 2, 16, 16, 7), (40, 2, 32, 16, None),
-    (12, 2, 128, 64, 150), (4, 2, 64, 16, 1000)]
+    (12, 2, 128, 64, 150), (4, 2, 64, 16, 1000),
+    (3, 1, 40, 16, None), (2, 2, 40, 8, 9)]        # a head size that is no multiple of 16: the wave-per-token kernel
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
