@@ -75,6 +75,12 @@ class CacheGroup:
     members: List[tuple]                  # (layer, mixer name) of every mixer that shares these pages
     pool: BlockPool
     tensors: Dict[str, torch.Tensor] = field(default_factory=dict)    # name -> [members, pages + 1, *page shape]
+    # The block tables as the kernels read them: int32 [slots + 1, width] on the device, row = a request's state
+    # slot (the last row belongs to the padding rows of captured steps and names the sink page). It lives from
+    # step to step; `changed` holds the entries that the book-keeping has changed since the last step took them
+    # along (flat index -> page), so a step costs the same whether its requests hold ten pages or ten thousand.
+    table: Optional[torch.Tensor] = None
+    changed: Dict[int, int] = field(default_factory=dict)
 
     @property
     def layers(self) -> List[int]:
@@ -90,6 +96,7 @@ class RequestCache:
     slot: int
     num_cached: int = 0
     tables: List[List[int]] = field(default_factory=list)   # per group, by page index
+    passed: List[int] = field(default_factory=list)         # per group: entries before this one are all given back
 
 
 class CacheManager:
@@ -143,6 +150,42 @@ class CacheManager:
                     group=index, tensors={n: slab[i] for n, slab in group.tensors.items()})
         self.slots = BlockPool(self.num_slots)
         self._requests: Dict[Hashable, RequestCache] = {}
+        self.table_width = 0
+
+    # ---------------------------------------------------------------- block tables on the device
+    def bind_tables(self, width: int) -> None:
+        """Make the device tables, `width` entries a request (once; the step function's builder calls this with
+        the most pages a request can hold)."""
+        if self.table_width:
+            if width != self.table_width:
+                raise ValueError(f"the block tables are {self.table_width} entries wide, not {width}")
+            return
+        self.table_width = int(width)
+        for group in self.groups:
+            table = torch.full((self.num_slots + 1, self.table_width), GONE, dtype=torch.int32)
+            table[self.sink_slot, 0] = group.sink_page
+            group.table = table.to(self.device) if self.device is not None else table
+            group.changed.clear()
+            # what requests hold already goes along with the next step
+            for entry in self._requests.values():
+                g = self.groups.index(group)
+                for i, page in enumerate(entry.tables[g]):
+                    group.changed[entry.slot * self.table_width + i] = page
+
+    def _note(self, group: CacheGroup, slot: int, index: int, page: int) -> None:
+        if self.table_width:
+            if index >= self.table_width:
+                raise ValueError(f"a request would hold more than {self.table_width} pages")
+            group.changed[slot * self.table_width + index] = page
+
+    def take_changes(self, g: int):
+        """-> (flat indexes, pages) of group g's table entries that changed since the last call, as lists."""
+        changed = self.groups[g].changed
+        if not changed:
+            return (), ()
+        out = (list(changed.keys()), list(changed.values()))
+        changed.clear()
+        return out
 
     # ---------------------------------------------------------------- views
     def layer(self, layer: int) -> LayerCache:
@@ -176,7 +219,7 @@ class CacheManager:
             raise OutOfBlocks(f"no free state slot (all {self.num_slots} in use)") from exc
         for slab in self._state_slabs:
             slab[slot].zero_()
-        entry = RequestCache(slot=slot, tables=[[] for _ in self.groups])
+        entry = RequestCache(slot=slot, tables=[[] for _ in self.groups], passed=[0 for _ in self.groups])
         self._requests[request_id] = entry
         return entry
 
@@ -234,8 +277,12 @@ class CacheManager:
             table = entry.tables[g]
             # pages the window has already passed are never taken
             while len(table) < last - need:
+                self._note(group, entry.slot, len(table), GONE)
                 table.append(GONE)
-            table.extend(group.pool.allocate(need))
+                entry.passed[g] = len(table)
+            for page in group.pool.allocate(need):
+                self._note(group, entry.slot, len(table), page)
+                table.append(page)
 
     def commit(self, request_id, num_new: int) -> None:
         """The step has written `num_new` more tokens; give back what windows have passed."""
@@ -246,11 +293,16 @@ class CacheManager:
                 continue
             table = entry.tables[g]
             stop = min(self._first_needed_page(group, entry.num_cached), len(table))
-            passed = [table[i] for i in range(stop) if table[i] != GONE]
-            if passed:
-                group.pool.free(passed)
-                for i in range(stop):
-                    table[i] = GONE
+            begin = entry.passed[g]
+            if stop > begin:
+                passed = [table[i] for i in range(begin, stop) if table[i] != GONE]
+                if passed:
+                    group.pool.free(passed)
+                for i in range(begin, stop):
+                    if table[i] != GONE:
+                        table[i] = GONE
+                        self._note(group, entry.slot, i, GONE)
+                entry.passed[g] = stop
 
     def _give_back_pages(self, entry: RequestCache) -> None:
         for g, group in enumerate(self.groups):
@@ -258,6 +310,7 @@ class CacheManager:
             if held:
                 group.pool.free(held)
             entry.tables[g] = []
+            entry.passed[g] = 0
         entry.num_cached = 0
 
     def reset(self, request_id) -> None:

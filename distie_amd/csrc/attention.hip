@@ -3,7 +3,8 @@
 //
 // out[t, h] = softmax_j(q[t, h] . k[j, h / G] * scale) v[j, h / G] over the keys j that token t may see:
 // first(t) <= j <= position(t), first = 0, or position - window + 1 on a windowed layer. Keys and values
-// are read through the block table of the token's request: key j lives in page table[j / P] at offset
+// are read through the block table of the token's request (row table_rows[request] of block_table, or row
+// `request` itself when table_rows is null): key j lives in page table[j / P] at offset
 // j % P of a cache laid out k [pages, kv_heads, P, D], v [pages, kv_heads, D, P]. The new tokens of the step are
 // already in the cache
 // (the reference writes before it reads too: worker/src/inference/qwen2/paged_attn.py:389-397), so
@@ -92,7 +93,7 @@ template <typename T, typename C, int WAVES>
 __global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_generic_kernel(
     const T* __restrict__ qkv, int64_t q_stride, const C* __restrict__ k_cache, const C* __restrict__ v_cache,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_request,
-    const int32_t* __restrict__ block_table, int table_width, T* __restrict__ out, int heads, int kv_heads,
+    const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ table_rows, T* __restrict__ out, int heads, int kv_heads,
     int block_size, float scale, int window) {
   __shared__ float q_s[D];
   __shared__ float p_s[WAVES][DISTIE_WAVE];
@@ -105,7 +106,8 @@ __global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_generic_kernel(
   const int h = blockIdx.y;
   const int kh = h / (heads / kv_heads);
   const int q_pos = positions[t];
-  const int32_t* table = block_table + static_cast<int64_t>(token_request[t]) * table_width;
+  const int request_of_token = token_request[t];
+  const int32_t* table = block_table + static_cast<int64_t>(table_rows != nullptr ? table_rows[request_of_token] : request_of_token) * table_width;
   const T* q = qkv + t * q_stride + static_cast<int64_t>(h) * D;
   for (int d = threadIdx.x; d < D; d += DISTIE_WAVE * WAVES) q_s[d] = to_float(q[d]);
   __syncthreads();
@@ -211,7 +213,7 @@ __global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_generic_kernel(
 extern "C" int distie_attention_generic(const void* qkv, int dtype, int64_t q_stride, const void* k_cache,
                                         const void* v_cache, int cache_dtype, const int32_t* positions,
                                         const int32_t* token_request, const int32_t* block_table,
-                                        int table_width, void* out, int tokens, int heads, int kv_heads,
+                                        int table_width, const int32_t* table_rows, void* out, int tokens, int heads, int kv_heads,
                                         int block_size, float scale, int window, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size < 1 || table_width < 1 || window < 0)
@@ -223,13 +225,13 @@ extern "C" int distie_attention_generic(const void* qkv, int dtype, int64_t q_st
     DISTIE_DISPATCH(dtype, T, DISTIE_DISPATCH(cache_dtype, C,
         (attn_generic_kernel<T, C, 8><<<grid, DISTIE_WAVE * 8, 0, stream>>>(
             static_cast<const T*>(qkv), q_stride, static_cast<const C*>(k_cache), static_cast<const C*>(v_cache),
-            positions, token_request, block_table, table_width, static_cast<T*>(out), heads, kv_heads, block_size,
+            positions, token_request, block_table, table_width, table_rows, static_cast<T*>(out), heads, kv_heads, block_size,
             scale, window))));
   } else {
     DISTIE_DISPATCH(dtype, T, DISTIE_DISPATCH(cache_dtype, C,
         (attn_generic_kernel<T, C, 1><<<grid, DISTIE_WAVE, 0, stream>>>(
             static_cast<const T*>(qkv), q_stride, static_cast<const C*>(k_cache), static_cast<const C*>(v_cache),
-            positions, token_request, block_table, table_width, static_cast<T*>(out), heads, kv_heads, block_size,
+            positions, token_request, block_table, table_width, table_rows, static_cast<T*>(out), heads, kv_heads, block_size,
             scale, window))));
   }
   return launch_status();
@@ -294,7 +296,7 @@ template <int MB>
 __global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ qkv, int64_t q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ kv_len, const int32_t* __restrict__ cu_q,
-    const int32_t* __restrict__ block_table, int table_width, float* __restrict__ part_o,
+    const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ table_rows, float* __restrict__ part_o,
     float* __restrict__ part_ml, int heads, int kv_heads, int block_size, float scale, int window, int split_hint,
     int max_splits, int dense_rows) {
   const int lane = threadIdx.x;
@@ -304,7 +306,7 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
   const float scale_log2 = scale * 1.4426950408889634f;
   const int request = blockIdx.z;
   const int kh = blockIdx.y;
-  const int32_t* table = block_table + static_cast<int64_t>(request) * table_width;
+  const int32_t* table = block_table + static_cast<int64_t>(table_rows != nullptr ? table_rows[request] : request) * table_width;
   // The pages of the run's first chunk are asked for before the request's length says where the run begins:
   // at the place it has if the runs are `split_hint` long and begin at key 0, which the host derives from the
   // longest request of the step (the entry is inside the table either way). Where the guess holds, which it
@@ -632,7 +634,7 @@ extern "C" int distie_attention_decode_columns() { return 16 * DECODE_MAX_MB; }
 // the run length the caller expects of the longest request; it only saves time where it is right.
 extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, const void* k_cache, const void* v_cache,
                                             const int32_t* kv_len, const int32_t* cu_q, const int32_t* block_table,
-                                            int table_width, void* out, float* part_o, float* part_ml,
+                                            int table_width, const int32_t* table_rows, void* out, float* part_o, float* part_ml,
                                             int num_requests, int heads, int kv_heads, int block_size, float scale,
                                             int window, int split_hint, int max_splits, int dense_rows,
                                             hipStream_t stream) {
@@ -647,7 +649,7 @@ extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, c
   const bf16_t* kc = static_cast<const bf16_t*>(k_cache);
   const bf16_t* vc = static_cast<const bf16_t*>(v_cache);
 #define DECODE_LAUNCH(MB)                                                                                             \
-  attn_decode_kernel<MB><<<grid, DISTIE_WAVE, 0, stream>>>(q, q_stride, kc, vc, kv_len, cu_q, block_table, table_width, \
+  attn_decode_kernel<MB><<<grid, DISTIE_WAVE, 0, stream>>>(q, q_stride, kc, vc, kv_len, cu_q, block_table, table_width, table_rows, \
                                                            part_o, part_ml, heads, kv_heads, block_size, scale, window, \
                                                            split_hint, max_splits, dense_rows)
   if (group <= 16) {
@@ -706,7 +708,7 @@ static_assert(PF_WAVES * 16 == PF_BN, "each wave brings one block of 16 keys of 
 __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_kernel(
     const bf16_t* __restrict__ qkv, int64_t q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ positions, const int32_t* __restrict__ cu_q,
-    const int32_t* __restrict__ block_table, int table_width, bf16_t* __restrict__ out, float* __restrict__ part_o,
+    const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ table_rows, bf16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, int tokens, int num_requests, int heads, int kv_heads, int block_size, float scale,
     int window, int min_q_len) {
   __shared__ __attribute__((aligned(16))) bf16_t k_lds[PF_BN * PF_K_STRIDE];
@@ -739,7 +741,7 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
   const int pos0 = positions[token0];                     // the tokens of a portion have consecutive positions
   const int key_begin = window > 0 ? max(0, pos0 - window + 1) : 0;
   const int key_end = pos0 + columns - 1;
-  const int32_t* table = block_table + static_cast<int64_t>(request) * table_width;
+  const int32_t* table = block_table + static_cast<int64_t>(table_rows != nullptr ? table_rows[request] : request) * table_width;
 
   // ---- this wave's columns
   const int wave_col0 = wave * PF_WAVE_COLS;
@@ -1048,7 +1050,7 @@ __global__ void attn_prefill_merge_kernel(const float* __restrict__ part_o, cons
 // bring fewer than min_q_len tokens are skipped (the decode kernel serves them).
 extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, const void* k_cache, const void* v_cache,
                                              const int32_t* positions, const int32_t* cu_q, const int32_t* block_table,
-                                             int table_width, void* out, int tokens, int num_requests, int heads,
+                                             int table_width, const int32_t* table_rows, void* out, int tokens, int num_requests, int heads,
                                              int kv_heads, int block_size, float scale, int window, int min_q_len,
                                              const int32_t* token_request, float* part_o, float* part_ml,
                                              int splits, hipStream_t stream) {
@@ -1063,7 +1065,7 @@ extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, 
   if (tiles > 65535) return DISTIE_BAD_ARGUMENT;
   attn_prefill_kernel<<<dim3(heads, tiles, splits), PF_THREADS, 0, stream>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),
-      positions, cu_q, block_table, table_width, static_cast<bf16_t*>(out), part_o, part_ml, tokens, num_requests, heads,
+      positions, cu_q, block_table, table_width, table_rows, static_cast<bf16_t*>(out), part_o, part_ml, tokens, num_requests, heads,
       kv_heads, block_size, scale, window, min_q_len);
   int status = launch_status();
   if (status != 0 || splits == 1) return status;
@@ -1078,13 +1080,13 @@ extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, 
 extern "C" int distie_attention_decode_columns() { return 0; }
 
 extern "C" int distie_attention_decode_bf16(const void*, int64_t, const void*, const void*, const int32_t*, const int32_t*,
-                                            const int32_t*, int, void*, void*, void*, int, int, int, int, float, int, int,
+                                            const int32_t*, int, const int32_t*, void*, void*, void*, int, int, int, int, float, int, int,
                                             int, int, hipStream_t) {
   return DISTIE_BAD_ARGUMENT;
 }
 
 extern "C" int distie_attention_prefill_bf16(const void*, int64_t, const void*, const void*, const int32_t*, const int32_t*,
-                                             const int32_t*, int, void*, int, int, int, int, int, float, int, int,
+                                             const int32_t*, int, const int32_t*, void*, int, int, int, int, int, float, int, int,
                                              const int32_t*, void*, void*, int, hipStream_t) {
   return DISTIE_BAD_ARGUMENT;
 }

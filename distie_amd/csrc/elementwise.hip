@@ -508,3 +508,22 @@ extern "C" int distie_gather_rows(const void* src, const int32_t* rows, void* ds
                                                 static_cast<uint8_t*>(dst), row_bytes, src_rows);
   return launch_status();
 }
+
+// ---------------------------------------------------------------- scattered int32 writes
+// table[index[i]] = value[i]: how the block tables on the device follow the host's book-keeping (a step
+// brings only the entries that changed since the step before). The indexes of one call are distinct.
+__global__ void scatter_i32_kernel(int32_t* __restrict__ table, const int32_t* __restrict__ index,
+                                   const int32_t* __restrict__ value, int count, int64_t size) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  const int64_t at = index[i];
+  if (at >= 0 && at < size) table[at] = value[i];
+}
+
+extern "C" int distie_scatter_i32(int32_t* table, const int32_t* index, const int32_t* value, int count, int64_t size,
+                                  hipStream_t stream) {
+  if (count <= 0) return 0;
+  if (size <= 0) return DISTIE_BAD_ARGUMENT;
+  scatter_i32_kernel<<<(count + 255) / 256, 256, 0, stream>>>(table, index, value, count, size);
+  return launch_status();
+}

@@ -1,10 +1,14 @@
 """From (request, its next tokens) to the flat tensors of one step.
 
 The fields are those of the reference's `build_batch`
-(worker/src/inference/qwen2/paged_attn.py:325-357): positions, slots, prefix sums, block
-table; plus the request of each token, a table and slots for every cache group, state
-slots, and the rows whose logits are wanted. Everything is packed into one int32 host
-buffer and reaches the device with one copy.
+(worker/src/inference/qwen2/paged_attn.py:325-357): positions, slots, prefix sums; plus the
+request of each token, slots for every cache group, state slots, and the rows whose logits
+are wanted. Everything is packed into one int32 host buffer and reaches the device with one
+copy. The block tables are not rebuilt: they live on the device (one row per state slot, kept
+by the cache manager), and a step brings only the entries that changed since the step before,
+so what the host does for a step does not grow with the length of its requests' contexts
+(the reference rebuilds a padded table from Python lists every step and names that as a large
+share of its step's host time: benchmarks/results/stage4-a100-vs-vllm.md:53).
 """
 
 from __future__ import annotations
@@ -15,7 +19,7 @@ from typing import Hashable, List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..cache.manager import GONE, CacheManager
+from ..cache.manager import CacheManager
 from ..kernels.interface import BatchMeta, GroupMeta
 
 
@@ -32,12 +36,14 @@ class StepEntry:
 class BatchBuilder:
     STAGING_BUFFERS = 3
 
-    def __init__(self, cache: CacheManager, max_model_len: int, device, vocab_size: int) -> None:
+    def __init__(self, cache: CacheManager, max_model_len: int, device, vocab_size: int, ops=None) -> None:
         self.cache = cache
         self.device = device
+        self.ops = ops
         self.vocab_size = vocab_size
         self.max_model_len = int(max_model_len)
         self.table_width = max(1, -(-self.max_model_len // cache.block_size))
+        cache.bind_tables(self.table_width)
         # pinned staging buffers for the step descriptions, used in turn: [host tensor, its numpy view, event of
         # the last copy out of it]. With them the copy to the device does not wait for the work queued before
         # it, so the host can prepare a step while the one before still runs.
@@ -48,8 +54,23 @@ class BatchBuilder:
         """Offsets of the fields inside the packed int32 buffer of a step with T tokens, B requests
         and R wanted rows."""
         G = len(self.cache.groups)
-        sizes = [T, T, T, B + 1, B, B, R] + [B * self.table_width] * G + [T] * G
+        sizes = [T, T, T, B + 1, B, B, R] + [T] * G
         return np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+
+    def flush_tables(self) -> None:
+        """Bring the device's block tables up to the book-keeping: the entries that changed since the last
+        call, as one small copy and one scattered write per group (nothing, if nothing changed)."""
+        for g, group in enumerate(self.cache.groups):
+            index, value = self.cache.take_changes(g)
+            if not index:
+                continue
+            both = np.asarray([index, value], dtype=np.int32)
+            if self.ops is not None:
+                dev = self.ops.upload(both)
+                self.ops.scatter_int32(group.table, dev[0], dev[1])
+            else:
+                dev = torch.from_numpy(both).to(group.table.device)
+                group.table.view(-1)[dev[0].long()] = dev[1]
 
     def fill(self, host: np.ndarray, entries: Sequence[StepEntry], pad_requests: int = 0, want_all: bool = False):
         """Write the step into `host` (int32, at least layout(...)[-1] long).
@@ -62,7 +83,6 @@ class BatchBuilder:
             raise ValueError("a step needs at least one entry")
         cache = self.cache
         P = cache.block_size
-        W = self.table_width
         G = len(cache.groups)
         B = len(entries) + pad_requests
         T = sum(len(e.tokens) for e in entries) + pad_requests
@@ -75,10 +95,7 @@ class BatchBuilder:
         host[:offsets[-1]] = 0
         cut = lambda i: host[offsets[i]:offsets[i + 1]]
         ids, positions, token_request, cu_q, kv_len, slots_state, want_rows = (cut(i) for i in range(7))
-        tables = [cut(7 + g).reshape(B, W) for g in range(G)]
-        slots = [cut(7 + G + g) for g in range(G)]
-        for t in tables:
-            t.fill(GONE)
+        slots = [cut(7 + g) for g in range(G)]
         t0 = 0
         r0 = 0
         max_q = max_kv = 1
@@ -110,7 +127,6 @@ class BatchBuilder:
                     page = table[past // P]
                     if page < 0:
                         raise AssertionError("a new token would be written to a page that was given back")
-                    tables[g][b, :len(table)] = table
                     slots[g][t0] = page * P + past % P
             else:
                 toks = np.asarray(entry.tokens, dtype=np.int64)
@@ -120,12 +136,13 @@ class BatchBuilder:
                 pos = np.arange(past, past + n, dtype=np.int64)
                 positions[t0:t0 + n] = pos
                 token_request[t0:t0 + n] = b
+                first_page = past // P
                 for g in range(G):
-                    table = np.asarray(state.tables[g], dtype=np.int64)
-                    if len(table) * P < past + n:
+                    if len(state.tables[g]) * P < past + n:
                         raise ValueError(f"request {entry.request_id!r}: pages were not reserved for this step")
-                    tables[g][b, :len(table)] = table
-                    pages = table[pos // P]
+                    # the pages of the new positions only: the cost does not grow with what is cached already
+                    table = np.asarray(state.tables[g][first_page:(past + n - 1) // P + 1], dtype=np.int64)
+                    pages = table[pos // P - first_page]
                     if (pages < 0).any():
                         raise AssertionError("a new token would be written to a page that was given back")
                     slots[g][t0:t0 + n] = pages * P + pos % P
@@ -145,7 +162,6 @@ class BatchBuilder:
             kv_len[b] = 1
             slots_state[b] = cache.sink_slot
             for g, group in enumerate(cache.groups):
-                tables[g][b, 0] = group.sink_page
                 slots[g][t0] = group.sink_page * P
             t0 += 1
         if want_all:
@@ -155,15 +171,13 @@ class BatchBuilder:
     def meta_of(self, dev: torch.Tensor, offsets, T: int, B: int, R: int, max_q: int, max_kv: int,
                 host_cu_q=None, host_past=None):
         """Views into the device copy `dev` of a packed buffer -> (ids, BatchMeta, want_rows)."""
-        G = len(self.cache.groups)
-        W = self.table_width
         dcut = lambda i: dev[int(offsets[i]):int(offsets[i + 1])]
         meta = BatchMeta(
             num_tokens=T, num_requests=B,
             positions=dcut(1), token_request=dcut(2), cu_q=dcut(3), kv_len=dcut(4), state_slots=dcut(5),
             max_q=max_q, max_kv=max_kv, block_size=self.cache.block_size,
-            groups=[GroupMeta(block_table=dcut(7 + g).view(B, W), slots=dcut(7 + G + g)) for g in range(G)],
-            host_cu_q=host_cu_q, host_past=host_past, all_decode=(max_q == 1),
+            groups=[GroupMeta(block_table=group.table, slots=dcut(7 + g)) for g, group in enumerate(self.cache.groups)],
+            host_cu_q=host_cu_q, host_past=host_past, all_decode=(max_q == 1), table_rows=dcut(5),
         )
         return dcut(0), meta, (dcut(6) if R else None)
 
@@ -172,6 +186,7 @@ class BatchBuilder:
         T = sum(len(e.tokens) for e in entries)
         R = sum(len(e.want) for e in entries)
         words = int(self.layout(T, len(entries), R)[-1])
+        self.flush_tables()
         if torch.device(self.device).type != "cuda":
             host = np.empty(words, dtype=np.int32)
             offsets, T, B, R, max_q, max_kv, cu_q, past = self.fill(host, entries)

@@ -138,6 +138,7 @@ class DecodeGraphs:
     def _run(self, bucket: _Bucket, entries: Sequence[StepEntry], feed: Optional[torch.Tensor],
              max_kv: int) -> Optional[torch.Tensor]:
         runner = self.runner
+        runner.builder.flush_tables()                    # outside the graph: the number of changed entries varies
         bucket.dev.copy_(bucket.host, non_blocking=True)
         bucket.copied.record()
         if feed is not None and feed.shape[0]:

@@ -27,7 +27,7 @@ class ModelRunner:
         self.ops = ops
         self.act_dtype = act_dtype
         self.max_model_len = int(max_model_len or model.spec.max_positions)
-        self.builder = BatchBuilder(cache, self.max_model_len, ops.device, model.spec.vocab_size)
+        self.builder = BatchBuilder(cache, self.max_model_len, ops.device, model.spec.vocab_size, ops)
         self.graphs = None          # set by the engine when captured decode steps are on
         model.prepare(ops)
 

@@ -191,6 +191,7 @@ class HipOps(Ops):
 
     def _declare(self) -> None:
         o = self._ops
+        o.distie_scatter_i32.argtypes = [_P, _P, _P, _I, _L, _P]
         o.distie_embed.argtypes = [_P, _P, _I, _P, _I, _I, _I, _P]
         o.distie_rmsnorm.argtypes = [_P, _P, _I, _I, _P, _I, _P, _I, _I, _I, _F, _P]
         o.distie_rope_kv_write.argtypes = [_P, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P]
@@ -252,11 +253,11 @@ class HipOps(Ops):
             if head_dim % 2 or not 2 <= head_dim <= 256:
                 raise KernelError(f"attention kernels take even head sizes up to 256, not {head_dim}")
             lib = ctypes.CDLL(str(build.ensure(f"attn_d{head_dim}")))
-            lib.distie_attention_generic.argtypes = [_P, _I, _L, _P, _P, _I, _P, _P, _P, _I, _P,
+            lib.distie_attention_generic.argtypes = [_P, _I, _L, _P, _P, _I, _P, _P, _P, _I, _P, _P,
                                                      _I, _I, _I, _I, _F, _I, _P]
-            lib.distie_attention_prefill_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I,
+            lib.distie_attention_prefill_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I,
                                                           _F, _I, _I, _P, _P, _P, _I, _P]
-            lib.distie_attention_decode_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I,
+            lib.distie_attention_decode_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I,
                                                          _I, _F, _I, _I, _I, _I, _P]
             if lib.distie_attention_head_dim() != head_dim:
                 raise KernelError("attention library was built for another head size")
@@ -280,6 +281,14 @@ class HipOps(Ops):
                               "v [pages, kv_heads, head_dim, block_size]")
 
     # ------------------------------------------------------------ operations
+    def scatter_int32(self, table, index, value):
+        self._own(table, index, value)
+        if table.dtype != torch.int32 or index.dtype != torch.int32 or value.dtype != torch.int32 or \
+                index.shape != value.shape:
+            raise KernelError("scatter_int32 takes int32 tensors, one value for each index")
+        _check(self._ops.distie_scatter_i32(table.data_ptr(), index.data_ptr(), value.data_ptr(), index.numel(),
+                                            table.numel(), self._stream()), "scatter_i32")
+
     def embed(self, ids, table):
         self._own(ids, table)
         out = torch.empty((ids.shape[0], table.shape[1]), dtype=torch.float32, device=self.device)
@@ -667,8 +676,11 @@ class HipOps(Ops):
         T = qkv.shape[0]
         table = meta.groups[group].block_table
         self._check_cache(k_cache, v_cache, num_kv_heads, meta.block_size, head_dim)
-        if T != meta.num_tokens or table.shape[0] != meta.num_requests:
+        rows = meta.table_rows
+        if T != meta.num_tokens or (rows is None and table.shape[0] != meta.num_requests) or \
+                (rows is not None and rows.shape[0] != meta.num_requests):
             raise KernelError("paged_attention: tensors do not match the batch")
+        rows_ptr = rows.data_ptr() if rows is not None else None
         out = torch.empty((T, num_heads * head_dim), dtype=qkv.dtype, device=self.device)
         bf16 = qkv.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16
         if bf16 and meta.block_size % 16 == 0 and head_dim % 16 == 0:
@@ -683,7 +695,7 @@ class HipOps(Ops):
             if plan["decode"]:
                 _check(lib.distie_attention_decode_bf16(
                     qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), meta.kv_len.data_ptr(),
-                    meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], out.data_ptr(),
+                    meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], rows_ptr, out.data_ptr(),
                     plan["decode_o"].data_ptr(), plan["decode_ml"].data_ptr(), meta.num_requests, num_heads,
                     num_kv_heads, meta.block_size, float(scale), int(window or 0), plan["split_len"],
                     plan["max_splits"], 1 if meta.all_decode else 0, self._stream()), "attention_decode_bf16")
@@ -691,7 +703,7 @@ class HipOps(Ops):
                 parts = plan["parts"]
                 _check(lib.distie_attention_prefill_bf16(
                     qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), meta.positions.data_ptr(),
-                    meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], out.data_ptr(), T, meta.num_requests,
+                    meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], rows_ptr, out.data_ptr(), T, meta.num_requests,
                     num_heads, num_kv_heads, meta.block_size, float(scale), int(window or 0),
                     2 if plan["decode"] else 1, meta.token_request.data_ptr(),
                     plan["prefill_o"].data_ptr() if parts > 1 else None,
@@ -700,7 +712,7 @@ class HipOps(Ops):
             return out
         _check(lib.distie_attention_generic(
             qkv.data_ptr(), _code(qkv), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), _code(k_cache),
-            meta.positions.data_ptr(), meta.token_request.data_ptr(), table.data_ptr(), table.shape[1],
+            meta.positions.data_ptr(), meta.token_request.data_ptr(), table.data_ptr(), table.shape[1], rows_ptr,
             out.data_ptr(), T, num_heads, num_kv_heads, meta.block_size, float(scale), int(window or 0),
             self._stream()), "attention_generic")
         return out

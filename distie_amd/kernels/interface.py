@@ -25,7 +25,9 @@ import torch
 class GroupMeta:
     """Addressing of one cache group for one step."""
 
-    block_table: torch.Tensor          # int32 [B, W]; -1 where a page was given back
+    block_table: torch.Tensor          # int32 [rows, W]; -1 where a page was given back. Row of request b:
+    #                                    BatchMeta.table_rows[b] (the request's state slot: the tables live on the
+    #                                    device from step to step), or b itself where table_rows is None
     slots: torch.Tensor                # int32 [T]; block * block_size + offset of each new token
 
 
@@ -50,6 +52,7 @@ class BatchMeta:
     host_cu_q: Optional[object] = None
     host_past: Optional[object] = None
     all_decode: bool = False           # every request brings exactly one token
+    table_rows: Optional[torch.Tensor] = None    # int32 [B]: each request's row of the groups' block tables
     scratch: dict = field(default_factory=dict)   # what an implementation computes once per step (cos/sin tables)
 
 
@@ -63,6 +66,11 @@ class Ops(abc.ABC):
         """A small host array (row indexes, sampling parameters) as a device tensor of the same dtype and
         shape. An implementation makes this a copy that does not wait for the work queued before it."""
         return torch.from_numpy(np.ascontiguousarray(values)).to(self.device)
+
+    def scatter_int32(self, table: torch.Tensor, index: torch.Tensor, value: torch.Tensor) -> None:
+        """table.view(-1)[index] = value for int32 tensors on the device (distinct indexes): the block tables'
+        changed entries of a step."""
+        table.view(-1)[index.long()] = value
 
     @abc.abstractmethod
     def embed(self, ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:

@@ -4,6 +4,7 @@ random orders of requests; windows give pages back; the pool's contract."""
 import random
 
 import pytest
+import torch
 
 from distie_amd.cache import GONE, BlockPool, CacheManager, OutOfBlocks, pages_needed
 from distie_amd.parts import FixedState, PagedKV
@@ -127,6 +128,22 @@ def test_slots_run_out_and_come_back():
 def test_random_orders_lose_nothing(seed):
     rng = random.Random(seed)
     m = manager(block=rng.choice([2, 4, 8]), pages=rng.randint(10, 30), slots=4, window=rng.randint(1, 20))
+    m.device = "cpu"
+    m.bind_tables(64)              # the tables as the kernels read them: kept up to date entry by entry
+
+    def tables_follow():
+        """After the changed entries went along with a step, a live request's row holds what its list holds,
+        wherever a kernel may look (from the first page a query can still read)."""
+        for g, group in enumerate(m.groups):
+            index, value = m.take_changes(g)
+            if index:
+                assert len(set(index)) == len(index)
+                group.table.view(-1)[torch.tensor(index)] = torch.tensor(value, dtype=torch.int32)
+            assert group.table[m.sink_slot, 0] == group.sink_page
+            for rid in m.live():
+                entry = m.request(rid)
+                assert group.table[entry.slot, :len(entry.tables[g])].tolist() == entry.tables[g]
+
     live = {}
     n = 0
     for _ in range(600):
@@ -155,6 +172,8 @@ def test_random_orders_lose_nothing(seed):
             m.release(rid)
             del live[rid]
         m.check()
+        if rng.random() < 0.3:
+            tables_follow()
         for rid, cached in live.items():
             entry = m.request(rid)
             assert entry.num_cached == cached
@@ -163,6 +182,7 @@ def test_random_orders_lose_nothing(seed):
             # every page a query at the next position may read is there
             first = max(0, cached - m.groups[1].requirement.window + 1) // m.block_size
             assert all(p != GONE for p in windowed[first:])
+    tables_follow()
     for rid in list(live):
         m.release(rid)
     assert m.free_pages() == [m.num_blocks] * 2 and m.slots.num_free == 4

@@ -112,3 +112,40 @@ def test_wanted_rows_and_empty_want(setup):
     assert (logits[0] - wa[8]).abs().max() < FP32_TOL
     assert (logits[1] - wa[5]).abs().max() < FP32_TOL
     assert (logits[2] - wb[11]).abs().max() < FP32_TOL
+
+
+def test_filling_a_step_does_not_grow_with_the_contexts():
+    """64 requests that decode: what the host does to describe the step is the same at 2,000 and at 32,000
+    cached tokens a request, since the block tables live on the device and only changed entries travel."""
+    import time
+
+    import numpy as np
+
+    from distie_amd.cache import CacheManager
+    from distie_amd.engine.batch import BatchBuilder
+    from distie_amd.parts import PagedKV
+
+    def seconds(context):
+        cache = CacheManager([PagedKV(1, 16), PagedKV(1, 16, 4096)], 16, 64 * (context // 16 + 2), 64, device="cpu",
+                             allocate=False)
+        builder = BatchBuilder(cache, 40000, "cpu", 100)
+        entries = []
+        for r in range(64):
+            cache.add(r)
+            cache.reserve(r, context)
+            cache.commit(r, context)
+            cache.reserve(r, 1)
+            entries.append(StepEntry(r, [1], [0]))
+        builder.flush_tables()
+        host = np.empty(int(builder.layout(64, 64, 64)[-1]), dtype=np.int32)
+        best = 1e9
+        for _ in range(5):
+            began = time.perf_counter()
+            for _ in range(20):
+                builder.fill(host, entries)
+                builder.flush_tables()
+            best = min(best, time.perf_counter() - began)
+        return best
+
+    short, long = seconds(2000), seconds(32000)
+    assert long < 1.5 * short + 1e-3, (short, long)

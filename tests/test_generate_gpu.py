@@ -146,6 +146,9 @@ def test_a_corrupted_cache_fails_the_comparison(tmp_path, name, block, dtype):
             table = runner.cache.request("a").tables[group]
             assert len(table) >= 2 and table[-1] >= 0 and table[-2] >= 0       # both held: no page out of bounds
             table[-1], table[-2] = table[-2], table[-1]
+            slot = runner.cache.request("a").slot
+            for i in (len(table) - 1, len(table) - 2):          # ... and on the device, where the kernels read them
+                runner.cache._note(runner.cache.groups[group], slot, i, table[i])
         return damage
 
     check_logits(run(lambda runner: None), weights, cfg, ids, dtype)

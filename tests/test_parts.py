@@ -701,7 +701,7 @@ class LatentMixer(Mixer):
         if writes_cache:
             latent[slots // P, slots % P] = c
             stamp[slots // P, slots % P] = meta.positions
-        table = meta.groups[cache.group].block_table.long()
+        table = meta.groups[cache.group].block_table.long()[meta.table_rows.long()]       # each request's own row
         out = torch.empty(x.shape[0], self.hidden, dtype=torch.float32, device=x.device)
         cu, positions = meta.cu_q.tolist(), meta.positions.tolist()          # the host waits here: not capturable
         for b in range(meta.num_requests):

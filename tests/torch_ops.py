@@ -66,6 +66,8 @@ class TorchOps(Ops):
         q_all = qkv.view(T, num_heads + 2 * num_kv_heads, head_dim)[:, :num_heads].float()
         out = torch.zeros(T, num_heads, head_dim, dtype=torch.float32, device=qkv.device)
         table = meta.groups[group].block_table.long()
+        if meta.table_rows is not None:
+            table = table[meta.table_rows.long()]
         cu = meta.cu_q.tolist()
         rep = num_heads // num_kv_heads
         for b in range(meta.num_requests):
