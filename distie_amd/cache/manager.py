@@ -152,6 +152,21 @@ class CacheManager:
         self._requests: Dict[Hashable, RequestCache] = {}
         self.table_width = 0
 
+    @staticmethod
+    def page_bytes(requirements: Sequence, block_size: int, dtype=torch.float32) -> int:
+        """What one more page costs, over all layers and tensors (each group holds a page of its own for
+        every page of the pool)."""
+        total = 0
+        for needs in requirements:
+            for need in (needs.values() if isinstance(needs, dict) else [needs]):
+                if isinstance(need, PagedTensors):
+                    for decl in need.tensors:
+                        count = 1
+                        for size in need.page_shape(decl, block_size):
+                            count *= size
+                        total += count * torch.empty((), dtype=decl.dtype or dtype).element_size()
+        return total
+
     # ---------------------------------------------------------------- block tables on the device
     def bind_tables(self, width: int) -> None:
         """Make the device tables, `width` entries a request (once; the step function's builder calls this with

@@ -35,6 +35,10 @@ def _engine_options(parser: argparse.ArgumentParser) -> None:
     parser.add_argument("--no-packed-weights", action="store_true",
                         help="no second copy of the weights in the matrix cores' order (half the weight memory, "
                              "slower decode)")
+    parser.add_argument("--packed-weights", default=None, metavar="ROLES",
+                        help="packed copies only for these products, comma-separated: qkv,attn_out,gate_up,down,head")
+    parser.add_argument("--gpu-mem-fraction", type=float, default=None,
+                        help="without --num-blocks: pages of the cache until this share of the card's memory is in use")
     parser.add_argument("--tune-products", action="store_true",
                         help="at start, let the library time its kernels for the products of a full portion")
 
@@ -46,7 +50,9 @@ def _build(args):
     engine = EngineConfig.from_env(
         dtype=args.dtype, block_size=args.block_size, num_blocks=args.num_blocks, max_seqs=args.max_seqs,
         token_budget=args.token_budget, use_graphs=False if args.no_decode_graphs else None,
-        step_stats=args.step_stats, seed=args.seed, packed_weights=False if args.no_packed_weights else None,
+        step_stats=args.step_stats, seed=args.seed, packed_weights=False if args.no_packed_weights else (
+            tuple(r for r in args.packed_weights.split(",") if r) if args.packed_weights else None),
+        gpu_mem_fraction=args.gpu_mem_fraction,
         tune_products=True if args.tune_products else None)
     config = json.loads(args.config_json.read_text()) if args.config_json else None
     if args.model is None and config is None:

@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import os
 from dataclasses import dataclass, replace
-from typing import Optional
+from typing import Optional, Tuple, Union
 
 DTYPE_NAMES = {
     "fp32": "float32", "float32": "float32", "float": "float32",
@@ -37,11 +37,16 @@ class EngineConfig:
     block_size: int = DEFAULT_BLOCK_SIZE
     num_blocks: Optional[int] = None        # pages of the cache; None = from max_cache_tokens or the default
     max_cache_tokens: Optional[int] = None  # pool made for this many cached tokens
+    # with neither of the two: pages until this share of the card's memory is in use (weights and their packed
+    # copies included); what stays outside holds a full portion's activations, the library's workspaces and the graphs
+    gpu_mem_fraction: Optional[float] = None
     max_seqs: int = DEFAULT_MAX_SEQS
     token_budget: int = DEFAULT_TOKEN_BUDGET
     max_model_len: Optional[int] = None     # None = the model's max positions
     use_graphs: bool = True
-    packed_weights: bool = True             # a second copy of the weights in the matrix cores' order, for decode
+    # a second copy of the weights in the matrix cores' order, for decode: True, False, or the roles that get one
+    # ("qkv", "attn_out", "gate_up", "down", "head")
+    packed_weights: Union[bool, Tuple[str, ...]] = True
     lookahead: bool = True                  # launch the next decode step before this step's tokens reach the host
     tune_products: bool = False             # at start, let the library time its kernels for a full portion's products
     step_stats: int = 0
@@ -53,12 +58,29 @@ class EngineConfig:
             raise ValueError("block_size, max_seqs and token_budget must be >= 1")
         if self.num_blocks is not None and self.num_blocks < 1:
             raise ValueError("num_blocks must be >= 1")
+        if self.gpu_mem_fraction is not None and not 0.0 < self.gpu_mem_fraction <= 1.0:
+            raise ValueError("gpu_mem_fraction must be in (0, 1]")
+        if not isinstance(self.packed_weights, bool):
+            object.__setattr__(self, "packed_weights", tuple(self.packed_weights))
 
-    def pages(self) -> int:
+    def pages(self, page_bytes: Optional[int] = None, free_bytes: Optional[int] = None,
+              total_bytes: Optional[int] = None) -> int:
+        """Pages of the cache. `page_bytes` (what one more page costs over all layers), `free_bytes` and
+        `total_bytes` (of the card, with the weights in place) are needed only for `gpu_mem_fraction`."""
         if self.num_blocks is not None:
             return self.num_blocks
         if self.max_cache_tokens is not None:
             return max(1, -(-self.max_cache_tokens // self.block_size))
+        if self.gpu_mem_fraction is not None:
+            if not page_bytes or free_bytes is None or total_bytes is None:
+                raise ValueError("gpu_mem_fraction needs the card's free and total memory and the bytes of a page")
+            room = free_bytes - int((1.0 - self.gpu_mem_fraction) * total_bytes)
+            pages = room // page_bytes - 1                    # one page more than the pool hands out is kept
+            if pages < 1:
+                raise ValueError(
+                    f"gpu_mem_fraction={self.gpu_mem_fraction}: {free_bytes / 2**30:.1f} GiB of "
+                    f"{total_bytes / 2**30:.1f} GiB are free, which leaves no room for a page of {page_bytes} bytes")
+            return int(pages)
         return DEFAULT_NUM_BLOCKS
 
     @classmethod
@@ -82,6 +104,9 @@ class EngineConfig:
         raw = os.getenv("WORKER_DECODE_GRAPHS", "").strip().lower()
         if raw:
             env["use_graphs"] = raw not in {"0", "false", "no", "off"}
+        raw = os.getenv("WORKER_GPU_MEM_FRACTION", "").strip()
+        if raw:
+            env["gpu_mem_fraction"] = float(raw)
         raw = os.getenv("WORKER_STEP_STATS", "").strip()
         if raw:
             env["step_stats"] = int(raw)

@@ -97,7 +97,14 @@ class LLM:
         spec = self.model.spec
         ec = self.engine_config
         self.max_model_len = min(ec.max_model_len or spec.max_positions, spec.max_positions)
-        self.cache = CacheManager(self.model.cache_requirements(), ec.block_size, ec.pages(), ec.max_seqs,
+        self.model.prepare(ops)                      # packed copies of the weights: in place before memory is counted
+        needs = self.model.cache_requirements()
+        free = total = None
+        if ec.gpu_mem_fraction is not None and ops.device.type == "cuda":
+            torch.cuda.empty_cache()
+            free, total = torch.cuda.mem_get_info(ops.device)
+        self.num_pages = ec.pages(CacheManager.page_bytes(needs, ec.block_size, self.dtype), free, total)
+        self.cache = CacheManager(needs, ec.block_size, self.num_pages, ec.max_seqs,
                                   device=ops.device, dtype=self.dtype)
         self.runner = ModelRunner(self.model, self.cache, ops, self.dtype, self.max_model_len)
         self.scheduler = Scheduler(self.cache, ec.max_seqs, ec.token_budget, self.max_model_len)
@@ -121,7 +128,7 @@ class LLM:
         if ec.tune_products and hasattr(ops, "tune_library_products"):
             self._tune_products()
         _log.info("engine ready: %s dtype=%s pages=%d x %d tokens, %d cache groups, %.1f MiB cache",
-                  spec.architecture, ec.dtype, ec.pages(), ec.block_size, len(self.cache.groups),
+                  spec.architecture, ec.dtype, self.num_pages, ec.block_size, len(self.cache.groups),
                   self.cache.bytes() / 2 ** 20)
 
     def _tune_products(self) -> None:

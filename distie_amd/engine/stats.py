@@ -109,3 +109,20 @@ class StepStats:
         if self._kinds:
             _log.info("step stats %s", self.format())
             self._kinds.clear()
+
+
+def distribution_ms(seconds) -> dict:
+    """Mean, median, 90th and 99th percentile and maximum of times given in seconds, in milliseconds; a
+    percentile between two samples is interpolated linearly (the reference's load generator reports
+    latencies this way: benchmarks/load/stats.py:42-64)."""
+    samples = sorted(1e3 * float(s) for s in seconds)
+    if not samples:
+        return {}
+
+    def at(share: float) -> float:
+        place = share * (len(samples) - 1)
+        below = int(place)
+        above = min(below + 1, len(samples) - 1)
+        return samples[below] + (place - below) * (samples[above] - samples[below])
+
+    return {"mean": sum(samples) / len(samples), "p50": at(0.5), "p90": at(0.9), "p99": at(0.99), "max": samples[-1]}

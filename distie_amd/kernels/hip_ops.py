@@ -142,14 +142,20 @@ class HipOps(Ops):
     DECODE_WAVES = 1024
     DECODE_MAX_RUNS = 256
 
-    def __init__(self, device="cuda:0", packed_weights: bool = True) -> None:
-        """`packed_weights`: keep a second copy of every bfloat16 weight in the order in which the
+    def __init__(self, device="cuda:0", packed_weights=True) -> None:
+        """`packed_weights` (True, False, or the roles that get one, as the parts name them in
+        `prepare_linear`: "qkv", "attn_out", "gate_up", "down", "head"): keep a second copy of every bfloat16 weight in the order in which the
         matrix cores take it, for products with at most `PACKED_MAX_ROWS_EAGER` rows (decode, short portions). It doubles
         the memory of the weights and makes those products 15-25 % faster, and it is what the fused
         epilogues (activation, rotation and cache write) work on; without it products of up to
         `SKINNY_MAX_ROWS` rows stream the weights as they are stored and larger ones go to the library."""
         self.device = torch.device(device)
-        self.packed_weights = bool(packed_weights)
+        if isinstance(packed_weights, (bool, int)) or packed_weights is None:
+            self.packed_weights = bool(packed_weights)
+            self.packed_roles = None
+        else:
+            self.packed_roles = frozenset(packed_weights)
+            self.packed_weights = bool(self.packed_roles)
         if self.device.type != "cuda" or not torch.cuda.is_available():
             raise KernelError("HipOps needs an AMD GPU (torch.cuda is not available): there is no CPU path")
         name = torch.cuda.get_device_properties(self.device).gcnArchName
@@ -394,7 +400,9 @@ class HipOps(Ops):
         row_blocks = -(-(N // 2) // 8) if gated else -(-N // 16)
         return row_blocks * -(-K // 32) * 512
 
-    def prepare_linear(self, weight, gated=False, rotary=None):
+    def prepare_linear(self, weight, gated=False, rotary=None, role=None):
+        if self.packed_roles is not None and role not in self.packed_roles:
+            return
         if not self.packed_weights or weight.dtype != torch.bfloat16 or weight.dim() != 2 or weight.shape[1] % 8:
             return
         N, K = weight.shape

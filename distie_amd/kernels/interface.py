@@ -99,10 +99,11 @@ class Ops(abc.ABC):
         tensor as it is. For parts that compute on a product's values themselves."""
         return x
 
-    def prepare_linear(self, weight: torch.Tensor, gated: bool = False, rotary=None) -> None:
+    def prepare_linear(self, weight: torch.Tensor, gated: bool = False, rotary=None, role: Optional[str] = None) -> None:
         """Called once for every weight of a `linear` after it is loaded (`gated`: the weight of a
         `linear_silu_mul`; `rotary = (num_heads, num_kv_heads, head_dim)`: the stacked q/k/v weight
-        of a `linear_rope_kv_write`). An implementation may build what its products need beside
+        of a `linear_rope_kv_write`; `role`: what the part calls this product, so that a setting
+        can name it). An implementation may build what its products need beside
         the tensor (the HIP kernels keep a second copy in the matrix cores' order for small
         batches)."""
 

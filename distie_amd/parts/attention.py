@@ -94,8 +94,9 @@ class Attention(Mixer):
         self.position.to_device(self.out_weight.device)
 
     def prepare(self, ops) -> None:
-        ops.prepare_linear(self.qkv_weight, rotary=(self.num_heads, self.num_kv_heads, self.head_dim))
-        ops.prepare_linear(self.out_weight)
+        ops.prepare_linear(self.qkv_weight, rotary=(self.num_heads, self.num_kv_heads, self.head_dim),
+                           role="qkv")
+        ops.prepare_linear(self.out_weight, role="attn_out")
 
     def capture_context(self, longest: int, limit: int):
         """Decode attention cuts the keys into runs by the longest context of the step, and that number is

@@ -46,7 +46,7 @@ class LinearHead(Head):
         self.weight = tensors["weight"] if self.tied_to else tensors["weight"].contiguous()
 
     def prepare(self, ops) -> None:
-        ops.prepare_linear(self.weight)
+        ops.prepare_linear(self.weight, role="head")
 
     def forward(self, ops, normed):
         return ops.linear_f32out(normed, self.weight)

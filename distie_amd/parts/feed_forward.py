@@ -30,8 +30,8 @@ class SwiGLU(FeedForward):
         self.down_weight = tensors["down_proj.weight"].contiguous()
 
     def prepare(self, ops) -> None:
-        ops.prepare_linear(self.gate_up_weight, gated=True)
-        ops.prepare_linear(self.down_weight)
+        ops.prepare_linear(self.gate_up_weight, gated=True, role="gate_up")
+        ops.prepare_linear(self.down_weight, role="down")
 
     def forward(self, ops, x, ctx):
         return ops.linear(ops.linear_silu_mul(x, self.gate_up_weight), self.down_weight)

@@ -76,6 +76,16 @@ def test_groups_by_need():
     assert m.layer(0)["mixer"].group == 0 and m.layer(1)["mixer"].group == 1 and m.layer(3)["mixer"].group == -1
 
 
+def test_page_bytes_counts_every_layer_and_tensor():
+    needs = [PagedKV(2, 16), PagedKV(2, 16, 6), PagedKV(2, 16), None, FixedState.of((3,))]
+    m = CacheManager(needs, 4, 12, 4)
+    per_page = CacheManager.page_bytes(needs, m.block_size, torch.float32)
+    paged = sum(t.numel() * t.element_size() for g in m.groups for t in g.tensors.values())
+    assert per_page * (m.num_blocks + 1) == paged
+    assert CacheManager.page_bytes(needs, m.block_size, torch.bfloat16) * 2 == per_page
+    assert CacheManager.page_bytes([None, FixedState.of((3,))], 4) == 0
+
+
 def test_reserve_commit_release_and_window():
     m = manager(block=4, pages=12, window=6)
     m.add("a")

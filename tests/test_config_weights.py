@@ -78,6 +78,38 @@ def test_engine_config():
         EngineConfig(token_budget=0)
 
 
+def test_cache_sized_from_the_cards_memory():
+    """Pages until the given share of the card is in use: the free memory minus what must stay free, in
+    pages, less the one page that the cache keeps beyond the pool."""
+    gib = 2 ** 30
+    config = EngineConfig(gpu_mem_fraction=0.75)
+    assert config.pages(page_bytes=gib, free_bytes=60 * gib, total_bytes=100 * gib) == 60 - 25 - 1
+    assert EngineConfig(gpu_mem_fraction=1.0).pages(page_bytes=3 * gib, free_bytes=10 * gib, total_bytes=64 * gib) == 2
+    assert EngineConfig(gpu_mem_fraction=0.5, num_blocks=7).pages() == 7          # a given size wins
+    with pytest.raises(ValueError, match="no room"):
+        config.pages(page_bytes=gib, free_bytes=25 * gib, total_bytes=100 * gib)
+    with pytest.raises(ValueError, match="needs the card"):
+        config.pages()
+    for bad in (0.0, 1.5, -1.0):
+        with pytest.raises(ValueError):
+            EngineConfig(gpu_mem_fraction=bad)
+    assert EngineConfig(packed_weights=["qkv", "head"]).packed_weights == ("qkv", "head")
+
+
+def test_latency_distribution_matches_numpy():
+    import numpy as np
+
+    from distie_amd.engine.stats import distribution_ms
+
+    values = torch.rand(37, generator=torch.Generator().manual_seed(3)).double().numpy()
+    got = distribution_ms(values)
+    for key, q in (("p50", 50), ("p90", 90), ("p99", 99)):
+        assert abs(got[key] - np.percentile(values * 1e3, q)) < 1e-9
+    assert abs(got["mean"] - values.mean() * 1e3) < 1e-9 and got["max"] == values.max() * 1e3
+    assert distribution_ms([0.25]) == {"mean": 250.0, "p50": 250.0, "p90": 250.0, "p99": 250.0, "max": 250.0}
+    assert distribution_ms([]) == {}
+
+
 def test_safetensors_round_trip_matches_the_library(tmp_path):
     from safetensors.torch import load_file, save_file
 

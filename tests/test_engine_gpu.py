@@ -49,19 +49,30 @@ def test_prompt_then_last_32_one_by_one(setup, ops):
     check_logits(replay_cut(runner, "a", ids, [88]), weights, cfg, ids, dtype, folder)
 
 
-def test_without_packed_weights(setup):
+@pytest.mark.parametrize("packed", [False, ("qkv", "down"), ("gate_up", "attn_out", "head")],
+                         ids=["none", "qkv+down", "gate_up+attn_out+head"])
+def test_without_packed_weights(setup, packed):
     """The products on the stored layout (no second copy of the weights), rotation and activation as
-    kernels of their own: the same requests, the same bounds."""
+    kernels of their own, for every weight or for some: the same requests, the same bounds."""
     from distie_amd.kernels.hip_ops import HipOps
 
     cfg, block, folder, weights, dtype = setup
-    plain_ops = HipOps("cuda:0", packed_weights=False)
+    plain_ops = HipOps("cuda:0", packed_weights=packed)
     runner = build_runner(folder, plain_ops, dtype, block_size=block)
     ids = random_ids(cfg, 120, 2)
     check_logits(replay_cut(runner, "a", ids, [40, 20, 17, 11]), weights, cfg, ids, dtype, folder)
-    tensors = [t for b in runner.model.blocks for part in (b.mixer, b.feed_forward) for t in vars(part).values()
-               if isinstance(t, torch.Tensor)] + [runner.model.head]
-    assert not any(hasattr(t, name) for t in tensors for name in ("_distie_packed", "_distie_gated", "_distie_rotary"))
+    copies = ("_distie_packed", "_distie_gated", "_distie_rotary")
+    has = lambda t: any(hasattr(t, name) for name in copies)
+    wanted = set(packed or ())
+    by_role = {"qkv": [b.mixer.qkv_weight for b in runner.model.blocks],
+               "attn_out": [b.mixer.out_weight for b in runner.model.blocks],
+               "gate_up": [b.feed_forward.gate_up_weight for b in runner.model.blocks],
+               "down": [b.feed_forward.down_weight for b in runner.model.blocks],
+               "head": [runner.model.head]}
+    for role, tensors in by_role.items():
+        # bfloat16 weights with rows of whole 16-byte pieces get the copy where it is asked for; others never
+        for t in tensors:
+            assert has(t) == (role in wanted and dtype == torch.bfloat16 and t.shape[1] % 8 == 0), role
 
 
 @pytest.mark.parametrize("cuts", [[2, 3, 5, 7, 2, 11, 4, 33, 2, 2, 19], [64, 2, 2, 2, 30], [1, 1, 2, 70, 9]])
