@@ -1,9 +1,10 @@
 """Building and finding the native libraries.
 
-Three kinds of shared library, all built from the sources beside this file:
+Four kinds of shared library, all built from the sources beside this file:
 
 * `core`  - the id pool of the cache manager (C++, host only, g++);
 * `ops`   - the HIP kernels that do not depend on the head size (hipcc, gfx950);
+* `library` - the calls of the vendor's matrix-product library for large products (hipcc, linked with hipBLASLt);
 * `attn_d<D>` - the attention kernels for head size D (hipcc, `-DDISTIE_HEAD_DIM=D`; the matrix-core
   kernels for multiples of 16, the wave-per-token kernel for every even size).
 
@@ -37,6 +38,8 @@ CXX_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-pthread"]
 
 OPS_SOURCES = ["elementwise.hip", "gemm.hip", "gemv.hip", "decode_products.hip", "sampling.hip"]
 ATTN_SOURCES = ["attention.hip"]
+LIBRARY_SOURCES = ["library_products.hip"]
+LINK_LIBS = {"library": ["-lhipblaslt"]}
 HEADERS = ["common.h"]
 OPS_HEADERS = ["no_alloc.h", "packed.h"]
 
@@ -67,6 +70,8 @@ def _spec(name: str):
         return ["block_pool.cpp"], os.environ.get("CXX", "g++"), list(CXX_FLAGS)
     if name == "ops":
         return list(OPS_SOURCES), _hipcc(), list(HIP_FLAGS)
+    if name == "library":
+        return list(LIBRARY_SOURCES), _hipcc(), list(HIP_FLAGS)
     if name.startswith("attn_d"):
         dim = int(name[len("attn_d"):])
         if dim < 2 or dim > 256 or dim % 2:
@@ -167,7 +172,10 @@ def build(name: str, force: bool = False) -> Path:
         objects = [str(scratch / (Path(s).stem + ".o")) for s in sources]
         link_flags = [f for f in flags if not f.startswith("-D")]
         staging = scratch / target.name
-        _run([compiler] + link_flags + ["-shared"] + objects + ["-o", str(staging)], f"{name} (link)")
+        libs = LINK_LIBS.get(name, [])
+        if libs:
+            libs = [f"-L{Path(compiler).resolve().parent.parent / 'lib'}"] + libs
+        _run([compiler] + link_flags + ["-shared"] + objects + libs + ["-o", str(staging)], f"{name} (link)")
         os.replace(staging, target)
     finally:
         shutil.rmtree(scratch, ignore_errors=True)
@@ -191,7 +199,7 @@ DEFAULT_HEAD_DIMS = (16, 32, 40, 48, 64, 80, 96, 112, 128, 256)
 
 
 def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True) -> List[Path]:
-    out = [build("core", force), build("ops", force)]
+    out = [build("core", force), build("ops", force), build("library", force)]
     for d in head_dims:
         out.append(build(f"attn_d{d}", force))
     return out

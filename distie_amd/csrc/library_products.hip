@@ -1,0 +1,198 @@
+// Large matrix products through hipBLASLt, with the plan of every shape kept: y[M, N] = x[M, K] . W[N, K]^T
+// (+ bias), bfloat16 operands, float32 sums, y in bfloat16 or float32 with rows `ldy` elements apart.
+//
+// The reference leaves these products to its library as well (torch.nn.functional.linear on cuBLAS:
+// worker/src/inference/qwen2/model.py:60-75). Calling the library from here instead of through torch saves
+// most of the host time of a call (descriptors and the choice of kernel are made once per shape), lets the
+// output be a column block of a wider matrix, adds the bias in float32, and lets the engine time the library's
+// candidate kernels itself for the shapes of a full portion.
+//
+// One device per process, one caller at a time (a mutex guards the table of plans). Nothing here allocates
+// after `distie_lib_init`, so a call can be recorded into a graph once its shape has been seen.
+#include "common.h"
+
+#include <hipblaslt/hipblaslt.h>
+
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#define DISTIE_LIB_UNSUPPORTED (-3)      // the library offers no kernel for this product: the caller takes another way
+#define DISTIE_LIB_NOT_READY (-4)
+
+namespace {
+
+constexpr size_t WORKSPACE_BYTES = size_t(128) << 20;
+constexpr int CANDIDATES = 16;
+constexpr int TIMED_RUNS = 4;
+
+struct Key {
+  int M, N, K, y_dtype, bias;
+  int64_t ldy;
+  bool operator==(const Key& o) const {
+    return M == o.M && N == o.N && K == o.K && y_dtype == o.y_dtype && bias == o.bias && ldy == o.ldy;
+  }
+};
+struct KeyHash {
+  size_t operator()(const Key& k) const {
+    uint64_t h = 1469598103934665603ull;
+    for (uint64_t v : {uint64_t(k.M), uint64_t(k.N), uint64_t(k.K), uint64_t(k.y_dtype), uint64_t(k.bias), uint64_t(k.ldy)}) {
+      h ^= v;
+      h *= 1099511628211ull;
+    }
+    return size_t(h);
+  }
+};
+struct Plan {
+  hipblasLtMatmulDesc_t product = nullptr;
+  hipblasLtMatrixLayout_t w = nullptr, x = nullptr, y = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+  bool timed = false;
+};
+
+std::mutex guard;
+hipblasLtHandle_t handle = nullptr;
+void* workspace = nullptr;
+int device_of_handle = -1;
+std::unordered_map<Key, Plan, KeyHash> plans;
+long plans_made = 0, plans_timed = 0;
+
+bool ok(hipblasStatus_t s) { return s == HIPBLAS_STATUS_SUCCESS; }
+
+void drop(Plan& p) {
+  if (p.product) hipblasLtMatmulDescDestroy(p.product);
+  if (p.w) hipblasLtMatrixLayoutDestroy(p.w);
+  if (p.x) hipblasLtMatrixLayoutDestroy(p.x);
+  if (p.y) hipblasLtMatrixLayoutDestroy(p.y);
+  p = Plan();
+}
+
+// In the library's column-major terms: y^T [N x M, ld ldy] = W^T (stored K x N, ld K, transposed) . x^T (stored K x M, ld K).
+int make_plan(const Key& key, Plan& plan, std::vector<hipblasLtMatmulHeuristicResult_t>& found) {
+  const hipDataType out_type = key.y_dtype == DISTIE_F32 ? HIP_R_32F : HIP_R_16BF;
+  if (!ok(hipblasLtMatmulDescCreate(&plan.product, HIPBLAS_COMPUTE_32F, HIP_R_32F))) return DISTIE_LIB_UNSUPPORTED;
+  const int32_t transposed = HIPBLAS_OP_T, plain = HIPBLAS_OP_N;
+  bool fine = ok(hipblasLtMatmulDescSetAttribute(plan.product, HIPBLASLT_MATMUL_DESC_TRANSA, &transposed, sizeof(transposed))) &&
+              ok(hipblasLtMatmulDescSetAttribute(plan.product, HIPBLASLT_MATMUL_DESC_TRANSB, &plain, sizeof(plain)));
+  if (fine && key.bias) {
+    const uint32_t epilogue = HIPBLASLT_EPILOGUE_BIAS;
+    const int32_t bias_type = HIP_R_32F;
+    fine = ok(hipblasLtMatmulDescSetAttribute(plan.product, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue))) &&
+           ok(hipblasLtMatmulDescSetAttribute(plan.product, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type)));
+  }
+  fine = fine && ok(hipblasLtMatrixLayoutCreate(&plan.w, HIP_R_16BF, key.K, key.N, key.K)) &&
+         ok(hipblasLtMatrixLayoutCreate(&plan.x, HIP_R_16BF, key.K, key.M, key.K)) &&
+         ok(hipblasLtMatrixLayoutCreate(&plan.y, out_type, key.N, key.M, key.ldy));
+  if (!fine) return DISTIE_LIB_UNSUPPORTED;
+  hipblasLtMatmulPreference_t preference = nullptr;
+  if (!ok(hipblasLtMatmulPreferenceCreate(&preference))) return DISTIE_LIB_UNSUPPORTED;
+  const uint64_t room = WORKSPACE_BYTES;
+  hipblasLtMatmulPreferenceSetAttribute(preference, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &room, sizeof(room));
+  found.assign(CANDIDATES, hipblasLtMatmulHeuristicResult_t());
+  int count = 0;
+  const hipblasStatus_t s = hipblasLtMatmulAlgoGetHeuristic(handle, plan.product, plan.w, plan.x, plan.y, plan.y, preference,
+                                                            CANDIDATES, found.data(), &count);
+  hipblasLtMatmulPreferenceDestroy(preference);
+  if (!ok(s) || count <= 0) return DISTIE_LIB_UNSUPPORTED;
+  found.resize(count);
+  plan.algo = found[0].algo;
+  return 0;
+}
+
+hipblasStatus_t run(const Plan& plan, const hipblasLtMatmulAlgo_t& algo, const void* x, const void* w, const void* bias,
+                    void* y, hipStream_t stream) {
+  const float one = 1.f, zero = 0.f;
+  if (bias != nullptr &&
+      !ok(hipblasLtMatmulDescSetAttribute(plan.product, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias))))
+    return HIPBLAS_STATUS_INVALID_VALUE;
+  return hipblasLtMatmul(handle, plan.product, &one, w, plan.w, x, plan.x, &zero, y, plan.y, y, plan.y, &algo, workspace,
+                         WORKSPACE_BYTES, stream);
+}
+
+}  // namespace
+
+// Once per process, with the device current: the library's handle and its workspace (128 MiB, kept until the
+// process ends).
+extern "C" int distie_lib_init(int device) {
+  std::lock_guard<std::mutex> lock(guard);
+  if (handle != nullptr) return device == device_of_handle ? 0 : DISTIE_BAD_ARGUMENT;
+  hipError_t e = hipSetDevice(device);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (!ok(hipblasLtCreate(&handle))) {
+    handle = nullptr;
+    return DISTIE_LIB_NOT_READY;
+  }
+  e = hipMalloc(&workspace, WORKSPACE_BYTES);
+  if (e != hipSuccess) {
+    hipblasLtDestroy(handle);
+    handle = nullptr;
+    return static_cast<int>(e);
+  }
+  device_of_handle = device;
+  return 0;
+}
+
+// plans made, and plans whose kernel was chosen by timing
+extern "C" void distie_lib_counts(long* made, long* timed) {
+  std::lock_guard<std::mutex> lock(guard);
+  *made = plans_made;
+  *timed = plans_timed;
+}
+
+// y = x . W^T (+ bias). `bias`: float32 [N] or null. `tune` != 0: a shape not yet timed has the library's candidate
+// kernels run TIMED_RUNS times each on `stream` (which is waited for: not inside a capture) and keeps the fastest;
+// otherwise a new shape takes the library's first choice. The output is written by every candidate run, each
+// time with the whole result.
+extern "C" int distie_lib_linear(const void* x, const void* w, const void* bias, void* y, int y_dtype, int M, int N, int K,
+                                 int64_t ldy, int tune, hipStream_t stream) {
+  if (M < 1 || N < 1 || K < 1 || ldy < N || (y_dtype != DISTIE_F32 && y_dtype != DISTIE_BF16) || x == nullptr ||
+      w == nullptr || y == nullptr)
+    return DISTIE_BAD_ARGUMENT;
+  std::lock_guard<std::mutex> lock(guard);
+  if (handle == nullptr) return DISTIE_LIB_NOT_READY;
+  const Key key{M, N, K, y_dtype, bias != nullptr ? 1 : 0, ldy};
+  auto it = plans.find(key);
+  std::vector<hipblasLtMatmulHeuristicResult_t> found;
+  if (it == plans.end() || (tune && !it->second.timed)) {
+    Plan fresh;
+    const int made = make_plan(key, fresh, found);
+    if (made != 0) {
+      drop(fresh);
+      return made;
+    }
+    if (it != plans.end()) {
+      drop(it->second);
+      it->second = fresh;
+    } else {
+      it = plans.emplace(key, fresh).first;
+      ++plans_made;
+    }
+    if (tune) {
+      hipEvent_t begin, end;
+      if (hipEventCreate(&begin) != hipSuccess || hipEventCreate(&end) != hipSuccess) return DISTIE_LIB_NOT_READY;
+      float best = -1.f;
+      for (const auto& candidate : found) {
+        if (!ok(run(it->second, candidate.algo, x, w, bias, y, stream))) continue;      // a warm-up, and a check
+        hipEventRecord(begin, stream);
+        bool all = true;
+        for (int r = 0; r < TIMED_RUNS; ++r) all = all && ok(run(it->second, candidate.algo, x, w, bias, y, stream));
+        hipEventRecord(end, stream);
+        if (hipEventSynchronize(end) != hipSuccess || !all) continue;
+        float ms = 0.f;
+        hipEventElapsedTime(&ms, begin, end);
+        if (best < 0.f || ms < best) {
+          best = ms;
+          it->second.algo = candidate.algo;
+        }
+      }
+      hipEventDestroy(begin);
+      hipEventDestroy(end);
+      if (best < 0.f) return DISTIE_LIB_UNSUPPORTED;
+      it->second.timed = true;
+      ++plans_timed;
+    }
+  }
+  const hipblasStatus_t s = run(it->second, it->second.algo, x, w, bias, y, stream);
+  if (!ok(s)) return DISTIE_LIB_UNSUPPORTED;
+  return launch_status();
+}

@@ -162,6 +162,9 @@ class HipOps(Ops):
         if not name.startswith("gfx950"):
             raise KernelError(f"the kernels are built for gfx950 (MI355X); this device is {name}")
         self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        self._compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
+        self._lib = None
+        self._tuning = False
         self._ops = ctypes.CDLL(str(build.ensure("ops")))
         self._declare()
         self._attn: Dict[int, ctypes.CDLL] = {}
@@ -223,23 +226,11 @@ class HipOps(Ops):
         o.distie_sample.argtypes = [_P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P]
 
     def tune_library_products(self, on: bool) -> None:
-        """While on, the library times its candidate kernels for every new shape of a large product and
-        keeps the fastest; afterwards it uses what it found (its own choice for shapes it has not
-        seen). Products of up to `PACKED_MAX_ROWS` rows do not go to the library at all (`PACKED_MAX_ROWS_EAGER`
+        """While on, every new shape of a large product has the library's candidate kernels timed, and the
+        fastest is kept for that shape from then on; shapes first met while off take the library's first choice.
+        Products of up to `PACKED_MAX_ROWS` rows do not go to the library at all (`PACKED_MAX_ROWS_EAGER`
         outside captured steps)."""
-        import os
-        import tempfile
-
-        try:
-            import torch.cuda.tunable as tunable
-        except ImportError:           # a torch without it: the library's own choice stands
-            return
-        if on:
-            # the library insists on a results file: keep it out of the working directory
-            folder = tempfile.mkdtemp(prefix=f"distie_tune_{os.getuid()}_")
-            tunable.set_filename(os.path.join(folder, "results.csv"))
-        tunable.enable(True)
-        tunable.tuning_enable(bool(on))
+        self._tuning = bool(on)
 
     def graphs_supported(self) -> bool:
         """Every kernel launches on torch's current stream and keeps its scratch at fixed
@@ -538,6 +529,74 @@ class HipOps(Ops):
     def _packed_rows(self) -> int:
         return self.PACKED_MAX_ROWS if self.captured else self.PACKED_MAX_ROWS_EAGER
 
+    def _library(self):
+        """The vendor library's products, called directly; loaded at the first large product."""
+        if self._lib is None:
+            lib = ctypes.CDLL(str(build.ensure("library")))
+            lib.distie_lib_init.argtypes = [ctypes.c_int]
+            lib.distie_lib_init.restype = ctypes.c_int
+            lib.distie_lib_linear.argtypes = [_P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                              ctypes.c_int64, ctypes.c_int, _P]
+            lib.distie_lib_linear.restype = ctypes.c_int
+            lib.distie_lib_counts.argtypes = [ctypes.POINTER(ctypes.c_long), ctypes.POINTER(ctypes.c_long)]
+            lib.distie_lib_counts.restype = None
+            with torch.cuda.device(self.device):
+                _check(lib.distie_lib_init(self._device_index), "lib_init")
+            self._lib = lib
+        return self._lib
+
+    def library_plans(self):
+        """(shapes the library has a plan for, shapes whose kernel was chosen by timing)"""
+        made, timed = ctypes.c_long(0), ctypes.c_long(0)
+        self._library().distie_lib_counts(ctypes.byref(made), ctypes.byref(timed))
+        return made.value, timed.value
+
+    LIBRARY_UNSUPPORTED = -3
+
+    def _library_linear(self, x, weight, bias, out_dtype):
+        """x [M, K] . weight [N, K]^T (+ float32 bias) by the library, float32 sums, into a new [M, N] of `out_dtype`."""
+        M, K = x.shape
+        N = weight.shape[0]
+        if x.stride(1) != 1 or x.stride(0) != K:
+            x = x.contiguous()
+        if weight.stride(1) != 1 or weight.stride(0) != K:
+            weight = weight.contiguous()
+        out = torch.empty((M, N), dtype=out_dtype, device=self.device)
+        lib = self._library()
+        code, size = _CODES[out_dtype], out.element_size()
+        # The library's large kernels work on tiles of 256 x 256, one a compute unit at a time: a product with a
+        # few tiles more than a whole number of rounds pays a full round for them (at 2,048 rows 16,384 columns
+        # take 82 us and 17,920 take 116). The last columns as a product of their own cost less (20 us for
+        # 1,536), written into the same output.
+        tail = self._library_tail(M, N) if out_dtype == torch.bfloat16 else 0
+        for lo, hi in (((0, N - tail), (N - tail, N)) if tail else ((0, N),)):
+            rc = lib.distie_lib_linear(
+                x.data_ptr(), weight.data_ptr() + lo * K * 2, bias.data_ptr() + lo * 4 if bias is not None else None,
+                out.data_ptr() + lo * size, code, M, hi - lo, K, N, 1 if self._tuning else 0, self._stream())
+            if rc == self.LIBRARY_UNSUPPORTED:
+                # no kernel of the library's for this product as asked for: through torch, which knows more ways
+                y = torch.mm(x, weight.t(), out_dtype=torch.float32)
+                y = y if bias is None else y + bias
+                return y if out_dtype == torch.float32 else y.to(out_dtype)
+            _check(rc, "lib_linear")
+        return out
+
+    LIBRARY_TILE = 256
+
+    def _library_tail(self, M: int, N: int) -> int:
+        """How many of the last columns of a large library product to run as a product of their own: those
+        beyond the last whole round of tiles over the compute units, if they are few (at most a quarter of a
+        round) and there is at least one whole round before them; else 0."""
+        tile = self.LIBRARY_TILE
+        row_tiles = -(-M // tile)
+        if row_tiles > self._compute_units:
+            return 0
+        round_columns = self._compute_units // row_tiles * tile
+        tail = N % round_columns
+        if N < round_columns or tail == 0 or tail > round_columns // 4 or tail % 8:
+            return 0
+        return tail
+
     def _pass_blocks(self, rows: int, elements: int) -> int:
         """Blocks of 16 rows of x per pass of the wide product over a weight of `elements` (0: one pass)."""
         if elements > self.TWO_PASS_MAX_ELEMENTS:
@@ -618,17 +677,7 @@ class HipOps(Ops):
             return PartialSums(out, out_dtype) if partial_ok else self.dense(PartialSums(out, out_dtype))
         if both_bf16:
             # large bfloat16 product: the library's matrix-core kernels
-            lib_bias = None
-            if bias is not None:
-                # the library adds a bias of the activations' type; keep that copy on the tensor itself
-                lib_bias = getattr(bias, "_distie_bf16", None)
-                if lib_bias is None:
-                    lib_bias = bias._distie_bf16 = bias.to(torch.bfloat16)
-            if out_dtype == torch.float32:
-                # the library writes its float32 sums unrounded (the logits)
-                y = torch.mm(x, weight.t(), out_dtype=torch.float32)
-                return y if bias is None else y + bias
-            return torch.nn.functional.linear(x, weight, lib_bias)
+            return self._library_linear(x, weight, bias, out_dtype)
         out = torch.empty((M, N), dtype=out_dtype, device=self.device)
         if M <= self.ROWS_MAX_ROWS and K % 8 == 0:
             # few rows in float32 (or against a weight kept in float32): the weights are streamed, FMAs only

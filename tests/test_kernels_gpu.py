@@ -415,7 +415,51 @@ def test_partial_sums_are_added_by_their_readers(ops):
 def test_gemm_large_bf16_uses_library_and_matches(ops):
     x, w, b = rand(300, 136, dtype=torch.bfloat16, seed=1), rand(250, 136, dtype=torch.bfloat16, seed=2), rand(250, seed=3)
     want = x.double() @ w.double().T + b.double()
+    before = ops.library_plans()[0]
     close(ops.linear(x, w, b), want, torch.bfloat16, scale=want.abs().max().item())
+    close(ops.linear(x, w), want - b.double(), torch.bfloat16, scale=want.abs().max().item())
+    assert ops.library_plans()[0] == before + 2          # with and without bias: two plans, made once
+    close(ops.linear(x, w, b), want, torch.bfloat16, scale=want.abs().max().item())
+    assert ops.library_plans()[0] == before + 2
+    # the head's product: float32 out, unrounded sums
+    logits = ops.linear_f32out(x, w)
+    assert logits.dtype == torch.float32
+    close(logits, want - b.double(), torch.float32, scale=want.abs().max().item())
+
+
+def test_library_kernels_chosen_by_timing(ops):
+    """With tuning on, a new shape has the library's candidates timed once; the result is the same product."""
+    x, w = rand(512, 264, dtype=torch.bfloat16, seed=4), rand(384, 264, dtype=torch.bfloat16, seed=5)
+    want = x.double() @ w.double().T
+    timed = ops.library_plans()[1]
+    ops.tune_library_products(True)
+    try:
+        got = ops.linear(x, w)
+    finally:
+        ops.tune_library_products(False)
+    assert ops.library_plans()[1] == timed + 1
+    close(got, want, torch.bfloat16, scale=want.abs().max().item())
+    close(ops.linear(x, w), want, torch.bfloat16, scale=want.abs().max().item())
+    assert ops.library_plans()[1] == timed + 1
+
+
+@pytest.mark.parametrize("bias", [False, True])
+def test_gemm_large_bf16_with_a_ragged_last_round(ops, bias, monkeypatch):
+    """A large product whose columns end a little after a whole round of the library's tiles is run as two
+    products into one output; with a tile of 16 (patched) a small case takes that path. The result is the
+    plain product's."""
+    monkeypatch.setattr(type(ops), "LIBRARY_TILE", 16)
+    M = 600
+    round_columns = ops._compute_units // -(-M // 16) * 16
+    N = 2 * round_columns + 24
+    assert ops._library_tail(M, N) == 24 and ops._library_tail(M, 2 * round_columns) == 0
+    assert ops._library_tail(M, round_columns + round_columns // 2) == 0        # many columns left: one product
+    x, w = rand(M, 136, dtype=torch.bfloat16, seed=1), rand(N, 136, dtype=torch.bfloat16, seed=2)
+    b = rand(N, seed=3) if bias else None
+    want = x.double() @ w.double().T + (b.double() if bias else 0)
+    got = ops.linear(x, w, b)
+    assert got.shape == (M, N) and got.is_contiguous()
+    close(got, want, torch.bfloat16, scale=want.abs().max().item())
 
 
 def make_meta(positions, token_request, cu_q, kv_len, tables, slots, block_size):
