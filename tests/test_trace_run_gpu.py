@@ -139,27 +139,29 @@ def test_generation_through_the_entry_point_and_the_command_line(tmp_path):
 
 
 def test_tuned_library_products(tmp_path):
-    """`tune_products`: the engine starts with one full portion while the library times its kernels for
-    the large products; results stay within the bounds, with whatever kernels it picked."""
-    import torch.cuda.tunable as tunable
-
+    """`tune_products`: the engine starts with one full portion while the library's candidate kernels are
+    timed for the large products; afterwards new shapes take the library's first choice. Results stay within
+    the bounds, with whatever kernels were picked."""
     from distie_amd import LLM
     from distie_amd.engine.batch import StepEntry
     from engine_util import check_logits
 
     cfg = plain.TINY_C
     folder, weights = make_model_dir(tmp_path, cfg, seed=5, dtype=torch.bfloat16)
-    try:
-        llm = LLM(folder, dtype="bf16", block_size=16, num_blocks=40, token_budget=200, tune_products=True)
-        assert tunable.is_enabled() and not tunable.tuning_is_enabled()
-        ids = random_ids(cfg, 150, 4)
-        logits = llm.step([StepEntry("a", ids, list(range(len(ids))))]).float().cpu()
-        llm.finish("a")
-        check_logits(logits, weights, cfg, ids, torch.bfloat16, folder)
-        llm.cache.check()
-    finally:
-        tunable.tuning_enable(False)
-        tunable.enable(False)
+    llm = LLM(folder, dtype="bf16", block_size=16, num_blocks=40, token_budget=400, tune_products=True,
+              packed_weights=False)                 # without packed copies 400 rows are the library's
+    made, timed = llm.ops.library_plans()
+    assert timed >= 1 and not llm.ops._tuning       # the full portion's products were timed, and tuning is off again
+    ids = random_ids(cfg, 300, 4)
+    logits = llm.step([StepEntry("a", ids, list(range(len(ids))))]).float().cpu()
+    llm.finish("a")
+    assert llm.ops.library_plans()[1] == timed      # another number of rows: not timed
+    check_logits(logits, weights, cfg, ids, torch.bfloat16, folder)
+    ids = random_ids(cfg, 400, 5)
+    logits = llm.step([StepEntry("b", ids, list(range(len(ids))))]).float().cpu()
+    llm.finish("b")
+    check_logits(logits, weights, cfg, ids, torch.bfloat16, folder)     # the timed shapes
+    llm.cache.check()
 
 
 def test_captured_steps_per_class_of_context_length(tmp_path, monkeypatch):
