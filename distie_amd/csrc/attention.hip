@@ -209,6 +209,206 @@ __global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_generic_kernel(
   }
 }
 
+// The same walk in float32 for requests that decode, with loads that cover whole rows: one workgroup per
+// (token, kv head, part of up to G query heads of it). For the scores eight lanes share a key: each reads an
+// eighth of the key's row of K (a run of D / 8 floats, so a wave's load covers eight whole rows; with a lane
+// to a key every 16-byte load of a wave touched 64 lines) against its slices of the heads' queries, which it
+// keeps in registers; the sums of the eight lanes are added by three exchanges. With G > 1 every row of K
+// and every value of V^T is read once for G heads; the caller takes G as large as leaves enough workgroups.
+constexpr bool GQ_FITS = D % 32 == 0;
+constexpr int GQ_SLICE = GQ_FITS ? D / 8 : 4;
+
+template <int G, int WAVES>
+__global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_grouped_f32_kernel(
+    const float* __restrict__ qkv, int64_t q_stride, const float* __restrict__ k_cache, const float* __restrict__ v_cache,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ token_request,
+    const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ table_rows,
+    float* __restrict__ out, int heads, int kv_heads, int parts, int block_size, float scale, int window) {
+  __shared__ float p_s[WAVES][G][DISTIE_WAVE];
+  __shared__ int64_t base_s[WAVES][DISTIE_WAVE];
+  __shared__ float m_s[WAVES][G], l_s[WAVES][G];
+  __shared__ float acc_s[WAVES][G][D];
+  const int lane = threadIdx.x % DISTIE_WAVE;
+  const int wave = threadIdx.x / DISTIE_WAVE;
+  const int64_t t = blockIdx.x;
+  const int group = heads / kv_heads;
+  const int kh = blockIdx.y / parts;
+  const int g0 = (blockIdx.y % parts) * G;
+  const int n = min(G, group - g0);                        // heads of this part
+  const int h0 = kh * group + g0;
+  const int q_pos = positions[t];
+  const int request_of_token = token_request[t];
+  const int32_t* table = block_table + static_cast<int64_t>(table_rows != nullptr ? table_rows[request_of_token] : request_of_token) * table_width;
+  const int sub = lane % 8;                                // which eighth of a row
+  const int key_in_pass = lane / 8;
+  float q_r[G][GQ_SLICE];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const float* q = qkv + t * q_stride + static_cast<int64_t>(h0 + min(g, n - 1)) * D + sub * GQ_SLICE;
+#pragma unroll
+    for (int d = 0; d < GQ_SLICE; d += 4) {
+      const float4 v = *reinterpret_cast<const float4*>(q + d);
+      q_r[g][d] = v.x; q_r[g][d + 1] = v.y; q_r[g][d + 2] = v.z; q_r[g][d + 3] = v.w;
+    }
+  }
+  const int first = window > 0 ? max(0, q_pos - window + 1) : 0;
+  const int last = q_pos;   // inclusive
+  float m[G], l[G];
+  float acc[G][DIMS_PER_LANE];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    m[g] = -INFINITY;
+    l[g] = 0.f;
+#pragma unroll
+    for (int i = 0; i < DIMS_PER_LANE; ++i) acc[g][i] = 0.f;
+  }
+
+  for (int c = first / DISTIE_WAVE * DISTIE_WAVE + wave * DISTIE_WAVE; c <= last; c += DISTIE_WAVE * WAVES) {
+    // Every load of a phase is issued before its results are used (a chunk costs a few trips to memory, not one
+    // for every pass and page): lane j looks up the page of key c + j, the addresses go from lane to lane.
+    const int key = c + lane;
+    const bool valid = key >= first && key <= last;
+    int64_t base = 0, row = 0;                              // keys that do not count read the start of the cache
+    if (valid) {
+      const int page = table[key / block_size];
+      base = (static_cast<int64_t>(page) * kv_heads + kh) * block_size * D;
+      row = base + static_cast<int64_t>(key % block_size) * D;
+    }
+    // ---- scores: eight keys a pass, four passes of loads in flight; afterwards lane j holds the scores of key c + j
+    float s[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) s[g] = 0.f;
+    constexpr int ROUND = G == 1 ? 8 : 4;                 // passes whose loads are in flight together: what the registers allow
+#pragma unroll
+    for (int round = 0; round < 8 / ROUND; ++round) {
+      float4 kk[ROUND][GQ_SLICE / 4];
+#pragma unroll
+      for (int ps = 0; ps < ROUND; ++ps) {
+        const int64_t from = __shfl(row, 8 * (ROUND * round + ps) + key_in_pass, DISTIE_WAVE);
+        const float* k = k_cache + from + sub * GQ_SLICE;
+#pragma unroll
+        for (int d = 0; d < GQ_SLICE / 4; ++d) kk[ps][d] = *reinterpret_cast<const float4*>(k + 4 * d);
+      }
+      __builtin_amdgcn_sched_barrier(0);                    // all of these loads are under way before the first is used
+#pragma unroll
+      for (int ps = 0; ps < ROUND; ++ps) {
+        const int pass = ROUND * round + ps;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          float v = 0.f;
+#pragma unroll
+          for (int d = 0; d < GQ_SLICE / 4; ++d) {
+            v = fmaf(q_r[g][4 * d], kk[ps][d].x, v);
+            v = fmaf(q_r[g][4 * d + 1], kk[ps][d].y, v);
+            v = fmaf(q_r[g][4 * d + 2], kk[ps][d].z, v);
+            v = fmaf(q_r[g][4 * d + 3], kk[ps][d].w, v);
+          }
+          v += __shfl_xor(v, 1, DISTIE_WAVE);
+          v += __shfl_xor(v, 2, DISTIE_WAVE);
+          v += __shfl_xor(v, 4, DISTIE_WAVE);
+          // the lane that owns this key for the softmax is lane 8 pass + (the key's place in the pass)
+          const float mine = __shfl(v, (lane % 8) * 8, DISTIE_WAVE);
+          if (lane / 8 == pass) s[g] = mine;
+        }
+      }
+    }
+    float alpha[G];
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const float sg = valid && g < n ? s[g] * scale : -INFINITY;
+      const float m_new = fmaxf(m[g], wave_max(sg));
+      alpha[g] = m_new == -INFINITY ? 0.f : expf(m[g] - m_new);     // 0 on the first chunk with a key (m = -inf)
+      const float p = valid && g < n ? expf(sg - m_new) : 0.f;
+      l[g] = l[g] * alpha[g] + wave_sum(p);
+      m[g] = m_new;
+      p_s[wave][g][lane] = p;
+    }
+    base_s[wave][lane] = base;
+    __builtin_amdgcn_wave_barrier();
+    // ---- output: the lane owns dimensions lane, lane + 64, ...; the chunk's values of a dimension are 16 pieces
+    // of four keys (a piece lies in one page: pages hold a multiple of four tokens)
+    const int lo = max(first - c, 0);                                   // keys lo .. hi of the chunk count
+    const int hi = min(DISTIE_WAVE - 1, last - c);
+#pragma unroll
+    for (int i = 0; i < DIMS_PER_LANE; ++i) {
+      const int d = lane + i * DISTIE_WAVE;
+      if (d >= D) continue;
+      float a[G];
+#pragma unroll
+      for (int g = 0; g < G; ++g) a[g] = acc[g][i] * alpha[g];
+      constexpr int GQ_PIECES = G == 1 ? 16 : 8;            // 16-byte pieces of V^T whose loads are in flight together
+#pragma unroll
+      for (int part = 0; part < 16 / GQ_PIECES; ++part) {
+        float4 vv[GQ_PIECES];
+#pragma unroll
+        for (int u = 0; u < GQ_PIECES; ++u) {
+          const int q = part * GQ_PIECES + u;
+          const int64_t page_base = base_s[wave][min(max(4 * q, lo), hi)];      // of a key that counts
+          vv[u] = *reinterpret_cast<const float4*>(v_cache + page_base + static_cast<int64_t>(d) * block_size +
+                                                   (c + 4 * q) % block_size);
+        }
+        __builtin_amdgcn_sched_barrier(0);                  // all of these loads are under way before the first is used
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+#pragma unroll
+          for (int u = 0; u < GQ_PIECES; ++u) {
+            const int q = part * GQ_PIECES + u;
+            const float4 pp = *reinterpret_cast<const float4*>(&p_s[wave][g][4 * q]);
+            const float v[4] = {vv[u].x, vv[u].y, vv[u].z, vv[u].w};
+            const float w[4] = {pp.x, pp.y, pp.z, pp.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int j = 4 * q + e;
+              // never a value of a key that does not count (a weight of zero times what lies there could be NaN)
+              a[g] = fmaf(w[e], (j >= lo && j <= hi) ? v[e] : 0.f, a[g]);
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < G; ++g) acc[g][i] = a[g];
+    }
+  }
+  // ---- the waves' parts, put together by wave 0 in wave order
+  if (lane == 0) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      m_s[wave][g] = m[g];
+      l_s[wave][g] = l[g];
+    }
+  }
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int i = 0; i < DIMS_PER_LANE; ++i) {
+      const int d = lane + i * DISTIE_WAVE;
+      if (d < D) acc_s[wave][g][d] = acc[g][i];
+    }
+  __syncthreads();
+  // wave w writes heads w, w + WAVES, ... of the part
+  for (int g = wave; g < n; g += WAVES) {
+    float top = -INFINITY;
+    for (int w = 0; w < WAVES; ++w) top = fmaxf(top, m_s[w][g]);
+    float total = 0.f;
+    float weight[WAVES];
+    for (int w = 0; w < WAVES; ++w) {
+      weight[w] = m_s[w][g] == -INFINITY ? 0.f : expf(m_s[w][g] - top);    // a wave without keys counts nothing
+      total += l_s[w][g] * weight[w];
+    }
+    const float inv = 1.f / total;
+    float* o = out + (t * heads + h0 + g) * D;
+#pragma unroll
+    for (int i = 0; i < DIMS_PER_LANE; ++i) {
+      const int d = lane + i * DISTIE_WAVE;
+      if (d >= D) continue;
+      float sum = 0.f;
+      for (int w = 0; w < WAVES; ++w) sum += acc_s[w][g][d] * weight[w];
+      o[d] = sum * inv;
+    }
+  }
+}
+
 // qkv: [T, q_stride] with q of head h at columns h*D; out: [T, heads*D]. window = 0: every earlier key.
 extern "C" int distie_attention_generic(const void* qkv, int dtype, int64_t q_stride, const void* k_cache,
                                         const void* v_cache, int cache_dtype, const int32_t* positions,
@@ -220,6 +420,26 @@ extern "C" int distie_attention_generic(const void* qkv, int dtype, int64_t q_st
     return DISTIE_BAD_ARGUMENT;
   if (heads > 65535) return DISTIE_BAD_ARGUMENT;
   dim3 grid(tokens, heads);
+  const int group = heads / kv_heads;
+  if (GQ_FITS && dtype == DISTIE_F32 && cache_dtype == DISTIE_F32 && q_stride % 4 == 0 && block_size % 4 == 0 &&
+      DISTIE_WAVE % block_size == 0 && static_cast<int64_t>(tokens) * heads < 2048) {
+    // requests that decode, float32: as many heads of a kv head to a workgroup as leaves a workgroup a compute unit
+    int per = 1;
+    for (int g : {2, 4})
+      if (group >= g && static_cast<int64_t>(tokens) * kv_heads * ((group + g - 1) / g) >= 256) per = g;
+    const int parts = (group + per - 1) / per;
+    const dim3 grouped(tokens, kv_heads * parts);
+#define DISTIE_GROUPED(G, WAVES)                                                                                   \
+    attn_grouped_f32_kernel<G, WAVES><<<grouped, DISTIE_WAVE * WAVES, 0, stream>>>(                                  \
+        static_cast<const float*>(qkv), q_stride, static_cast<const float*>(k_cache),                               \
+        static_cast<const float*>(v_cache), positions, token_request, block_table, table_width, table_rows,         \
+        static_cast<float*>(out), heads, kv_heads, parts, block_size, scale, window)
+    if (per == 4) DISTIE_GROUPED(4, 8);
+    else if (per == 2) DISTIE_GROUPED(2, 8);
+    else DISTIE_GROUPED(1, 8);
+#undef DISTIE_GROUPED
+    return launch_status();
+  }
   // few (token, head) pairs, as when requests decode: eight waves share each pair's keys
   if (static_cast<int64_t>(tokens) * heads < 2048) {
     DISTIE_DISPATCH(dtype, T, DISTIE_DISPATCH(cache_dtype, C,
