@@ -88,6 +88,19 @@ def check_logits(got, weights, cfg, ids, dtype, folder=None):
     rms = diff.pow(2).mean().sqrt().item()
     assert err < scale / 16, f"max error {err} vs oracle, largest logit {scale}"
     assert rms < scale / 64, f"rms error {rms} vs oracle, largest logit {scale}"
+    # The reference judges half precision by the share of positions whose largest logit is the same token as
+    # the oracle's, at least 0.98 on real checkpoints (benchmarks/correctness/metrics.py:16-22, 62-69). With
+    # random weights the two largest logits of a position lie 0.26-0.43 apart in the median where the rounding
+    # moves a logit by up to 0.16, and the share measured on these models is 0.97-0.99 (whole sequences of 100
+    # tokens, two seeds each): so a position whose winner is clear (ahead by more than twice the largest error
+    # met) must agree, every one, and the share over all positions must stay near what was measured.
+    if got.shape[0] >= 8:
+        same = got.argmax(-1) == want.argmax(-1)
+        top2 = want.topk(2, -1).values
+        clear = (top2[:, 0] - top2[:, 1]) > 2 * err
+        assert bool(same[clear].all()), "a position with a clear winner has another token on top"
+        share = same.float().mean().item()
+        assert share >= 0.9, f"top-1 agreement {share}"
 
 
 def plain_uniform(seed, counter):

@@ -64,6 +64,33 @@ def test_pool_threads():
     assert not errors and pool.num_free == 64
 
 
+@pytest.mark.parametrize("sanitizers", ["address,undefined", "thread"])
+def test_pool_under_sanitizers(tmp_path, sanitizers):
+    """The C++ id pool, driven from eight threads through its C interface (tests/pool_driver.cpp), built with
+    the host compiler's sanitizers: no report, exit status 0."""
+    import os
+    import shutil
+    import subprocess
+    from pathlib import Path
+
+    compiler = shutil.which(os.environ.get("CXX", "g++"))
+    if compiler is None:
+        pytest.skip("no host compiler")
+    here = Path(__file__).resolve().parent
+    source = here.parent / "distie_amd" / "csrc" / "block_pool.cpp"
+    binary = tmp_path / "pool_driver"
+    static = ["-static-libasan"] if "address" in sanitizers else ["-static-libtsan"]
+    build = subprocess.run([compiler, "-std=c++17", "-O1", "-g", "-pthread", f"-fsanitize={sanitizers}",
+                            "-fno-sanitize-recover=all", *static, str(source), str(here / "pool_driver.cpp"),
+                            "-o", str(binary)], capture_output=True, text=True)
+    if build.returncode != 0 and "sanitize" in build.stderr.lower() + build.stdout.lower():
+        pytest.skip("the host compiler has no runtime for these sanitizers")
+    assert build.returncode == 0, build.stderr
+    run = subprocess.run([str(binary)], capture_output=True, text=True, timeout=120)   # runtimes linked statically
+    assert run.returncode == 0 and "pool driver: fine" in run.stdout, run.stdout + run.stderr
+    assert "Sanitizer" not in run.stderr, run.stderr
+
+
 def manager(block=4, pages=12, slots=4, window=6):
     needs = [PagedKV(2, 16), PagedKV(2, 16, window), PagedKV(2, 16), None, FixedState.of((3,))]
     return CacheManager(needs, block, pages, slots, allocate=False)
