@@ -179,6 +179,8 @@ def main() -> int:
     parser.add_argument("--shape", default="1.5b", choices=sorted(SHAPES))
     parser.add_argument("--serve", action="store_true", help="the 64-request serving workload instead of fixed batches")
     parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--context", type=int, default=None,
+                        help="tokens behind every request when decoding starts (the shape's own: 2,048 or 8,192)")
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     parser.add_argument("--no-points", action="store_true", help="skip the other batch sizes")
     parser.add_argument("--no-tune", action="store_true",
@@ -201,7 +203,7 @@ def main() -> int:
     layers = shape["num_hidden_layers"]
     layers_run = args.layers or layers
     shape["num_hidden_layers"] = layers_run
-    context, prefill_tokens = preset["context"], preset["prefill"]
+    context, prefill_tokens = args.context or preset["context"], preset["prefill"]
     points_at = () if args.no_points or args.serve else preset["points"]
     max_batch = SERVE["requests"] if args.serve else max((args.batch,) + tuple(points_at))
     tokens_per_request = context + args.warmup + args.steps + early_tokens(max_batch, context)
@@ -211,7 +213,8 @@ def main() -> int:
     fraction = args.gpu_mem_fraction
     if fraction is None and (args.shape == "32b" or args.serve):
         fraction = 0.9
-    pages = None if fraction is not None else max_batch * -(-tokens_per_request // BLOCK_SIZE) + 8
+    pages = None if fraction is not None else max(max_batch * -(-tokens_per_request // BLOCK_SIZE),
+                                                  -(-prefill_tokens // BLOCK_SIZE)) + 8
     packed = True
     if args.packed_weights is not None:
         packed = False if args.packed_weights == "none" else tuple(r for r in args.packed_weights.split(",") if r)
