@@ -459,8 +459,9 @@ extern "C" int distie_attention_generic(const void* qkv, int dtype, int64_t q_st
 
 #if DISTIE_MATRIX_CORE_ATTENTION
 // ===================================================================================================
-//  Matrix-core kernels (bfloat16, pages of a multiple of 16 tokens). Both work on 16-wide blocks of
-//  "columns" against blocks of 16 keys with two products:
+//  Matrix-core kernels (bfloat16, pages of a multiple of 16 tokens). The decode kernel works on 16-wide
+//  blocks of "columns" against blocks of 16 keys with two products (the tiled kernel for portions of prompts
+//  does the same with 32-wide blocks and is described where it stands):
 //        S^T[key, col] = K[key, :] . q[col, :]        (v_mfma_f32_16x16x32_bf16, K rows as the A operand)
 //        online softmax over keys, per column, in float32 (weights as 2^x: scores are scaled by log2 e)
 //        O[col, d]  += P[col, key] . V^T[d, key]      (values are stored transposed inside a page, so the
@@ -896,31 +897,34 @@ extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, c
 //  * attn_prefill: the tiled kernel for portions of prompts. A workgroup of four waves owns PF_BM
 //    consecutive new tokens of one request and one head; it walks over the keys 64 at a time. The K tile
 //    [64, D] and the V^T tile [D, 64] are put into LDS once per workgroup (global loads of the next tile
-//    are in flight while the current one is used) and every wave multiplies its own 16 * PF_MB query
-//    columns against them with the same two products and the same register layout as attn_decode.
-//    The kernel is bound by its reads from LDS (every wave reads the whole tile): two blocks of columns
-//    per wave halve them per product, for the registers of head sizes up to 128 (with one tile of loads in
-//    flight instead of two; at 32,768 keys 570 instead of 850 us for 2,048 tokens of 12 heads).
+//    are in flight while the current one is used) and every wave multiplies its own 32 query columns
+//    against them with the 32 x 32 x 16 products (per flop they read half the operands of the 16-wide ones,
+//    which is what bounds those here):
+//        S^T[key, col] = K[key, :] . q[col, :]     K rows from LDS as the A operand, q in registers
+//        O^T[d, col]  += V^T[d, key] . P^T[key, col]
+//    A lane holds, of a 32 x 32 score tile, keys 8i + 4h + j (i, j < 4) of column c (c = lane % 32,
+//    h = lane / 32): so a lane's 32 scores of a key tile, its running maximum and sum and its 32 D / 64
+//    output sums all belong to one query token, and nothing but the column's maximum moves between lanes.
+//    The B operand of the second product wants 8 of 16 summed keys per lane: those are the lane's own
+//    scores if the 16 keys of a step are taken in the order (4h..4h+3, 8+4h..8+4h+3), and V^T is read
+//    from LDS in the same order.
+//    Head sizes that are no multiple of 32 compute a last block of 32 output rows of which 16 are zeros.
 //    Requests that bring fewer than `min_q_len` tokens are left to the decode kernel.
 // ===================================================================================================
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 constexpr int PF_BN = 64;                               // keys per tile
 constexpr int PF_WAVES = 4;
 constexpr int PF_THREADS = PF_WAVES * DISTIE_WAVE;
-#ifndef DISTIE_PF_MB
-#define DISTIE_PF_MB ((D <= 128) ? 2 : 1)
-#endif
-#ifndef DISTIE_PF_DEPTH
-#define DISTIE_PF_DEPTH ((DISTIE_PF_MB == 2) ? 1 : 2)
-#endif
-constexpr int PF_MB = DISTIE_PF_MB;                     // blocks of 16 query columns per wave
-constexpr int PF_WAVE_COLS = 16 * PF_MB;
+constexpr int PF_WAVE_COLS = 32;
 constexpr int PF_BM = PF_WAVES * PF_WAVE_COLS;          // query tokens per workgroup
-constexpr int PF_DEPTH = DISTIE_PF_DEPTH;                             // key tiles whose loads are in flight
-// Rows of K in LDS, in elements. Lane (r, g) reads 16 bytes at row r, byte 16 g (+ a constant): that is free
-// of bank conflicts when the row stride is 32 bytes more than a multiple of 64 (measured with the LDS
-// conflict counter: 16 or 48 bytes more cost every read twice).
-constexpr int PF_K_STRIDE = (D % 32 == 0) ? D + 16 : D;
-constexpr int PF_V_STRIDE = PF_BN + 8;
+constexpr float PF_GROW = 8.f;                          // in units of log 2: how far a score may pass a column's reference
+constexpr int PF_DK = D / 16;                           // steps of the q.k product
+constexpr int PF_DB = (D + 31) / 32;                    // blocks of 32 output rows
+// Rows in LDS, in elements. A lane reads 16 bytes of row (lane % 32) of K, and two times 8 bytes of row
+// (lane % 32) of V^T: free of bank conflicts when a row is an odd number of such pieces long (measured: K rows
+// of 272 and 304 bytes read at 198 B/clk a compute unit, of 288 at 112; V^T rows of 136 bytes 207, of 144 116).
+constexpr int PF_K_STRIDE = D + 8;
+constexpr int PF_V_STRIDE = PF_BN + 4;
 constexpr int PF_BLOCK_CHUNKS = 2 * D;                  // 16-byte pieces of 16 keys of K, and of V^T: [16, D] or [D, 16]
 constexpr int PF_PASSES = (PF_BLOCK_CHUNKS + DISTIE_WAVE - 1) / DISTIE_WAVE;   // pieces a lane carries per block
 static_assert(PF_WAVES * 16 == PF_BN, "each wave brings one block of 16 keys of a tile");
@@ -932,12 +936,12 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
     float* __restrict__ part_ml, int tokens, int num_requests, int heads, int kv_heads, int block_size, float scale,
     int window, int min_q_len) {
   __shared__ __attribute__((aligned(16))) bf16_t k_lds[PF_BN * PF_K_STRIDE];
-  __shared__ __attribute__((aligned(16))) bf16_t v_lds[D * PF_V_STRIDE];
+  __shared__ __attribute__((aligned(16))) bf16_t v_lds[32 * PF_DB * PF_V_STRIDE];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / DISTIE_WAVE);   // uniform: what depends on it alone stays scalar
   const int lane = tid % DISTIE_WAVE;
-  const int r = lane % 16;
-  const int g = lane / 16;
+  const int c = lane % 32;
+  const int h = lane / 32;
   const int group = heads / kv_heads;
   const float scale_log2 = scale * 1.4426950408889634f;      // scores in units of log 2: weights are exp2
 
@@ -963,37 +967,34 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
   const int key_end = pos0 + columns - 1;
   const int32_t* table = block_table + static_cast<int64_t>(table_rows != nullptr ? table_rows[request] : request) * table_width;
 
-  // ---- this wave's columns
+  // the rows of V^T past the head size, read by the last block of output rows, stay zero
+  if (D % 32 != 0)
+    for (int i = tid; i < (32 * PF_DB - D) * PF_V_STRIDE; i += PF_THREADS) v_lds[D * PF_V_STRIDE + i] = static_cast<bf16_t>(0.f);
+
+  // ---- this wave's columns; the lane's column
   const int wave_col0 = wave * PF_WAVE_COLS;
   const int wave_cols = max(0, min(PF_WAVE_COLS, columns - wave_col0));
   const int wave_last = pos0 + wave_col0 + wave_cols - 1;
   const int wave_first = window > 0 ? max(0, pos0 + wave_col0 - window + 1) : 0;
-  int col_pos[PF_MB];
-  bf16x8 q_reg[PF_MB][DK32 > 0 ? DK32 : 1];
-  shortx4 q_tail[PF_MB];
-#pragma unroll
-  for (int mb = 0; mb < PF_MB; ++mb) {
-    const int col = min(wave_col0 + 16 * mb + r, columns - 1);    // columns past the end repeat the last; dropped later
-    col_pos[mb] = pos0 + col;
+  const int col = min(wave_col0 + c, columns - 1);        // columns past the end repeat the last; dropped later
+  const int col_last = pos0 + col;                        // the last key the column sees, and the first
+  const int col_first = window > 0 ? max(0, col_last - window + 1) : 0;
+  bf16x8 q_reg[PF_DK];
+  {
     const bf16_t* q = qkv + (token0 + col) * q_stride + static_cast<int64_t>(head) * D;
 #pragma unroll
-    for (int dk = 0; dk < DK32; ++dk) q_reg[mb][dk] = *reinterpret_cast<const bf16x8*>(q + 32 * dk + 8 * g);
-    if (DK_TAIL) q_tail[mb] = *reinterpret_cast<const shortx4*>(q + (D - 16) + 4 * g);
+    for (int dk = 0; dk < PF_DK; ++dk) q_reg[dk] = *reinterpret_cast<const bf16x8*>(q + 16 * dk + 8 * h);
   }
-  floatx4 o_acc[PF_MB][DB16];
-  float m_run[PF_MB], l_run[PF_MB];
+  floatx16 o_acc[PF_DB];
 #pragma unroll
-  for (int mb = 0; mb < PF_MB; ++mb) {
-    m_run[mb] = -INFINITY;
-    l_run[mb] = 0.f;
+  for (int db = 0; db < PF_DB; ++db)
 #pragma unroll
-    for (int db = 0; db < DB16; ++db) o_acc[mb][db] = floatx4{0.f, 0.f, 0.f, 0.f};
-  }
+    for (int e = 0; e < 16; ++e) o_acc[db][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
 
   // ---- staging of one tile in registers. Wave w brings block w of the tile (keys k0 + 16 w .. + 15): one page
   // lookup a wave, the 16 rows of K are one run of 16 D elements in their page, V^T is D runs of 16.
-  // PF_DEPTH tiles are in flight: a tile's trip from memory is longer than the work on a tile.
-  uint4 k_stages[PF_DEPTH][PF_PASSES], v_stages[PF_DEPTH][PF_PASSES];
+  uint4 k_stage[PF_PASSES], v_stage[PF_PASSES];
   const int block_shift = (block_size & (block_size - 1)) == 0 ? __builtin_ctz(block_size) : -1;
   // Every lane issues the same loads for every tile, with no branch around them: a block that belongs to no
   // page reads the start of the cache instead and is cleared when it is stored.
@@ -1006,7 +1007,7 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
     const int slot = block_shift >= 0 ? key >> block_shift : key / block_size;
     return table[min(slot, table_width - 1)];
   };
-  auto fetch = [&](int k0, int page_of_block, uint4 (&k_stage)[PF_PASSES], uint4 (&v_stage)[PF_PASSES]) {
+  auto fetch = [&](int k0, int page_of_block) {
     const int key = k0 + 16 * wave;
     const bool live = block_live(key);
     const int offset = live ? (block_shift >= 0 ? key & (block_size - 1) : key % block_size) : 0;
@@ -1021,198 +1022,176 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
       v_stage[p] = *reinterpret_cast<const uint4*>(v_block + static_cast<int64_t>(j / 2) * block_size + 8 * (j % 2));
     }
   };
-  auto stash = [&](int k0, const uint4 (&k_stage)[PF_PASSES], const uint4 (&v_stage)[PF_PASSES]) {
-    const int key = k0 + 16 * wave;
+  // where a lane's pieces go in LDS: the same for every tile (a row of V^T is a multiple of 8 bytes long,
+  // not of 16: its pieces are stored as two halves)
+  int k_slot[PF_PASSES], v_slot[PF_PASSES];
+#pragma unroll
+  for (int p = 0; p < PF_PASSES; ++p) {
+    const int j = min(lane + p * DISTIE_WAVE, PF_BLOCK_CHUNKS - 1);
+    k_slot[p] = (16 * wave + j / (D / 8)) * PF_K_STRIDE + 8 * (j % (D / 8));
+    v_slot[p] = (j / 2) * PF_V_STRIDE + 16 * wave + 8 * (j % 2);
+  }
+  auto stash = [&](int k0) {
+    const int key = k0 + 16 * wave;                       // the same for the whole wave: the branches are uniform
     const bool live = block_live(key);
     // Slots after the last key of this workgroup were not written by this request, and blocks outside the keys
     // of this workgroup were not read: cleared (a weight of zero times NaN would still be NaN).
     const bool whole = live && key + 15 <= key_end;
+    if (whole) {
+#pragma unroll
+      for (int p = 0; p < PF_PASSES; ++p) {
+        if (lane + p * DISTIE_WAVE >= PF_BLOCK_CHUNKS) continue;
+        *reinterpret_cast<uint4*>(k_lds + k_slot[p]) = k_stage[p];
+        *reinterpret_cast<uint2*>(v_lds + v_slot[p]) = uint2{v_stage[p].x, v_stage[p].y};
+        *reinterpret_cast<uint2*>(v_lds + v_slot[p] + 4) = uint2{v_stage[p].z, v_stage[p].w};
+      }
+      return;
+    }
 #pragma unroll
     for (int p = 0; p < PF_PASSES; ++p) {
       const int j = lane + p * DISTIE_WAVE;
       if (j >= PF_BLOCK_CHUNKS) continue;
-      const uint4 k_raw = live ? k_stage[p] : uint4{0u, 0u, 0u, 0u};
-      *reinterpret_cast<uint4*>(k_lds + (16 * wave + j / (D / 8)) * PF_K_STRIDE + 8 * (j % (D / 8))) = k_raw;
-      uint4 v_raw = v_stage[p];
-      if (!whole) {
-        const int written = live ? key_end - (key + 8 * (j % 2)) + 1 : 0;        // of this piece's eight keys
-        const uint32_t w[4] = {v_raw.x, v_raw.y, v_raw.z, v_raw.w};
-        uint32_t m[4];
+      *reinterpret_cast<uint4*>(k_lds + k_slot[p]) = live ? k_stage[p] : uint4{0u, 0u, 0u, 0u};
+      const int written = live ? key_end - (key + 8 * (j % 2)) + 1 : 0;        // of this piece's eight keys
+      const uint32_t w[4] = {v_stage[p].x, v_stage[p].y, v_stage[p].z, v_stage[p].w};
+      uint32_t m[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          m[e] = written >= 2 * e + 2 ? w[e] : (written == 2 * e + 1 ? (w[e] & 0x0000ffffu) : 0u);
-        v_raw = uint4{m[0], m[1], m[2], m[3]};
-      }
-      *reinterpret_cast<uint4*>(v_lds + (j / 2) * PF_V_STRIDE + 16 * wave + 8 * (j % 2)) = v_raw;
+      for (int e = 0; e < 4; ++e)
+        m[e] = written >= 2 * e + 2 ? w[e] : (written == 2 * e + 1 ? (w[e] & 0x0000ffffu) : 0u);
+      *reinterpret_cast<uint2*>(v_lds + v_slot[p]) = uint2{m[0], m[1]};
+      *reinterpret_cast<uint2*>(v_lds + v_slot[p] + 4) = uint2{m[2], m[3]};
     }
   };
 
   auto compute = [&](int k0) {
     if (wave_cols <= 0 || k0 > wave_last || k0 + PF_BN - 1 < wave_first) return;
 
-    // ---- scores: 64 keys x the wave's columns
-    floatx4 s[PF_MB][4];
+    // ---- scores: 64 keys x the wave's 32 columns, as two blocks of 32 keys
+    floatx16 s[2];
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
+    for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int mb = 0; mb < PF_MB; ++mb) s[mb][kb] = floatx4{0.f, 0.f, 0.f, 0.f};
-      const bf16_t* k_row = k_lds + (16 * kb + r) * PF_K_STRIDE;
+      for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
 #pragma unroll
-      for (int dk = 0; dk < DK32; ++dk) {
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(k_row + 32 * dk + 8 * g);
+    for (int dk = 0; dk < PF_DK; ++dk)
 #pragma unroll
-        for (int mb = 0; mb < PF_MB; ++mb)
-          s[mb][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, q_reg[mb][dk], s[mb][kb], 0, 0, 0);
+      for (int kb = 0; kb < 2; ++kb) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(k_lds + (32 * kb + c) * PF_K_STRIDE + 16 * dk + 8 * h);
+        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, q_reg[dk], s[kb], 0, 0, 0);
       }
-      if (DK_TAIL) {
-        const shortx4 a = *reinterpret_cast<const shortx4*>(k_row + (D - 16) + 4 * g);
-#pragma unroll
-        for (int mb = 0; mb < PF_MB; ++mb) {
-          const floatx4 tail = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, q_tail[mb], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) s[mb][kb][i] += tail[i];
-        }
-      }
-    }
-    // ---- softmax step per column. A tile whose keys every column of the wave sees needs no mask: that is
-    // every tile but those on the diagonal and at a window's edge.
+    // ---- softmax step of the lane's column. A tile whose keys every column of the wave sees needs no mask:
+    // that is every tile but those on the diagonal and at a window's edge.
     const bool tile_open = k0 + PF_BN - 1 <= pos0 + wave_col0 &&
                            (window <= 0 || k0 >= pos0 + wave_col0 + wave_cols - window);
-    bf16x8 p_reg[PF_MB][2];
-    float alpha[PF_MB];
+    if (!tile_open) {
 #pragma unroll
-    for (int mb = 0; mb < PF_MB; ++mb) {
-      const int last = col_pos[mb];
-      const int first = window > 0 ? max(0, last - window + 1) : 0;
-      float best = -INFINITY;
-      if (tile_open) {
+      for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float v = s[mb][kb][i] * scale_log2;
-            s[mb][kb][i] = v;
-            best = fmaxf(best, v);
-          }
-      } else {
-#pragma unroll
-        for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int key = k0 + 16 * kb + 4 * g + i;
-            const float v = (key >= first && key <= last) ? s[mb][kb][i] * scale_log2 : -INFINITY;
-            s[mb][kb][i] = v;
-            best = fmaxf(best, v);
-          }
-      }
-      best = fmaxf(best, __shfl_xor(best, 16, DISTIE_WAVE));
-      best = fmaxf(best, __shfl_xor(best, 32, DISTIE_WAVE));
-      const float m_new = fmaxf(m_run[mb], best);
-      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      alpha[mb] = fast_exp2(m_run[mb] - m_safe);
-      float sum = 0.f;
-#pragma unroll
-      for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float p = fast_exp2(s[mb][kb][i] - m_safe);
-          sum += p;
-          p_reg[mb][kb / 2][4 * (kb % 2) + i] = static_cast<bf16_t>(p);
+        for (int e = 0; e < 16; ++e) {
+          const int key = k0 + 32 * kb + 8 * (e / 4) + 4 * h + e % 4;
+          if (key < col_first || key > col_last) s[kb][e] = -INFINITY;
         }
-      l_run[mb] = l_run[mb] * alpha[mb] + sum;
-      m_run[mb] = m_new;
     }
+    // The running reference m of a column (scores count from it: weights are 2^(score - m)) follows the
+    // largest score only when that has grown by more than PF_GROW since m was set: then the sums so far are
+    // scaled down, for all columns of the wave at once. In between a weight may reach 2^PF_GROW, which
+    // float32 sums and bfloat16 weights hold as well as they hold 1, and the scaling of the sums becomes rare.
+    float top = -INFINITY;
 #pragma unroll
-    for (int mb = 0; mb < PF_MB; ++mb) {
-      float a4[4];
+    for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) a4[i] = __shfl(alpha[mb], 4 * g + i, DISTIE_WAVE);
+      for (int e = 0; e < 16; ++e) top = fmaxf(top, s[kb][e]);
+    top = fmaxf(top, __shfl_xor(top, 32, DISTIE_WAVE));
+    const float best = top * scale_log2;                  // the scale is positive: the largest stays the largest
+    if (__any(best > m_run + PF_GROW)) {                  // also the first score of a column (m = -inf)
+      const float m_new = fmaxf(m_run, best);
+      const float alpha = m_new == -INFINITY ? 1.f : fast_exp2(m_run - m_new);   // 0 while m was -inf
+      l_run *= alpha;
+      m_run = m_new;
 #pragma unroll
-      for (int db = 0; db < DB16; ++db)
+      for (int db = 0; db < PF_DB; ++db)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o_acc[mb][db][i] *= a4[i];
+        for (int e = 0; e < 16; ++e) o_acc[db][e] *= alpha;
     }
-    // ---- O += P . V: two steps of 32 keys, each the pair of 16-key blocks (2 ks, 2 ks + 1)
+    const float from = m_run == -INFINITY ? 0.f : -m_run;
+    bf16x8 p_reg[4];                                      // step t: keys 16 t + (4h..4h+3, 8+4h..8+4h+3) of the tile
+    float sum = 0.f;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
+    for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int db = 0; db < DB16; ++db) {
-        const bf16_t* v_row = v_lds + (16 * db + r) * PF_V_STRIDE + 32 * ks + 4 * g;
+      for (int e = 0; e < 16; ++e) {
+        const float p = fast_exp2(fmaf(s[kb][e], scale_log2, from));
+        sum += p;
+        p_reg[2 * kb + e / 8][e % 8] = static_cast<bf16_t>(p);
+      }
+    l_run += sum;
+    // ---- O^T += V^T . P^T: four steps of 16 keys
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int db = 0; db < PF_DB; ++db) {
+        const bf16_t* v_row = v_lds + (32 * db + c) * PF_V_STRIDE + 16 * t + 4 * h;
         const uint2 lo = *reinterpret_cast<const uint2*>(v_row);
-        const uint2 hi = *reinterpret_cast<const uint2*>(v_row + 16);
+        const uint2 hi = *reinterpret_cast<const uint2*>(v_row + 8);
         const uintx4 words = {lo.x, lo.y, hi.x, hi.y};
-        const bf16x8 v = __builtin_bit_cast(bf16x8, words);
-#pragma unroll
-        for (int mb = 0; mb < PF_MB; ++mb)
-          o_acc[mb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_reg[mb][ks], v, o_acc[mb][db], 0, 0, 0);
+        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, words), p_reg[t], o_acc[db], 0, 0, 0);
       }
   };
 
   // With gridDim.z > 1 the key tiles of these tokens are cut in that many parts, one workgroup each, which write
   // unnormalised partial results that attn_prefill_merge_kernel combines: the last tokens of a long
-  // portion walk over many key tiles one after the other, and this halves the longest walk.
-  // PF_DEPTH tiles of loads are in flight (tiles past the last key load the start of the cache and are not used)
+  // portion walk over many key tiles one after the other, and this shortens the longest walk.
+  // One tile of loads is in flight (tiles past the last key load the start of the cache and are not used).
   const int all_tile0 = key_begin / PF_BN * PF_BN;
   const int all_tiles = (key_end - all_tile0) / PF_BN + 1;
   const int per_split = (all_tiles + gridDim.z - 1) / gridDim.z;
   const int tile0 = all_tile0 + static_cast<int>(blockIdx.z) * per_split * PF_BN;
   const int loop_end = min(key_end, tile0 + per_split * PF_BN - 1);            // last key of this workgroup's walk
-  int pages_ahead[PF_DEPTH];
-  {
-    int first_pages[PF_DEPTH];
-#pragma unroll
-    for (int d = 0; d < PF_DEPTH; ++d) first_pages[d] = lookup(tile0 + d * PF_BN);
-#pragma unroll
-    for (int d = 0; d < PF_DEPTH; ++d) {
-      fetch(tile0 + d * PF_BN, first_pages[d], k_stages[d], v_stages[d]);
-      pages_ahead[d] = lookup(tile0 + (PF_DEPTH + d) * PF_BN);
-    }
+  fetch(tile0, lookup(tile0));
+  int page_ahead = lookup(tile0 + PF_BN);
+  for (int k0 = tile0; k0 <= loop_end; k0 += PF_BN) {
+    __syncthreads();                       // every wave is done with the tile in LDS
+    stash(k0);
+    __syncthreads();
+    fetch(k0 + PF_BN, page_ahead);
+    page_ahead = lookup(k0 + 2 * PF_BN);
+    compute(k0);
   }
-  for (int k0 = tile0; k0 <= loop_end; k0 += PF_DEPTH * PF_BN) {
+  // ---- write: the lane holds, of its column, output rows 32 db + 8 i + 4 h + (0..3)
+  l_run += __shfl_xor(l_run, 32, DISTIE_WAVE);
+  if (wave_col0 + c >= columns) return;
+  const int64_t row = static_cast<int64_t>(token0 + wave_col0 + c) * heads + head;
+  if (gridDim.z == 1) {
+    bf16_t* o = out + row * D;
+    const float inv = 1.f / l_run;
 #pragma unroll
-    for (int d = 0; d < PF_DEPTH; ++d) {
-      const int k = k0 + d * PF_BN;
-      if (k > loop_end) break;
-      __syncthreads();                       // every wave is done with the tile in LDS
-      stash(k, k_stages[d], v_stages[d]);
-      __syncthreads();
-      fetch(k + PF_DEPTH * PF_BN, pages_ahead[d], k_stages[d], v_stages[d]);
-      pages_ahead[d] = lookup(k + 2 * PF_DEPTH * PF_BN);
-      compute(k);
-    }
-  }
-  // ---- write: the lane holds columns 4g..4g+3 of each block, output dim 16 db + r
+    for (int db = 0; db < PF_DB; ++db)
 #pragma unroll
-  for (int mb = 0; mb < PF_MB; ++mb) {
-    l_run[mb] += __shfl_xor(l_run[mb], 16, DISTIE_WAVE);
-    l_run[mb] += __shfl_xor(l_run[mb], 32, DISTIE_WAVE);
-  }
+      for (int i = 0; i < 4; ++i) {
+        const int d = 32 * db + 8 * i + 4 * h;
+        if (d >= D) continue;
+        uint32_t half[4];
 #pragma unroll
-  for (int mb = 0; mb < PF_MB; ++mb)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int col = 16 * mb + 4 * g + i;
-      const float l_col = __shfl(l_run[mb], 4 * g + i, DISTIE_WAVE);
-      const float m_col = __shfl(m_run[mb], 4 * g + i, DISTIE_WAVE);
-      if (col >= wave_cols) continue;
-      const int64_t row = static_cast<int64_t>(token0 + wave_col0 + col) * heads + head;
-      if (gridDim.z == 1) {
-        bf16_t* o = out + row * D;
-        const float inv = 1.f / l_col;
-#pragma unroll
-        for (int db = 0; db < DB16; ++db) o[16 * db + r] = static_cast<bf16_t>(o_acc[mb][db][i] * inv);
-      } else {
-        // a part without a key for this column leaves l = 0, and the merge does not read its sums
-        const int64_t at = static_cast<int64_t>(blockIdx.z) * tokens * heads + row;
-        float* po = part_o + at * D;
-#pragma unroll
-        for (int db = 0; db < DB16; ++db) po[16 * db + r] = o_acc[mb][db][i];
-        if (r == 0) {
-          part_ml[2 * at] = m_col;
-          part_ml[2 * at + 1] = l_col;
-        }
+        for (int j = 0; j < 4; ++j) half[j] = __builtin_bit_cast(uint16_t, static_cast<bf16_t>(o_acc[db][4 * i + j] * inv));
+        *reinterpret_cast<uint2*>(o + d) = uint2{half[0] | (half[1] << 16), half[2] | (half[3] << 16)};
       }
+  } else {
+    // a part without a key for this column leaves l = 0, and the merge does not read its sums
+    const int64_t at = static_cast<int64_t>(blockIdx.z) * tokens * heads + row;
+    float* po = part_o + at * D;
+#pragma unroll
+    for (int db = 0; db < PF_DB; ++db)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int d = 32 * db + 8 * i + 4 * h;
+        if (d >= D) continue;
+        *reinterpret_cast<float4*>(po + d) = float4{o_acc[db][4 * i], o_acc[db][4 * i + 1], o_acc[db][4 * i + 2], o_acc[db][4 * i + 3]};
+      }
+    if (h == 0) {
+      part_ml[2 * at] = m_run;
+      part_ml[2 * at + 1] = l_run;
     }
+  }
 }
 
 // Combines the `splits` parts of attn_prefill_kernel with gridDim.z > 1, in order: one block per token; tokens
@@ -1278,7 +1257,7 @@ extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, 
   // part_o (float32 [splits, tokens, heads, D]) and part_ml (float32 [splits, tokens, heads, 2]) in between.
   if (tokens <= 0) return 0;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size % 16 != 0 || table_width < 1 || window < 0 ||
-      num_requests < 1 || heads > 65535 || min_q_len < 1 || splits < 1 || splits > PF_MAX_SPLITS ||
+      num_requests < 1 || heads > 65535 || min_q_len < 1 || splits < 1 || splits > PF_MAX_SPLITS || !(scale > 0.f) ||
       (splits > 1 && (part_o == nullptr || part_ml == nullptr || token_request == nullptr)))
     return DISTIE_BAD_ARGUMENT;
   const int tiles = (tokens + PF_BM - 1) / PF_BM + num_requests;     // an upper bound; spare blocks leave at once

@@ -727,6 +727,8 @@ class HipOps(Ops):
 
     def paged_attention(self, qkv, meta: BatchMeta, group, k_cache, v_cache, num_heads, num_kv_heads, head_dim,
                         scale, window):
+        if not scale > 0:
+            raise KernelError(f"paged_attention: the scale of the scores must be positive, not {scale}")
         qkv = self.dense(qkv)
         self._own(qkv, k_cache, v_cache)
         lib = self.attention_library(head_dim)

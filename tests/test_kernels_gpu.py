@@ -620,6 +620,38 @@ def test_paged_attention_decode_step(ops, dtype, heads, kv_heads, dim, P, window
         close(got, want, dtype, scale=want.abs().max().item())
 
 
+@pytest.mark.parametrize("heads,kv_heads,dim,P", [(12, 2, 128, 16), (4, 2, 64, 16), (3, 1, 48, 16), (2, 1, 256, 32)])
+@pytest.mark.parametrize("per_key", [0.1, 1.0, -0.1, 0.02])
+def test_prefill_attention_scores_that_grow_along_the_keys(ops, heads, kv_heads, dim, P, per_key):
+    """The tiled kernel lets a column's reference score lag behind its largest score by up to a factor of 2^8
+    in weight before it scales the sums down. Scores that rise by `per_key` (in units of log 2) from one key
+    to the next cross that bound every few tiles of 64 keys (0.1), every tile (1.0), never after the first
+    (falling scores) or once in a long while (0.02); a portion without a past and one behind 500 tokens."""
+    dtype = torch.bfloat16
+    lens, q_lens = [700, 900], [700, 400]
+    meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, lens, q_lens, dtype, seed=11)
+    scale = dim ** -0.5
+    q = qkv.view(qkv.shape[0], heads + 2 * kv_heads, dim)
+    q[:, :heads, 0] = 8.0
+    slope = per_key / (8.0 * scale * 1.4426950408889634)
+    for b, n in enumerate(lens):
+        for pos in range(n):
+            page = int(meta.groups[0].block_table[b, pos // P])
+            k[page, :, pos % P, 0] = slope * pos
+    want = TorchOps("cuda").paged_attention(qkv.double(), meta, 0, k.double(), v.double(), heads, kv_heads, dim, scale, None)
+    got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, scale, None)
+    close(got, want, dtype, scale=want.abs().max().item())
+
+
+def test_attention_takes_a_positive_scale_only(ops):
+    from distie_amd.kernels.hip_ops import KernelError
+
+    meta, qkv, k, v = paged_case(4, 2, 32, 16, [40], [40], torch.bfloat16, seed=2)
+    for scale in (0.0, -0.1, float("nan")):
+        with pytest.raises(KernelError, match="scale"):
+            ops.paged_attention(qkv, meta, 0, k, v, 4, 2, 32, scale, None)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_finds_one_far_key(ops, dtype):
     """One key among hundreds gets a large score: the output must be that key's value,
