@@ -920,6 +920,10 @@ constexpr int PF_BM = PF_WAVES * PF_WAVE_COLS;          // query tokens per work
 constexpr float PF_GROW = 8.f;                          // in units of log 2: how far a score may pass a column's reference
 constexpr int PF_DK = D / 16;                           // steps of the q.k product
 constexpr int PF_DB = (D + 31) / 32;                    // blocks of 32 output rows
+#ifndef DISTIE_PF_AHEAD
+#define DISTIE_PF_AHEAD 6
+#endif
+constexpr int PF_AHEAD = DISTIE_PF_AHEAD;               // reads from LDS in flight ahead of the products
 // Rows in LDS, in elements. A lane reads 16 bytes of row (lane % 32) of K, and two times 8 bytes of row
 // (lane % 32) of V^T: free of bank conflicts when a row is an odd number of such pieces long (measured: K rows
 // of 272 and 304 bytes read at 198 B/clk a compute unit, of 288 at 112; V^T rows of 136 bytes 207, of 144 116).
@@ -1072,13 +1076,25 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
+    // PF_AHEAD reads from LDS are under way when the first product is issued, and every product is followed
+    // by one more read: left to itself the compiler keeps two reads in flight, which is less than the trip takes
+    {
+      bf16x8 a[2 * PF_DK];
 #pragma unroll
-    for (int dk = 0; dk < PF_DK; ++dk)
+      for (int i = 0; i < 2 * PF_DK; ++i)
+        a[i] = *reinterpret_cast<const bf16x8*>(k_lds + (32 * (i % 2) + c) * PF_K_STRIDE + 16 * (i / 2) + 8 * h);
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(k_lds + (32 * kb + c) * PF_K_STRIDE + 16 * dk + 8 * h);
-        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, q_reg[dk], s[kb], 0, 0, 0);
+      for (int i = 0; i < 2 * PF_DK; ++i)
+        s[i % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], q_reg[i / 2], s[i % 2], 0, 0, 0);
+      constexpr int ahead = 2 * PF_DK < PF_AHEAD ? 2 * PF_DK : PF_AHEAD;
+      __builtin_amdgcn_sched_group_barrier(0x100, ahead, 0);
+#pragma unroll
+      for (int i = 0; i < 2 * PF_DK - ahead; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
+      __builtin_amdgcn_sched_group_barrier(0x008, ahead, 0);
+    }
     // ---- softmax step of the lane's column. A tile whose keys every column of the wave sees needs no mask:
     // that is every tile but those on the diagonal and at a window's edge.
     const bool tile_open = k0 + PF_BN - 1 <= pos0 + wave_col0 &&
@@ -1126,16 +1142,28 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
       }
     l_run += sum;
     // ---- O^T += V^T . P^T: four steps of 16 keys
+    {
+      bf16x8 vt[4 * PF_DB];
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-      for (int db = 0; db < PF_DB; ++db) {
-        const bf16_t* v_row = v_lds + (32 * db + c) * PF_V_STRIDE + 16 * t + 4 * h;
+      for (int i = 0; i < 4 * PF_DB; ++i) {
+        const bf16_t* v_row = v_lds + (32 * (i % PF_DB) + c) * PF_V_STRIDE + 16 * (i / PF_DB) + 4 * h;
         const uint2 lo = *reinterpret_cast<const uint2*>(v_row);
         const uint2 hi = *reinterpret_cast<const uint2*>(v_row + 8);
         const uintx4 words = {lo.x, lo.y, hi.x, hi.y};
-        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, words), p_reg[t], o_acc[db], 0, 0, 0);
+        vt[i] = __builtin_bit_cast(bf16x8, words);
       }
+#pragma unroll
+      for (int i = 0; i < 4 * PF_DB; ++i)
+        o_acc[i % PF_DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vt[i], p_reg[i / PF_DB], o_acc[i % PF_DB], 0, 0, 0);
+      constexpr int ahead = 4 * PF_DB < PF_AHEAD ? 4 * PF_DB : PF_AHEAD;
+      __builtin_amdgcn_sched_group_barrier(0x100, ahead, 1);
+#pragma unroll
+      for (int i = 0; i < 4 * PF_DB - ahead; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, ahead, 1);
+    }
   };
 
   // With gridDim.z > 1 the key tiles of these tokens are cut in that many parts, one workgroup each, which write
