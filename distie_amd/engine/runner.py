@@ -48,15 +48,10 @@ class ModelRunner:
             if entry.request_id not in self.cache:
                 self.cache.add(entry.request_id)
         if reserve:
-            done = []
-            try:
-                for entry in entries:
-                    self.cache.reserve(entry.request_id, len(entry.tokens))
-                    done.append(entry)
-            except Exception:
-                # nothing was written yet; pages taken for this step stay with their
-                # requests and are returned when those end
-                raise
+            # if a reservation fails nothing was written yet; pages taken for this step stay with
+            # their requests and are returned when those end
+            for entry in entries:
+                self.cache.reserve(entry.request_id, len(entry.tokens))
         logits, ran = None, False
         if self.graphs is not None:
             logits = self.graphs.try_run(entries, feed)   # a view of the bucket's buffer: use it before the next step
