@@ -1,5 +1,7 @@
 // Large matrix products through hipBLASLt, with the plan of every shape kept: y[M, N] = x[M, K] . W[N, K]^T
-// (+ bias), bfloat16 operands, float32 sums, y in bfloat16 or float32 with rows `ldy` elements apart.
+// (+ bias), float32 sums, y with rows `ldy` elements apart. The operands are both bfloat16 (y in bfloat16 or
+// float32) or both float32 (y in float32: products and sums in float32, the library's plain 32-bit compute type,
+// no reduced-precision mode).
 //
 // The reference leaves these products to its library as well (torch.nn.functional.linear on cuBLAS:
 // worker/src/inference/qwen2/model.py:60-75). Calling the library from here instead of through torch saves
@@ -32,16 +34,16 @@ constexpr size_t FLUSH_BYTES = size_t(384) << 20;      // more than the 256 MB o
 constexpr float WORTH_TIMING = 1.3f;     // a candidate whose first run takes this much longer than the best so far is dropped
 
 struct Key {
-  int M, N, K, y_dtype, bias;
+  int M, N, K, x_dtype, y_dtype, bias;
   int64_t ldy;
   bool operator==(const Key& o) const {
-    return M == o.M && N == o.N && K == o.K && y_dtype == o.y_dtype && bias == o.bias && ldy == o.ldy;
+    return M == o.M && N == o.N && K == o.K && x_dtype == o.x_dtype && y_dtype == o.y_dtype && bias == o.bias && ldy == o.ldy;
   }
 };
 struct KeyHash {
   size_t operator()(const Key& k) const {
     uint64_t h = 1469598103934665603ull;
-    for (uint64_t v : {uint64_t(k.M), uint64_t(k.N), uint64_t(k.K), uint64_t(k.y_dtype), uint64_t(k.bias), uint64_t(k.ldy)}) {
+    for (uint64_t v : {uint64_t(k.M), uint64_t(k.N), uint64_t(k.K), uint64_t(k.x_dtype), uint64_t(k.y_dtype), uint64_t(k.bias), uint64_t(k.ldy)}) {
       h ^= v;
       h *= 1099511628211ull;
     }
@@ -63,6 +65,7 @@ std::unordered_map<Key, Plan, KeyHash> plans;
 long plans_made = 0, plans_timed = 0;
 
 bool ok(hipblasStatus_t s) { return s == HIPBLAS_STATUS_SUCCESS; }
+hipDataType type_of(int dtype) { return dtype == DISTIE_F32 ? HIP_R_32F : HIP_R_16BF; }
 
 void drop(Plan& p) {
   if (p.product) hipblasLtMatmulDescDestroy(p.product);
@@ -74,7 +77,7 @@ void drop(Plan& p) {
 
 // In the library's column-major terms: y^T [N x M, ld ldy] = W^T (stored K x N, ld K, transposed) . x^T (stored K x M, ld K).
 int make_plan(const Key& key, Plan& plan, std::vector<hipblasLtMatmulHeuristicResult_t>& found) {
-  const hipDataType out_type = key.y_dtype == DISTIE_F32 ? HIP_R_32F : HIP_R_16BF;
+  const hipDataType in_type = type_of(key.x_dtype), out_type = type_of(key.y_dtype);
   if (!ok(hipblasLtMatmulDescCreate(&plan.product, HIPBLAS_COMPUTE_32F, HIP_R_32F))) return DISTIE_LIB_UNSUPPORTED;
   const int32_t transposed = HIPBLAS_OP_T, plain = HIPBLAS_OP_N;
   bool fine = ok(hipblasLtMatmulDescSetAttribute(plan.product, HIPBLASLT_MATMUL_DESC_TRANSA, &transposed, sizeof(transposed))) &&
@@ -85,8 +88,8 @@ int make_plan(const Key& key, Plan& plan, std::vector<hipblasLtMatmulHeuristicRe
     fine = ok(hipblasLtMatmulDescSetAttribute(plan.product, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue))) &&
            ok(hipblasLtMatmulDescSetAttribute(plan.product, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type)));
   }
-  fine = fine && ok(hipblasLtMatrixLayoutCreate(&plan.w, HIP_R_16BF, key.K, key.N, key.K)) &&
-         ok(hipblasLtMatrixLayoutCreate(&plan.x, HIP_R_16BF, key.K, key.M, key.K)) &&
+  fine = fine && ok(hipblasLtMatrixLayoutCreate(&plan.w, in_type, key.K, key.N, key.K)) &&
+         ok(hipblasLtMatrixLayoutCreate(&plan.x, in_type, key.K, key.M, key.K)) &&
          ok(hipblasLtMatrixLayoutCreate(&plan.y, out_type, key.N, key.M, key.ldy));
   if (!fine) return DISTIE_LIB_UNSUPPORTED;
   hipblasLtMatmulPreference_t preference = nullptr;
@@ -144,18 +147,19 @@ extern "C" void distie_lib_counts(long* made, long* timed) {
   *timed = plans_timed;
 }
 
-// y = x . W^T (+ bias). `bias`: float32 [N] or null. `tune` != 0: a shape not yet timed has the library's candidate
+// y = x . W^T (+ bias). `x_dtype`: of x and W, `y_dtype`: of y. `bias`: float32 [N] or null. `tune` != 0: a shape not yet timed has the library's candidate
 // kernels run TIMED_RUNS times each on `stream` (which is waited for: not inside a capture) and keeps the fastest;
 // otherwise a new shape takes the library's first choice. The output is written by every candidate run, each
 // time with the whole result.
-extern "C" int distie_lib_linear(const void* x, const void* w, const void* bias, void* y, int y_dtype, int M, int N, int K,
-                                 int64_t ldy, int tune, hipStream_t stream) {
-  if (M < 1 || N < 1 || K < 1 || ldy < N || (y_dtype != DISTIE_F32 && y_dtype != DISTIE_BF16) || x == nullptr ||
-      w == nullptr || y == nullptr)
+extern "C" int distie_lib_linear(const void* x, const void* w, const void* bias, void* y, int x_dtype, int y_dtype, int M,
+                                 int N, int K, int64_t ldy, int tune, hipStream_t stream) {
+  if (M < 1 || N < 1 || K < 1 || ldy < N || (y_dtype != DISTIE_F32 && y_dtype != DISTIE_BF16) ||
+      (x_dtype != DISTIE_F32 && x_dtype != DISTIE_BF16) || (x_dtype == DISTIE_F32 && y_dtype != DISTIE_F32) ||
+      x == nullptr || w == nullptr || y == nullptr)
     return DISTIE_BAD_ARGUMENT;
   std::lock_guard<std::mutex> lock(guard);
   if (handle == nullptr) return DISTIE_LIB_NOT_READY;
-  const Key key{M, N, K, y_dtype, bias != nullptr ? 1 : 0, ldy};
+  const Key key{M, N, K, x_dtype, y_dtype, bias != nullptr ? 1 : 0, ldy};
   auto it = plans.find(key);
   std::vector<hipblasLtMatmulHeuristicResult_t> found;
   if (it == plans.end() || (tune && !it->second.timed)) {
@@ -179,10 +183,10 @@ extern "C" int distie_lib_linear(const void* x, const void* w, const void* bias,
       std::vector<hipblasLtMatmulAlgo_t> candidates;
       for (const auto& r : found) candidates.push_back(r.algo);
       {
-        const hipDataType out_type = y_dtype == DISTIE_F32 ? HIP_R_32F : HIP_R_16BF;
+        const hipDataType in_type = type_of(x_dtype), out_type = type_of(y_dtype);
         std::vector<hipblasLtMatmulHeuristicResult_t> all;
         if (ok(hipblaslt_ext::getAllAlgos(handle, hipblaslt_ext::GemmType::HIPBLASLT_GEMM, HIPBLAS_OP_T, HIPBLAS_OP_N,
-                                          HIP_R_16BF, HIP_R_16BF, out_type, out_type, HIPBLAS_COMPUTE_32F, all))) {
+                                          in_type, in_type, out_type, out_type, HIPBLAS_COMPUTE_32F, all))) {
           const float one = 1.f, zero = 0.f;
           for (auto& r : all) {
             size_t needs = 0;

@@ -536,7 +536,7 @@ class HipOps(Ops):
             lib.distie_lib_init.argtypes = [ctypes.c_int]
             lib.distie_lib_init.restype = ctypes.c_int
             lib.distie_lib_linear.argtypes = [_P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-                                              ctypes.c_int64, ctypes.c_int, _P]
+                                              ctypes.c_int, ctypes.c_int64, ctypes.c_int, _P]
             lib.distie_lib_linear.restype = ctypes.c_int
             lib.distie_lib_counts.argtypes = [ctypes.POINTER(ctypes.c_long), ctypes.POINTER(ctypes.c_long)]
             lib.distie_lib_counts.restype = None
@@ -554,7 +554,9 @@ class HipOps(Ops):
     LIBRARY_UNSUPPORTED = -3
 
     def _library_linear(self, x, weight, bias, out_dtype):
-        """x [M, K] . weight [N, K]^T (+ float32 bias) by the library, float32 sums, into a new [M, N] of `out_dtype`."""
+        """x [M, K] . weight [N, K]^T (+ float32 bias) by the library, float32 sums, into a new [M, N] of `out_dtype`.
+        x and weight are both bfloat16, or both float32 (then every product is a float32 product). None if the
+        library has no kernel for the product as asked."""
         M, K = x.shape
         N = weight.shape[0]
         if x.stride(1) != 1 or x.stride(0) != K:
@@ -563,21 +565,18 @@ class HipOps(Ops):
             weight = weight.contiguous()
         out = torch.empty((M, N), dtype=out_dtype, device=self.device)
         lib = self._library()
-        code, size = _CODES[out_dtype], out.element_size()
-        # The library's large kernels work on tiles of 256 x 256, one a compute unit at a time: a product with a
-        # few tiles more than a whole number of rounds pays a full round for them (at 2,048 rows 16,384 columns
-        # take 82 us and 17,920 take 116). The last columns as a product of their own cost less (20 us for
-        # 1,536), written into the same output.
+        code, size, w_size = _CODES[out_dtype], out.element_size(), weight.element_size()
+        # The library's large bfloat16 kernels work on tiles of 256 x 256, one a compute unit at a time: a product
+        # with a few tiles more than a whole number of rounds pays a full round for them (at 2,048 rows 16,384
+        # columns take 82 us and 17,920 take 116). The last columns as a product of their own cost less (20 us
+        # for 1,536), written into the same output.
         tail = self._library_tail(M, N) if out_dtype == torch.bfloat16 else 0
         for lo, hi in (((0, N - tail), (N - tail, N)) if tail else ((0, N),)):
             rc = lib.distie_lib_linear(
-                x.data_ptr(), weight.data_ptr() + lo * K * 2, bias.data_ptr() + lo * 4 if bias is not None else None,
-                out.data_ptr() + lo * size, code, M, hi - lo, K, N, 1 if self._tuning else 0, self._stream())
+                x.data_ptr(), weight.data_ptr() + lo * K * w_size, bias.data_ptr() + lo * 4 if bias is not None else None,
+                out.data_ptr() + lo * size, _code(x), code, M, hi - lo, K, N, 1 if self._tuning else 0, self._stream())
             if rc == self.LIBRARY_UNSUPPORTED:
-                # no kernel of the library's for this product as asked for: through torch, which knows more ways
-                y = torch.mm(x, weight.t(), out_dtype=torch.float32)
-                y = y if bias is None else y + bias
-                return y if out_dtype == torch.float32 else y.to(out_dtype)
+                return None
             _check(rc, "lib_linear")
         return out
 
@@ -677,7 +676,19 @@ class HipOps(Ops):
             return PartialSums(out, out_dtype) if partial_ok else self.dense(PartialSums(out, out_dtype))
         if both_bf16:
             # large bfloat16 product: the library's matrix-core kernels
-            return self._library_linear(x, weight, bias, out_dtype)
+            out = self._library_linear(x, weight, bias, out_dtype)
+            if out is None:
+                # no kernel of the library's for this product as asked for: through torch, which knows more ways
+                out = torch.mm(x, weight.t(), out_dtype=torch.float32)
+                out = out if bias is None else out + bias
+                out = out if out_dtype == torch.float32 else out.to(out_dtype)
+            return out
+        both_f32 = x.dtype == torch.float32 and weight.dtype == torch.float32 and out_dtype == torch.float32
+        if both_f32 and M > self.ROWS_MAX_ROWS:
+            # large float32 product: the library's float32 kernels (float32 products and sums); else the generic one
+            out = self._library_linear(x, weight, bias, out_dtype)
+            if out is not None:
+                return out
         out = torch.empty((M, N), dtype=out_dtype, device=self.device)
         if M <= self.ROWS_MAX_ROWS and K % 8 == 0:
             # few rows in float32 (or against a weight kept in float32): the weights are streamed, FMAs only

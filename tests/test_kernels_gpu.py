@@ -443,6 +443,30 @@ def test_library_kernels_chosen_by_timing(ops):
     assert ops.library_plans()[1] == timed + 1
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 250, 136), (2048, 1536, 1024), (65, 1000, 333)])
+def test_gemm_large_float32_is_a_float32_product(ops, M, N, K):
+    """Large float32 products go to the library's float32 kernels: every product and sum in float32. An error
+    bound far below what a product of operands cut to 10 or 7 bits of mantissa would leave (a relative 5e-4 and
+    4e-3 per product) pins that no reduced-precision mode is in use; with a bias, with tuning, and with a K that
+    is no multiple of 8."""
+    x, w, b = rand(M, K, seed=1), rand(N, K, seed=2), rand(N, seed=3)
+    want = x.double() @ w.double().T
+    scale = (x.double().abs() @ w.double().abs().T).max().item()       # what the rounding errors scale with
+    before = ops.library_plans()[0]
+    got = ops.linear(x, w)
+    assert got.dtype == torch.float32 and ops.library_plans()[0] == before + 1
+    assert (got.double() - want).abs().max().item() < 3e-6 * scale
+    got = ops.linear(x, w, b)
+    assert (got.double() - want - b.double()).abs().max().item() < 3e-6 * scale
+    ops.tune_library_products(True)
+    try:
+        tuned = ops.linear(x, w)
+    finally:
+        ops.tune_library_products(False)
+    assert (tuned.double() - want).abs().max().item() < 3e-6 * scale
+    assert (ops.linear_f32out(x, w).double() - want).abs().max().item() < 3e-6 * scale
+
+
 @pytest.mark.parametrize("bias", [False, True])
 def test_gemm_large_bf16_with_a_ragged_last_round(ops, bias, monkeypatch):
     """A large product whose columns end a little after a whole round of the library's tiles is run as two
