@@ -1226,9 +1226,10 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
 // of requests that the kernel skipped (fewer than min_q_len tokens) are skipped here as well.
 constexpr int PF_MAX_SPLITS = 16;
 
+template <typename OUT>
 __global__ void attn_prefill_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                           const int32_t* __restrict__ token_request, const int32_t* __restrict__ cu_q,
-                                          bf16_t* __restrict__ out, int tokens, int heads, int min_q_len, int splits) {
+                                          OUT* __restrict__ out, int tokens, int heads, int min_q_len, int splits) {
   const int64_t token = blockIdx.x;
   const int request = token_request[token];
   if (cu_q[request + 1] - cu_q[request] < min_q_len) return;
@@ -1266,10 +1267,14 @@ __global__ void attn_prefill_merge_kernel(const float* __restrict__ part_o, cons
     }
     const float inv = 1.f / l;
     const float v[4] = {sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv};
-    uint32_t h[4];
+    if constexpr (sizeof(OUT) == 4) {
+      *reinterpret_cast<float4*>(out + row * D + d) = float4{v[0], v[1], v[2], v[3]};
+    } else {
+      uint32_t h[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) h[e] = __builtin_bit_cast(uint16_t, static_cast<bf16_t>(v[e]));
-    *reinterpret_cast<uint2*>(out + row * D + d) = uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+      for (int e = 0; e < 4; ++e) h[e] = __builtin_bit_cast(uint16_t, static_cast<bf16_t>(v[e]));
+      *reinterpret_cast<uint2*>(out + row * D + d) = uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+    }
   }
 }
 
@@ -1297,9 +1302,301 @@ extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, 
   int status = launch_status();
   if (status != 0 || splits == 1) return status;
   const int work = heads * (D / 4);
-  attn_prefill_merge_kernel<<<tokens, work >= 512 ? 512 : (work >= 256 ? 256 : 64), 0, stream>>>(
+  attn_prefill_merge_kernel<bf16_t><<<tokens, work >= 512 ? 512 : (work >= 256 ? 256 : 64), 0, stream>>>(
       part_o, part_ml, token_request, cu_q, static_cast<bf16_t*>(out), tokens, heads, min_q_len, splits);
   return launch_status();
+}
+
+// ===================================================================================================
+//  * attn_prefill_f32: the tiled kernel in float32, for head sizes that are multiples of 32 up to 128. The same
+//    walk as attn_prefill (a workgroup of four waves owns 128 new tokens of one head, 32 query columns a wave,
+//    K and V^T tiles of 64 keys through LDS, the keys cut into parts that are merged) on the float32 products
+//    v_mfma_f32_32x32x2_f32: float32 operands, products and sums, no reduced precision anywhere. Such a product
+//    sums over two values, one from each half of the wave; four of them in a row take a lane's 16 bytes of a K or
+//    V^T row, so the head dimension (first product) and the keys (second product) are summed in the order in
+//    which the lanes hold them: d = 8 g + 4 h + e and key = 8 i + 4 h + j for step e or j of group g or i.
+//    The weights stay where the scores were (the accumulators' layout is the B operand's), in float32.
+// ===================================================================================================
+#if (DISTIE_HEAD_DIM % 32 == 0) && (DISTIE_HEAD_DIM <= 128)
+constexpr int PF32_K_STRIDE = D + 4;                    // floats: rows of an odd number of 16-byte pieces
+constexpr int PF32_V_STRIDE = PF_BN + 4;
+constexpr int PF32_CHUNKS = 4 * D;                      // 16-byte pieces of 16 keys of K ([16, D]), and of V^T ([D, 16])
+constexpr int PF32_PASSES = PF32_CHUNKS / DISTIE_WAVE;  // pieces a lane carries per block
+constexpr int PF32_AHEAD = 2;                           // reads from LDS ahead of the products (four products a read)
+
+__global__ __launch_bounds__(PF_THREADS, 1) void attn_prefill_f32_kernel(
+    const float* __restrict__ qkv, int64_t q_stride, const float* __restrict__ k_cache,
+    const float* __restrict__ v_cache, const int32_t* __restrict__ positions, const int32_t* __restrict__ cu_q,
+    const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ table_rows, float* __restrict__ out,
+    float* __restrict__ part_o, float* __restrict__ part_ml, int tokens, int num_requests, int heads, int kv_heads,
+    int block_size, float scale, int window, int min_q_len) {
+  __shared__ __attribute__((aligned(16))) float k_lds[PF_BN * PF32_K_STRIDE];
+  __shared__ __attribute__((aligned(16))) float v_lds[D * PF32_V_STRIDE];
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / DISTIE_WAVE);
+  const int lane = tid % DISTIE_WAVE;
+  const int c = lane % 32;
+  const int h = lane / 32;
+  const int group = heads / kv_heads;
+  const float scale_log2 = scale * 1.4426950408889634f;
+
+  // ---- which tokens (as in attn_prefill)
+  int tile = gridDim.y - 1 - blockIdx.y;
+  int request = 0, begin = 0, end = 0;
+  for (; request < num_requests; ++request) {
+    begin = cu_q[request];
+    end = cu_q[request + 1];
+    if (end - begin < min_q_len) continue;
+    const int tiles = (end - begin + PF_BM - 1) / PF_BM;
+    if (tile < tiles) break;
+    tile -= tiles;
+  }
+  if (request >= num_requests) return;
+  const int head = blockIdx.x;
+  const int kh = head / group;
+  const int token0 = begin + tile * PF_BM;
+  const int columns = min(PF_BM, end - token0);
+  const int pos0 = positions[token0];
+  const int key_begin = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int key_end = pos0 + columns - 1;
+  const int32_t* table = block_table + static_cast<int64_t>(table_rows != nullptr ? table_rows[request] : request) * table_width;
+
+  const int wave_col0 = wave * PF_WAVE_COLS;
+  const int wave_cols = max(0, min(PF_WAVE_COLS, columns - wave_col0));
+  const int wave_last = pos0 + wave_col0 + wave_cols - 1;
+  const int wave_first = window > 0 ? max(0, pos0 + wave_col0 - window + 1) : 0;
+  const int col = min(wave_col0 + c, columns - 1);
+  const int col_last = pos0 + col;
+  const int col_first = window > 0 ? max(0, col_last - window + 1) : 0;
+  float4 q_reg[D / 8];                                    // of the lane's column: d = 8 g + 4 h + (0..3)
+  {
+    const float* q = qkv + (token0 + col) * q_stride + static_cast<int64_t>(head) * D;
+#pragma unroll
+    for (int g = 0; g < D / 8; ++g) q_reg[g] = *reinterpret_cast<const float4*>(q + 8 * g + 4 * h);
+  }
+  floatx16 o_acc[D / 32];
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o_acc[db][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  // ---- staging: wave w brings block w of the tile (keys k0 + 16 w .. + 15)
+  uint4 k_stage[PF32_PASSES], v_stage[PF32_PASSES];
+  const int block_shift = (block_size & (block_size - 1)) == 0 ? __builtin_ctz(block_size) : -1;
+  auto block_live = [&](int key) { return key <= key_end && key + 15 >= key_begin; };
+  auto lookup = [&](int k0) {
+    const int key = k0 + 16 * wave;
+    const int slot = block_shift >= 0 ? key >> block_shift : key / block_size;
+    return table[min(slot, table_width - 1)];
+  };
+  auto fetch = [&](int k0, int page_of_block) {
+    const int key = k0 + 16 * wave;
+    const bool live = block_live(key);
+    const int offset = live ? (block_shift >= 0 ? key & (block_size - 1) : key % block_size) : 0;
+    const int64_t base = live ? (static_cast<int64_t>(page_of_block) * kv_heads + kh) * block_size * D : 0;
+    const float* k_block = k_cache + base + static_cast<int64_t>(offset) * D;
+    const float* v_block = v_cache + base + offset;
+#pragma unroll
+    for (int p = 0; p < PF32_PASSES; ++p) {
+      const int j = lane + p * DISTIE_WAVE;
+      k_stage[p] = *reinterpret_cast<const uint4*>(k_block + 4 * j);
+      v_stage[p] = *reinterpret_cast<const uint4*>(v_block + static_cast<int64_t>(j / 4) * block_size + 4 * (j % 4));
+    }
+  };
+  int k_slot[PF32_PASSES], v_slot[PF32_PASSES];
+#pragma unroll
+  for (int p = 0; p < PF32_PASSES; ++p) {
+    const int j = lane + p * DISTIE_WAVE;
+    k_slot[p] = (16 * wave + j / (D / 4)) * PF32_K_STRIDE + 4 * (j % (D / 4));
+    v_slot[p] = (j / 4) * PF32_V_STRIDE + 16 * wave + 4 * (j % 4);
+  }
+  // Slots after the last key of this workgroup were not written by this request, and blocks outside the keys
+  // of this workgroup were not read: cleared (a weight of zero times NaN would still be NaN).
+  auto stash = [&](int k0) {
+    const int key = k0 + 16 * wave;
+    const bool live = block_live(key);
+    if (live && key + 15 <= key_end) {
+#pragma unroll
+      for (int p = 0; p < PF32_PASSES; ++p) {
+        *reinterpret_cast<uint4*>(k_lds + k_slot[p]) = k_stage[p];
+        *reinterpret_cast<uint4*>(v_lds + v_slot[p]) = v_stage[p];
+      }
+      return;
+    }
+#pragma unroll
+    for (int p = 0; p < PF32_PASSES; ++p) {
+      const int j = lane + p * DISTIE_WAVE;
+      *reinterpret_cast<uint4*>(k_lds + k_slot[p]) = live ? k_stage[p] : uint4{0u, 0u, 0u, 0u};
+      const int written = live ? key_end - (key + 4 * (j % 4)) + 1 : 0;        // of this piece's four keys
+      *reinterpret_cast<uint4*>(v_lds + v_slot[p]) =
+          uint4{written >= 1 ? v_stage[p].x : 0u, written >= 2 ? v_stage[p].y : 0u, written >= 3 ? v_stage[p].z : 0u,
+                written >= 4 ? v_stage[p].w : 0u};
+    }
+  };
+
+  auto compute = [&](int k0) {
+    if (wave_cols <= 0 || k0 > wave_last || k0 + PF_BN - 1 < wave_first) return;
+    // ---- scores: 64 keys x the wave's 32 columns, as two blocks of 32 keys
+    floatx16 s[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
+    {
+      float4 a[D / 4];
+#pragma unroll
+      for (int i = 0; i < D / 4; ++i)
+        a[i] = *reinterpret_cast<const float4*>(k_lds + (32 * (i % 2) + c) * PF32_K_STRIDE + 8 * (i / 2) + 4 * h);
+#pragma unroll
+      for (int i = 0; i < D / 4; ++i) {
+        s[i % 2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].x, q_reg[i / 2].x, s[i % 2], 0, 0, 0);
+        s[i % 2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].y, q_reg[i / 2].y, s[i % 2], 0, 0, 0);
+        s[i % 2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].z, q_reg[i / 2].z, s[i % 2], 0, 0, 0);
+        s[i % 2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].w, q_reg[i / 2].w, s[i % 2], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x100, PF32_AHEAD, 0);
+#pragma unroll
+      for (int i = 0; i < D / 4 - PF32_AHEAD; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4 * PF32_AHEAD, 0);
+    }
+    const bool tile_open = k0 + PF_BN - 1 <= pos0 + wave_col0 &&
+                           (window <= 0 || k0 >= pos0 + wave_col0 + wave_cols - window);
+    if (!tile_open) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int key = k0 + 32 * kb + 8 * (e / 4) + 4 * h + e % 4;
+          if (key < col_first || key > col_last) s[kb][e] = -INFINITY;
+        }
+    }
+    // the column's reference follows its largest score when that has outgrown it (see attn_prefill)
+    float top = -INFINITY;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) top = fmaxf(top, s[kb][e]);
+    top = fmaxf(top, __shfl_xor(top, 32, DISTIE_WAVE));
+    const float best = top * scale_log2;
+    if (__any(best > m_run + PF_GROW)) {
+      const float m_new = fmaxf(m_run, best);
+      const float alpha = m_new == -INFINITY ? 1.f : fast_exp2(m_run - m_new);
+      l_run *= alpha;
+      m_run = m_new;
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o_acc[db][e] *= alpha;
+    }
+    const float from = m_run == -INFINITY ? 0.f : -m_run;
+    float sum = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        s[kb][e] = fast_exp2(fmaf(s[kb][e], scale_log2, from));
+        sum += s[kb][e];
+      }
+    l_run += sum;
+    // ---- O^T += V^T . P^T: eight groups of four keys for each block of 32 output rows
+    {
+      constexpr int reads = 8 * (D / 32);
+      float4 vt[reads];
+#pragma unroll
+      for (int i = 0; i < reads; ++i) {
+        const int db = i % (D / 32), group_of_keys = i / (D / 32);        // group: kb = / 4, i = % 4
+        vt[i] = *reinterpret_cast<const float4*>(v_lds + (32 * db + c) * PF32_V_STRIDE + 8 * group_of_keys + 4 * h);
+      }
+#pragma unroll
+      for (int i = 0; i < reads; ++i) {
+        const int db = i % (D / 32), kb = (i / (D / 32)) / 4, e = 4 * ((i / (D / 32)) % 4);
+        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(vt[i].x, s[kb][e], o_acc[db], 0, 0, 0);
+        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(vt[i].y, s[kb][e + 1], o_acc[db], 0, 0, 0);
+        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(vt[i].z, s[kb][e + 2], o_acc[db], 0, 0, 0);
+        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(vt[i].w, s[kb][e + 3], o_acc[db], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x100, PF32_AHEAD, 1);
+#pragma unroll
+      for (int i = 0; i < reads - PF32_AHEAD; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4 * PF32_AHEAD, 1);
+    }
+  };
+
+  const int all_tile0 = key_begin / PF_BN * PF_BN;
+  const int all_tiles = (key_end - all_tile0) / PF_BN + 1;
+  const int per_split = (all_tiles + gridDim.z - 1) / gridDim.z;
+  const int tile0 = all_tile0 + static_cast<int>(blockIdx.z) * per_split * PF_BN;
+  const int loop_end = min(key_end, tile0 + per_split * PF_BN - 1);
+  fetch(tile0, lookup(tile0));
+  int page_ahead = lookup(tile0 + PF_BN);
+  for (int k0 = tile0; k0 <= loop_end; k0 += PF_BN) {
+    __syncthreads();                       // every wave is done with the tile in LDS
+    stash(k0);
+    __syncthreads();
+    fetch(k0 + PF_BN, page_ahead);
+    page_ahead = lookup(k0 + 2 * PF_BN);
+    compute(k0);
+  }
+  // ---- write: the lane holds, of its column, output rows 32 db + 8 i + 4 h + (0..3)
+  l_run += __shfl_xor(l_run, 32, DISTIE_WAVE);
+  if (wave_col0 + c >= columns) return;
+  const int64_t row = static_cast<int64_t>(token0 + wave_col0 + c) * heads + head;
+  const bool whole = gridDim.z == 1;
+  const int64_t at = whole ? row : static_cast<int64_t>(blockIdx.z) * tokens * heads + row;
+  float* o = (whole ? out : part_o) + at * D;
+  const float factor = whole ? 1.f / l_run : 1.f;         // a part without a key for this column leaves l = 0: not read
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      *reinterpret_cast<float4*>(o + 32 * db + 8 * i + 4 * h) =
+          float4{o_acc[db][4 * i] * factor, o_acc[db][4 * i + 1] * factor, o_acc[db][4 * i + 2] * factor, o_acc[db][4 * i + 3] * factor};
+  if (!whole && h == 0) {
+    part_ml[2 * at] = m_run;
+    part_ml[2 * at + 1] = l_run;
+  }
+}
+#endif
+
+extern "C" int distie_attention_prefill_f32_fits() { return (D % 32 == 0 && D <= 128) ? 1 : 0; }
+
+// As distie_attention_prefill_bf16, for float32 queries and a float32 cache; head sizes for which
+// distie_attention_prefill_f32_fits() says 1.
+extern "C" int distie_attention_prefill_f32(const void* qkv, int64_t q_stride, const void* k_cache, const void* v_cache,
+                                            const int32_t* positions, const int32_t* cu_q, const int32_t* block_table,
+                                            int table_width, const int32_t* table_rows, void* out, int tokens, int num_requests, int heads,
+                                            int kv_heads, int block_size, float scale, int window, int min_q_len,
+                                            const int32_t* token_request, float* part_o, float* part_ml,
+                                            int splits, hipStream_t stream) {
+#if (DISTIE_HEAD_DIM % 32 == 0) && (DISTIE_HEAD_DIM <= 128)
+  if (tokens <= 0) return 0;
+  if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size % 16 != 0 || table_width < 1 || window < 0 ||
+      num_requests < 1 || heads > 65535 || min_q_len < 1 || splits < 1 || splits > PF_MAX_SPLITS || !(scale > 0.f) ||
+      q_stride % 4 != 0 ||
+      (splits > 1 && (part_o == nullptr || part_ml == nullptr || token_request == nullptr)))
+    return DISTIE_BAD_ARGUMENT;
+  const int tiles = (tokens + PF_BM - 1) / PF_BM + num_requests;
+  if (tiles > 65535) return DISTIE_BAD_ARGUMENT;
+  attn_prefill_f32_kernel<<<dim3(heads, tiles, splits), PF_THREADS, 0, stream>>>(
+      static_cast<const float*>(qkv), q_stride, static_cast<const float*>(k_cache), static_cast<const float*>(v_cache),
+      positions, cu_q, block_table, table_width, table_rows, static_cast<float*>(out), part_o, part_ml, tokens, num_requests,
+      heads, kv_heads, block_size, scale, window, min_q_len);
+  int status = launch_status();
+  if (status != 0 || splits == 1) return status;
+  const int work = heads * (D / 4);
+  attn_prefill_merge_kernel<float><<<tokens, work >= 512 ? 512 : (work >= 256 ? 256 : 64), 0, stream>>>(
+      part_o, part_ml, token_request, cu_q, static_cast<float*>(out), tokens, heads, min_q_len, splits);
+  return launch_status();
+#else
+  return DISTIE_BAD_ARGUMENT;
+#endif
 }
 
 #else   // a head size that is no multiple of 16: the wave-per-token kernel is all there is
@@ -1315,6 +1612,14 @@ extern "C" int distie_attention_decode_bf16(const void*, int64_t, const void*, c
 extern "C" int distie_attention_prefill_bf16(const void*, int64_t, const void*, const void*, const int32_t*, const int32_t*,
                                              const int32_t*, int, const int32_t*, void*, int, int, int, int, int, float, int, int,
                                              const int32_t*, void*, void*, int, hipStream_t) {
+  return DISTIE_BAD_ARGUMENT;
+}
+
+extern "C" int distie_attention_prefill_f32_fits() { return 0; }
+
+extern "C" int distie_attention_prefill_f32(const void*, int64_t, const void*, const void*, const int32_t*, const int32_t*,
+                                            const int32_t*, int, const int32_t*, void*, int, int, int, int, int, float, int, int,
+                                            const int32_t*, void*, void*, int, hipStream_t) {
   return DISTIE_BAD_ARGUMENT;
 }
 

@@ -137,6 +137,7 @@ class HipOps(Ops):
     # 4,096 keys, 5 at 8,192, 8 from 16,384 on; the kernel takes up to 16)
     PREFILL_PARTS = ((1024, 3), (8192, 5), (16384, 8))
     PREFILL_WORKGROUPS = 512         # as many workgroups a short portion's attention should have, if its keys allow
+    PREFILL_F32_MIN_TOKENS = 32      # float32 steps with a portion of at least this many tokens go to the tiled float32 kernel
     # decode attention cuts the keys into runs so that about DECODE_WAVES waves are at work, with at most
     # DECODE_MAX_RUNS places for partial results per request and head
     DECODE_WAVES = 1024
@@ -254,6 +255,7 @@ class HipOps(Ops):
                                                      _I, _I, _I, _I, _F, _I, _P]
             lib.distie_attention_prefill_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I,
                                                           _F, _I, _I, _P, _P, _P, _I, _P]
+            lib.distie_attention_prefill_f32.argtypes = lib.distie_attention_prefill_bf16.argtypes
             lib.distie_attention_decode_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I,
                                                          _I, _F, _I, _I, _I, _I, _P]
             if lib.distie_attention_head_dim() != head_dim:
@@ -780,6 +782,23 @@ class HipOps(Ops):
                     plan["prefill_ml"].data_ptr() if parts > 1 else None, parts, self._stream()),
                     "attention_prefill_bf16")
             return out
+        f32 = qkv.dtype == torch.float32 and k_cache.dtype == torch.float32
+        if f32 and meta.max_q >= self.PREFILL_F32_MIN_TOKENS and meta.block_size % 16 == 0 and \
+                qkv.shape[1] % 4 == 0 and lib.distie_attention_prefill_f32_fits():
+            # portions of prompts in float32: the tiled kernel on float32 matrix products takes the whole step
+            key = ("attention_f32", int(window or 0), num_heads, head_dim, meta.max_kv, self.PREFILL_PARTS,
+                   self.PREFILL_WORKGROUPS)
+            plan = meta.scratch.get(key)
+            if plan is None:
+                plan = meta.scratch[key] = self._prefill_parts(meta, T, num_heads, head_dim, window)
+            parts = plan["parts"]
+            _check(lib.distie_attention_prefill_f32(
+                qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), meta.positions.data_ptr(),
+                meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], rows_ptr, out.data_ptr(), T, meta.num_requests,
+                num_heads, num_kv_heads, meta.block_size, float(scale), int(window or 0), 1,
+                meta.token_request.data_ptr(), plan["prefill_o"].data_ptr() if parts > 1 else None,
+                plan["prefill_ml"].data_ptr() if parts > 1 else None, parts, self._stream()), "attention_prefill_f32")
+            return out
         _check(lib.distie_attention_generic(
             qkv.data_ptr(), _code(qkv), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), _code(k_cache),
             meta.positions.data_ptr(), meta.token_request.data_ptr(), table.data_ptr(), table.shape[1], rows_ptr,
@@ -809,22 +828,27 @@ class HipOps(Ops):
                                             device=self.device)
         plan["prefill"] = singles < meta.num_requests or not plan["decode"]
         if plan["prefill"]:
-            # portions of prompts (and single tokens too, if the decode kernel did not take them). Long
-            # walks over the keys are cut into parts that run side by side.
-            visible = min(meta.max_kv, int(window) + 128) if window else meta.max_kv
-            parts = 1
-            for keys, cut in self.PREFILL_PARTS:
-                if visible >= keys:
-                    parts = cut
-            # few new tokens make few workgroups (one per 128 tokens of a request and head), each walking all
-            # the keys alone: more parts then, down to 128 keys a part
-            tiles = -(-T // 128) + meta.num_requests
-            wanted = -(-self.PREFILL_WORKGROUPS // (tiles * num_heads))
-            parts = max(parts, min(wanted, visible // 128, 16))
-            plan["parts"] = parts
-            if parts > 1:
-                plan["prefill_o"] = torch.empty((parts, T, num_heads, head_dim), dtype=torch.float32, device=self.device)
-                plan["prefill_ml"] = torch.empty((parts, T, num_heads, 2), dtype=torch.float32, device=self.device)
+            plan.update(self._prefill_parts(meta, T, num_heads, head_dim, window))
+        return plan
+
+    def _prefill_parts(self, meta: BatchMeta, T, num_heads, head_dim, window) -> dict:
+        """Into how many parts the tiled kernel cuts its walk over the keys, and the buffers between it and the
+        merge. Portions of prompts (and single tokens too, if no other kernel took them): long walks over the
+        keys are cut into parts that run side by side."""
+        visible = min(meta.max_kv, int(window) + 128) if window else meta.max_kv
+        parts = 1
+        for keys, cut in self.PREFILL_PARTS:
+            if visible >= keys:
+                parts = cut
+        # few new tokens make few workgroups (one per 128 tokens of a request and head), each walking all
+        # the keys alone: more parts then, down to 128 keys a part
+        tiles = -(-T // 128) + meta.num_requests
+        wanted = -(-self.PREFILL_WORKGROUPS // (tiles * num_heads))
+        parts = max(parts, min(wanted, visible // 128, 16))
+        plan = {"parts": parts}
+        if parts > 1:
+            plan["prefill_o"] = torch.empty((parts, T, num_heads, head_dim), dtype=torch.float32, device=self.device)
+            plan["prefill_ml"] = torch.empty((parts, T, num_heads, 2), dtype=torch.float32, device=self.device)
         return plan
 
     def silu_mul(self, gate_up):

@@ -594,11 +594,12 @@ def test_paged_attention_long_portions(ops, dtype, heads, kv_heads, dim, P, wind
 @pytest.mark.parametrize("heads,kv_heads,dim,P,window", [(4, 2, 16, 16, None), (12, 2, 128, 16, None), (3, 1, 48, 16, 700),
                                                          (2, 1, 256, 32, 100), (6, 2, 64, 64, None)])
 @pytest.mark.parametrize("parts", [2, 3, 5, 8, 16])
-def test_paged_attention_keys_walked_in_parts(ops, heads, kv_heads, dim, P, window, parts, monkeypatch):
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_keys_walked_in_parts(ops, dtype, heads, kv_heads, dim, P, window, parts, monkeypatch):
     """From 1,024 visible keys on, the tiled kernel cuts the walk over the keys into parts and merges: a long
     portion without a past, one that starts in the middle of a tile after a long past, a short one, a
-    two-token one, and single tokens (which the decode kernel takes, or the tiled kernel too)."""
-    dtype = torch.bfloat16
+    two-token one, and single tokens (which the decode kernel takes, or the tiled kernel too). In float32 the
+    tiled float32 kernel takes the whole step where the head size allows it."""
     lens, q_lens = [1300, 1500, 90, 777, 40, 1100], [1300, 100, 90, 1, 2, 1]
     meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, lens, q_lens, dtype, seed=5)
     monkeypatch.setattr(type(ops), "PREFILL_PARTS", ((64, parts),))      # as a longer context would have it
@@ -646,12 +647,14 @@ def test_paged_attention_decode_step(ops, dtype, heads, kv_heads, dim, P, window
 
 @pytest.mark.parametrize("heads,kv_heads,dim,P", [(12, 2, 128, 16), (4, 2, 64, 16), (3, 1, 48, 16), (2, 1, 256, 32)])
 @pytest.mark.parametrize("per_key", [0.1, 1.0, -0.1, 0.02])
-def test_prefill_attention_scores_that_grow_along_the_keys(ops, heads, kv_heads, dim, P, per_key):
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_prefill_attention_scores_that_grow_along_the_keys(ops, dtype, heads, kv_heads, dim, P, per_key):
     """The tiled kernel lets a column's reference score lag behind its largest score by up to a factor of 2^8
     in weight before it scales the sums down. Scores that rise by `per_key` (in units of log 2) from one key
     to the next cross that bound every few tiles of 64 keys (0.1), every tile (1.0), never after the first
     (falling scores) or once in a long while (0.02); a portion without a past and one behind 500 tokens."""
-    dtype = torch.bfloat16
+    if dtype == torch.float32 and per_key == 1.0:
+        pytest.skip("scores near 7,000 are known to float32 to 5e-4 only: the weights of the last keys cannot be compared")
     lens, q_lens = [700, 900], [700, 400]
     meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, lens, q_lens, dtype, seed=11)
     scale = dim ** -0.5
