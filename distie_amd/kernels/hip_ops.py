@@ -13,6 +13,7 @@ the kernels refuse, raises: there is no fallback.
 from __future__ import annotations
 
 import ctypes
+import logging
 from typing import Dict, Optional
 
 import numpy as np
@@ -20,6 +21,8 @@ import torch
 
 from ..csrc import build
 from .interface import BatchMeta, Ops
+
+_log = logging.getLogger(__name__)
 
 _F32, _BF16 = 0, 1
 _CODES = {torch.float32: _F32, torch.bfloat16: _BF16}
@@ -137,6 +140,7 @@ class HipOps(Ops):
     # 4,096 keys, 5 at 8,192, 8 from 16,384 on; the kernel takes up to 16)
     PREFILL_PARTS = ((1024, 3), (8192, 5), (16384, 8))
     PREFILL_WORKGROUPS = 512         # as many workgroups a short portion's attention should have, if its keys allow
+    PACKED_KEEPS_FREE = 0.3          # share of the device's memory that packed weight copies leave free
     PREFILL_F32_MIN_TOKENS = 32      # float32 steps with a portion of at least this many tokens go to the tiled float32 kernel
     # decode attention cuts the keys into runs so that about DECODE_WAVES waves are at work, with at most
     # DECODE_MAX_RUNS places for partial results per request and head
@@ -166,6 +170,7 @@ class HipOps(Ops):
         self._compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         self._lib = None
         self._tuning = False
+        self._packed_left_out = 0
         self._ops = ctypes.CDLL(str(build.ensure("ops")))
         self._declare()
         self._attn: Dict[int, ctypes.CDLL] = {}
@@ -417,6 +422,15 @@ class HipOps(Ops):
         if row_map.numel() % 16 or int(row_map.max()) >= N or int(row_map.min()) < -1 or \
                 row_map.numel() // 16 * -(-K // 32) * 512 != self._packed_elements(N, K, gated):
             raise KernelError("prepare_linear: bad row map")
+        # The copies are for speed, the cache is needed: a copy that would leave less than PACKED_KEEPS_FREE of the
+        # card's memory free is left out (the product then streams the stored layout), said once.
+        free, total = torch.cuda.mem_get_info(self.device)
+        if free - 2 * self._packed_elements(N, K, gated) < self.PACKED_KEEPS_FREE * total:
+            if not self._packed_left_out:
+                _log.warning("packed weight copies are left out from here on: less than %.0f %% of the device's "
+                             "memory would stay free", 100 * self.PACKED_KEEPS_FREE)
+            self._packed_left_out += 1
+            return
         row_map = row_map.to(device=self.device, dtype=torch.int32)
         packed = torch.empty(self._packed_elements(N, K, gated), dtype=torch.bfloat16, device=self.device)
         _check(self._ops.distie_pack_rows(weight.data_ptr(), packed.data_ptr(), row_map.data_ptr(),

@@ -412,6 +412,27 @@ def test_partial_sums_are_added_by_their_readers(ops):
     close(ops.dense(part), dense, torch.bfloat16, scale=dense.abs().max().item())
 
 
+def test_packed_copies_are_left_out_when_memory_is_short(ops, monkeypatch, caplog):
+    """A packed copy that would leave less than PACKED_KEEPS_FREE of the device's memory free is not made; the
+    product then streams the stored layout and gives the same result."""
+    import logging
+
+    x, w = rand(8, 264, dtype=torch.bfloat16, seed=1), rand(1000, 264, dtype=torch.bfloat16, seed=2)
+    want = x.double() @ w.double().T
+    free, total = torch.cuda.mem_get_info()
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda *a: (int(0.3 * total) + 1000, total))
+    left_out = ops._packed_left_out
+    with caplog.at_level(logging.WARNING, logger="distie_amd.kernels.hip_ops"):
+        ops.prepare_linear(w, role="down")
+    assert not hasattr(w, "_distie_packed") and ops._packed_left_out == left_out + 1
+    assert left_out > 0 or "left out" in caplog.text
+    close(ops.dense(ops.linear(x, w)), want, torch.bfloat16, scale=want.abs().max().item())
+    monkeypatch.undo()
+    ops.prepare_linear(w, role="down")
+    assert hasattr(w, "_distie_packed")
+    close(ops.dense(ops.linear(x, w)), want, torch.bfloat16, scale=want.abs().max().item())
+
+
 def test_gemm_large_bf16_uses_library_and_matches(ops):
     x, w, b = rand(300, 136, dtype=torch.bfloat16, seed=1), rand(250, 136, dtype=torch.bfloat16, seed=2), rand(250, seed=3)
     want = x.double() @ w.double().T + b.double()
