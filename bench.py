@@ -77,6 +77,21 @@ def early_tokens(batch, context):
     return batch * -(-context // TOKEN_BUDGET) + batch + 8
 
 
+def check_logits(logits, rows, what):
+    """A line is printed only for a model that computes: the logits of the last step are numbers, differ along
+    the vocabulary and from request to request (random prompts), and are of the size a model with these
+    weights gives (not zeros, not overflow)."""
+    import torch
+
+    assert logits is not None and logits.shape[0] >= rows, f"{what}: no logits for {rows} rows"
+    logits = logits[:rows].float()
+    assert bool(torch.isfinite(logits).all()), f"{what}: logits are not finite"
+    spread = logits.std(dim=1)
+    assert bool((spread > 1e-3).all()) and bool((spread < 1e3).all()), f"{what}: logits are constant or blown up"
+    if rows > 1:
+        assert bool((logits[1:] - logits[:1]).abs().amax(dim=1).gt(1e-3).all()), f"{what}: every request has the same logits"
+
+
 def decode_run(llm, batch, context, steps, warmup, vocab, seed):
     """-> (seconds per step, mean context over the timed steps)"""
     import torch
@@ -99,6 +114,9 @@ def decode_run(llm, batch, context, steps, warmup, vocab, seed):
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     assert all(s.num_tokens == b + steps for s, b in zip(seqs, before)), "a timed step did not decode every request"
+    check_logits(llm.last_logits, batch, f"decode at batch {batch}")
+    picked = {s.output_ids[-1] for s in seqs} | {t for s in seqs[:1] for t in s.output_ids[-steps:]}
+    assert len(picked) > 1, "every decoded token is the same"
     # keys a decode step reads for a request: everything cached before it, plus its own token
     mean_ctx = sum(before) / len(before) + (steps - 1) / 2.0
     for i in ids:
@@ -124,10 +142,11 @@ def prefill_run(llm, tokens, portion, vocab, repeats=PREFILL_REPEATS):
         t0 = time.perf_counter()
         for begin in range(0, tokens, portion):
             part = ids[begin:begin + portion]
-            llm.step([StepEntry(f"prefill-{r}", part, [len(part) - 1] if begin + portion >= tokens else [])])
+            logits = llm.step([StepEntry(f"prefill-{r}", part, [len(part) - 1] if begin + portion >= tokens else [])])
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         llm.finish(f"prefill-{r}")
+        check_logits(logits, 1, "prefill")
         if r > 0:                                          # the first run warms up
             times.append(dt)
     return statistics.median(times)

@@ -38,12 +38,11 @@ GONE = -1
 
 
 def pages_needed(token_count: int, block_size: int) -> int:
-    """worker/src/inference/kv_cache.py:28-33: (0,16)=0, (16,16)=1, (17,16)=2."""
+    """Pages that hold `token_count` tokens: (0,16)=0, (16,16)=1, (17,16)=2
+    (worker/src/inference/kv_cache.py:28-33)."""
     if block_size < 1:
         raise ValueError("block_size must be >= 1")
-    if token_count <= 0:
-        return 0
-    return (token_count + block_size - 1) // block_size
+    return -(-max(0, token_count) // block_size)
 
 
 class CacheView:

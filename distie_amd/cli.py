@@ -31,12 +31,16 @@ def _engine_options(parser: argparse.ArgumentParser) -> None:
     parser.add_argument("--max-seqs", type=int, default=None)
     parser.add_argument("--token-budget", type=int, default=None)
     parser.add_argument("--no-decode-graphs", action="store_true")
+    parser.add_argument("--graph-buckets", default=None, metavar="SIZES",
+                        help="batch sizes that get a captured decode step, comma-separated (default: 1,2,4,8, then "
+                             "every multiple of 8 up to --max-seqs)")
     parser.add_argument("--step-stats", type=int, default=None, help="log a time breakdown every N steps")
     parser.add_argument("--no-packed-weights", action="store_true",
                         help="no second copy of the weights in the matrix cores' order (half the weight memory, "
                              "slower decode)")
     parser.add_argument("--packed-weights", default=None, metavar="ROLES",
-                        help="packed copies only for these products, comma-separated: qkv,attn_out,gate_up,down,head")
+                        help="packed copies only for the products the model's parts name so, comma-separated "
+                             "(this architecture's parts name qkv, attn_out, gate_up, down, head)")
     parser.add_argument("--gpu-mem-fraction", type=float, default=None,
                         help="without --num-blocks: pages of the cache until this share of the card's memory is in use")
     parser.add_argument("--tune-products", action="store_true",
@@ -50,6 +54,7 @@ def _build(args):
     engine = EngineConfig.from_env(
         dtype=args.dtype, block_size=args.block_size, num_blocks=args.num_blocks, max_seqs=args.max_seqs,
         token_budget=args.token_budget, use_graphs=False if args.no_decode_graphs else None,
+        graph_buckets=tuple(int(b) for b in args.graph_buckets.split(",") if b) if args.graph_buckets else None,
         step_stats=args.step_stats, seed=args.seed, packed_weights=False if args.no_packed_weights else (
             tuple(r for r in args.packed_weights.split(",") if r) if args.packed_weights else None),
         gpu_mem_fraction=args.gpu_mem_fraction,

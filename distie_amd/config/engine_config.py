@@ -44,8 +44,12 @@ class EngineConfig:
     token_budget: int = DEFAULT_TOKEN_BUDGET
     max_model_len: Optional[int] = None     # None = the model's max positions
     use_graphs: bool = True
-    # a second copy of the weights in the matrix cores' order, for decode: True, False, or the roles that get one
-    # ("qkv", "attn_out", "gate_up", "down", "head")
+    # batch sizes that get a captured decode step of their own; None = 1, 2, 4, 8, then every multiple of 8 up to
+    # max_seqs (a step is padded up to the next size; one with more rows than the largest runs uncaptured)
+    graph_buckets: Optional[Tuple[int, ...]] = None
+    # a second copy of the weights in the matrix cores' order, for decode: True, False, or the roles that get one.
+    # A role is whatever name a part gives its product in `Ops.prepare_linear(role=...)`; the parts of the Qwen2
+    # decoder name "qkv", "attn_out", "gate_up", "down" and "head", another part may name others
     packed_weights: Union[bool, Tuple[str, ...]] = True
     lookahead: bool = True                  # launch the next decode step before this step's tokens reach the host
     tune_products: bool = False             # at start, let the library time its kernels for a full portion's products
@@ -60,6 +64,11 @@ class EngineConfig:
             raise ValueError("num_blocks must be >= 1")
         if self.gpu_mem_fraction is not None and not 0.0 < self.gpu_mem_fraction <= 1.0:
             raise ValueError("gpu_mem_fraction must be in (0, 1]")
+        if self.graph_buckets is not None:
+            buckets = tuple(sorted({int(b) for b in self.graph_buckets}))
+            if not buckets or buckets[0] < 1:
+                raise ValueError("graph_buckets must be batch sizes >= 1")
+            object.__setattr__(self, "graph_buckets", buckets)
         if not isinstance(self.packed_weights, bool):
             object.__setattr__(self, "packed_weights", tuple(self.packed_weights))
 
@@ -104,6 +113,9 @@ class EngineConfig:
         raw = os.getenv("WORKER_DECODE_GRAPHS", "").strip().lower()
         if raw:
             env["use_graphs"] = raw not in {"0", "false", "no", "off"}
+        raw = os.getenv("WORKER_GRAPH_BUCKETS", "").strip()
+        if raw:
+            env["graph_buckets"] = tuple(int(b) for b in raw.split(","))
         raw = os.getenv("WORKER_GPU_MEM_FRACTION", "").strip()
         if raw:
             env["gpu_mem_fraction"] = float(raw)

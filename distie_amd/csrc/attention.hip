@@ -94,7 +94,7 @@ __global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_generic_kernel(
     const T* __restrict__ qkv, int64_t q_stride, const C* __restrict__ k_cache, const C* __restrict__ v_cache,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_request,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ table_rows, T* __restrict__ out, int heads, int kv_heads,
-    int block_size, float scale, int window) {
+    int block_size, float scale, int window, const float* __restrict__ head_slopes, float score_cap) {
   __shared__ float q_s[D];
   __shared__ float p_s[WAVES][DISTIE_WAVE];
   __shared__ int64_t base_s[WAVES][DISTIE_WAVE];
@@ -115,6 +115,7 @@ __global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_generic_kernel(
   const int first = window > 0 ? max(0, q_pos - window + 1) : 0;
   const int last = q_pos;   // inclusive
   const bool by_page = block_size % 4 == 0 && DISTIE_WAVE % block_size == 0;
+  const float slope = head_slopes != nullptr ? head_slopes[h] : 0.f;
   float m = -INFINITY, l = 0.f;
   float acc[DIMS_PER_LANE];
 #pragma unroll
@@ -129,6 +130,10 @@ __global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_generic_kernel(
       const int page = table[key / block_size];
       base = (static_cast<int64_t>(page) * kv_heads + kh) * block_size * D;
       s = dot_row<C>(q_s, k_cache + base + static_cast<int64_t>(key % block_size) * D) * scale;
+      // what a variant of attention adds to a score (both off for plain attention): a cap that bends large
+      // scores, then a bias by the distance to the key with the head's own slope
+      if (score_cap > 0.f) s = score_cap * tanhf(s / score_cap);
+      s += slope * static_cast<float>(key - q_pos);
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float alpha = m_new == -INFINITY ? 0.f : expf(m - m_new);     // 0 on the first chunk with a key (m = -inf)
@@ -410,18 +415,23 @@ __global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_grouped_f32_kernel(
 }
 
 // qkv: [T, q_stride] with q of head h at columns h*D; out: [T, heads*D]. window = 0: every earlier key.
+// head_slopes (float32 [heads], may be null): score += slope[h] * (key - position); score_cap > 0: the scaled score
+// goes through cap * tanh(score / cap) first. Only this kernel takes the two.
 extern "C" int distie_attention_generic(const void* qkv, int dtype, int64_t q_stride, const void* k_cache,
                                         const void* v_cache, int cache_dtype, const int32_t* positions,
                                         const int32_t* token_request, const int32_t* block_table,
                                         int table_width, const int32_t* table_rows, void* out, int tokens, int heads, int kv_heads,
-                                        int block_size, float scale, int window, hipStream_t stream) {
+                                        int block_size, float scale, int window, const float* head_slopes,
+                                        float score_cap, hipStream_t stream) {
   if (tokens <= 0) return 0;
-  if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size < 1 || table_width < 1 || window < 0)
+  if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size < 1 || table_width < 1 || window < 0 ||
+      score_cap < 0.f)
     return DISTIE_BAD_ARGUMENT;
+  const bool plain_scores = head_slopes == nullptr && score_cap == 0.f;
   if (heads > 65535) return DISTIE_BAD_ARGUMENT;
   dim3 grid(tokens, heads);
   const int group = heads / kv_heads;
-  if (GQ_FITS && dtype == DISTIE_F32 && cache_dtype == DISTIE_F32 && q_stride % 4 == 0 && block_size % 4 == 0 &&
+  if (plain_scores && GQ_FITS && dtype == DISTIE_F32 && cache_dtype == DISTIE_F32 && q_stride % 4 == 0 && block_size % 4 == 0 &&
       DISTIE_WAVE % block_size == 0 && static_cast<int64_t>(tokens) * heads < 2048) {
     // requests that decode, float32: as many heads of a kv head to a workgroup as leaves a workgroup a compute unit
     int per = 1;
@@ -446,13 +456,13 @@ extern "C" int distie_attention_generic(const void* qkv, int dtype, int64_t q_st
         (attn_generic_kernel<T, C, 8><<<grid, DISTIE_WAVE * 8, 0, stream>>>(
             static_cast<const T*>(qkv), q_stride, static_cast<const C*>(k_cache), static_cast<const C*>(v_cache),
             positions, token_request, block_table, table_width, table_rows, static_cast<T*>(out), heads, kv_heads, block_size,
-            scale, window))));
+            scale, window, head_slopes, score_cap))));
   } else {
     DISTIE_DISPATCH(dtype, T, DISTIE_DISPATCH(cache_dtype, C,
         (attn_generic_kernel<T, C, 1><<<grid, DISTIE_WAVE, 0, stream>>>(
             static_cast<const T*>(qkv), q_stride, static_cast<const C*>(k_cache), static_cast<const C*>(v_cache),
             positions, token_request, block_table, table_width, table_rows, static_cast<T*>(out), heads, kv_heads, block_size,
-            scale, window))));
+            scale, window, head_slopes, score_cap))));
   }
   return launch_status();
 }

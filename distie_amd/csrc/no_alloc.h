@@ -17,8 +17,12 @@
 // reports both numbers.
 //
 // The array (DISTIE_ARGMAX_STATIC_ENTRIES * 8 bytes = 8 KiB) exists once on every GPU the library runs
-// on and stays until the process ends. Its address on a device is looked up at the first call on that
-// device. Every call on a GPU uses that GPU's one array, which keeps what the last call left: nothing
+// on and stays until the process ends. Its address on a device is looked up once, by
+// `distie_argmax_static_prepare` (with that device current) or by the first call of
+// `distie_argmax_static` on the device. The lookup is no stream operation and must not happen while a
+// stream captures: a caller that captures calls `distie_argmax_static_prepare` (or the entry point
+// itself once, eagerly) on the device first; `distie_argmax_static` on a capturing stream of a device
+// that was not prepared launches nothing and returns hipErrorStreamCaptureUnsupported. Every call on a GPU uses that GPU's one array, which keeps what the last call left: nothing
 // in it has to start at zero, since a call writes every entry before it reads it; but two calls that
 // overlap on one GPU (different streams, or threads) race on it. Calls that follow each other on one
 // stream are safe.
@@ -32,4 +36,5 @@
 #define DISTIE_ARGMAX_STATIC_MAX_ROWS 1024
 
 extern "C" int distie_argmax_static(const float* logits, int32_t* out, int rows, int vocab, hipStream_t stream);
+extern "C" int distie_argmax_static_prepare(void);      // 0, or a hipError_t
 extern "C" void distie_argmax_static_limits(int* max_rows, int* max_entries);

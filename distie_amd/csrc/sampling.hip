@@ -124,14 +124,17 @@ constexpr int STATIC_MAX_DEVICES = 64;
 static void* scratch_of_device[STATIC_MAX_DEVICES];
 static std::mutex scratch_lookup;
 
-// -> 0 and the array's address on the current device, or a hipError_t
-static int static_scratch(void** address) {
+// -> 0 and the array's address on the current device, or a hipError_t. The address is looked up once per device;
+// that lookup is no operation a capturing stream may see, so with `may_look_up` false (the caller's stream
+// captures) a device whose address is not known yet is an error instead.
+static int static_scratch(void** address, bool may_look_up) {
   int device = -1;
   hipError_t status = hipGetDevice(&device);
   if (status != hipSuccess) return static_cast<int>(status);
   if (device < 0 || device >= STATIC_MAX_DEVICES) return static_cast<int>(hipErrorInvalidDevice);
   std::lock_guard<std::mutex> hold(scratch_lookup);
   if (scratch_of_device[device] == nullptr) {
+    if (!may_look_up) return static_cast<int>(hipErrorStreamCaptureUnsupported);
     void* found = nullptr;
     status = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
     if (status != hipSuccess) return static_cast<int>(status);
@@ -140,6 +143,11 @@ static int static_scratch(void** address) {
   }
   *address = scratch_of_device[device];
   return 0;
+}
+
+extern "C" int distie_argmax_static_prepare(void) {
+  void* base = nullptr;
+  return static_scratch(&base, true);
 }
 
 extern "C" void distie_argmax_static_limits(int* max_rows, int* max_entries) {
@@ -157,8 +165,10 @@ extern "C" int distie_argmax_static(const float* logits, int32_t* out, int rows,
     return launch_status();
   }
   if (static_cast<int64_t>(rows) * parts > DISTIE_ARGMAX_STATIC_ENTRIES) return DISTIE_TOO_LARGE;
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) capturing = hipStreamCaptureStatusNone;
   void* base = nullptr;
-  const int status = static_scratch(&base);
+  const int status = static_scratch(&base, capturing == hipStreamCaptureStatusNone);
   if (status != 0) return status;
   // every entry that the second launch reads is written by the first: nothing has to be cleared
   float* piece_value = static_cast<float*>(base);

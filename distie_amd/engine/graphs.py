@@ -36,15 +36,21 @@ from .batch import StepEntry
 _log = logging.getLogger(__name__)
 
 
-def decode_buckets(max_batch: int) -> Tuple[int, ...]:
-    """(32) -> 1,2,4,8,16,24,32; (5) -> 1,2,4,5; (1) -> 1
-    (worker/tests/test_batch_decode.py:50-56)."""
+def decode_buckets(max_batch: int, chosen: Optional[Sequence[int]] = None) -> Tuple[int, ...]:
+    """Batch sizes that get a captured step of their own. By default the reference's rule
+    (worker/src/inference/qwen2/batch_decode.py:43-48, vectors in worker/tests/test_batch_decode.py:50-56):
+    (32) -> 1,2,4,8,16,24,32; (5) -> 1,2,4,5; (1) -> 1. `chosen` (`EngineConfig.graph_buckets`) replaces the
+    rule: sizes above `max_batch` are dropped, and steps with more rows than the largest left run uncaptured."""
     if max_batch < 1:
         raise ValueError("max_batch must be >= 1")
-    sizes = {b for b in (1, 2, 4, 8) if b < max_batch}
-    sizes.update(range(16, max_batch, 8))
-    sizes.add(max_batch)
-    return tuple(sorted(sizes))
+    if chosen is not None:
+        sizes = sorted({int(b) for b in chosen})
+        if not sizes or sizes[0] < 1:
+            raise ValueError("graph_buckets must be batch sizes >= 1")
+        return tuple(b for b in sizes if b <= max_batch) or (max_batch,)
+    small = [b for b in (1, 2, 4, 8) if b < max_batch]          # powers of two below the maximum,
+    eights = list(range(16, max_batch, 8))                      # then every multiple of 8 below it,
+    return tuple(small + eights + [max_batch])                  # and the maximum itself
 
 
 def bucket_for(buckets: Sequence[int], rows: int) -> int:
@@ -71,10 +77,10 @@ class DecodeGraphs:
     RETRY_AFTER_STEPS = 512     # after a failure, steps run uncaptured for so long before a capture is tried again
     MAX_FAILURES = 3            # ... and after so many failures for good
 
-    def __init__(self, runner, max_batch: int) -> None:
+    def __init__(self, runner, max_batch: int, buckets: Optional[Sequence[int]] = None) -> None:
         self.runner = runner
-        self.buckets = decode_buckets(max_batch)
-        self.max_batch = max_batch
+        self.buckets = decode_buckets(max_batch, buckets)
+        self.max_batch = self.buckets[-1]
         self._made: Dict[int, _Bucket] = {}
         self._pool = None
         self.replays = 0

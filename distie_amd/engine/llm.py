@@ -65,12 +65,13 @@ class Trace:
 
 class LLM:
     def __init__(self, model: Union[str, Path, None] = None, *, config=None, random_weights: bool = False,
-                 seed: int = 0, device: str = "cuda:0", ops=None, engine: Optional[EngineConfig] = None,
-                 **options) -> None:
+                 seed: int = 0, weights_std: float = 0.02, device: str = "cuda:0", ops=None,
+                 engine: Optional[EngineConfig] = None, **options) -> None:
         """`model`: a folder with config.json and model.safetensors. Without it, `config` (a typed
         configuration or the dict of a config.json) and `random_weights=True` make a model with
         random weights on the device (drawn from `seed`, which is also the engine's seed for sampling
-        unless `options` or `engine` name another). `options` are fields of `EngineConfig`. `ops` is the kernel
+        unless `options` or `engine` name another, with the spread `weights_std`: the model that
+        `write_random_model` writes for the same configuration, seed and spread). `options` are fields of `EngineConfig`. `ops` is the kernel
         surface; by default the HIP kernels, which need the GPU."""
         if engine is None:
             options.setdefault("seed", seed)          # one seed for random weights and for the requests' draws
@@ -91,7 +92,7 @@ class LLM:
         if model is not None and not random_weights:
             load_into(self.model, model, ops.device, self.dtype)
         elif random_weights:
-            random_into(self.model, seed, ops.device, self.dtype)
+            random_into(self.model, seed, ops.device, self.dtype, std=weights_std)
         else:
             raise ValueError("a config without a model folder needs random_weights=True")
         spec = self.model.spec
@@ -116,12 +117,13 @@ class LLM:
         self._picked = None           # pinned host buffer for the sampled ids
         self._ahead_failed = None     # (plan, error) of a step planned ahead whose launch raised
         self.steps_ahead = 0          # steps launched before the tokens of the step before were known
+        self.last_logits = None       # of the step completed last: a view that a later step may overwrite (for checks)
         self._outputs: Dict[Hashable, RequestOutput] = {}     # until `generate`, `stream` or `take_output` hands them out
         if ec.use_graphs and hasattr(ops, "graphs_supported") and ops.graphs_supported():
             if self.model.capturable:
                 from .graphs import DecodeGraphs
 
-                self.runner.graphs = DecodeGraphs(self.runner, ec.max_seqs)
+                self.runner.graphs = DecodeGraphs(self.runner, ec.max_seqs, ec.graph_buckets)
             else:
                 names = sorted({type(p).__name__ for p in self.model.parts() if not p.capturable})
                 _log.info("decode steps are not captured: %s cannot be recorded into a graph", ", ".join(names))
@@ -232,6 +234,7 @@ class LLM:
             t2 = time.perf_counter()
             sampling = [p for p in plan.portions if p.samples]
             drawn: List[Optional[int]] = [None] * len(plan.portions)
+            self.last_logits = logits
             if sampling:
                 chosen = self.sampler.sample_device(
                     logits, [p.request.params.temperature for p in sampling], [p.request.seed for p in sampling],
@@ -292,6 +295,16 @@ class LLM:
         self._ahead = None
         self.scheduler.requeue(p.request for p in ahead_plan.portions)
 
+    def _forget_ahead(self) -> None:
+        """When every request ended in the step that was being completed, the step launched behind it is
+        worth nothing, and the loop ends without another turn that would drop it: let go of its plan, its
+        requests and its view of a captured step's logits here. (If one of its requests is still seated
+        the step is needed and stays.)"""
+        if self._ahead is not None and not any(p.request.phase is Phase.SEATED for p in self._ahead[0].portions):
+            self._ahead = None
+        if self._ahead_failed is not None and not self.scheduler.has_work():
+            self._ahead_failed = None
+
     def _to_host(self, chosen: torch.Tensor):
         """Start the copy of the sampled ids to the host; the returned function waits for it."""
         if chosen.device.type != "cuda":
@@ -344,6 +357,7 @@ class LLM:
                 del self._outputs[rid]
         for rid in mine:
             self._outputs.pop(rid, None)
+        self._forget_ahead()
 
     def generate(self, prompts: Seq[Seq[int]], params=None) -> List[RequestOutput]:
         """Token ids in, `RequestOutput`s out, in the order of the prompts. `params`: one
@@ -351,6 +365,7 @@ class LLM:
         ids = self._submit_all(prompts, params)
         while self.scheduler.has_work():
             self.run_step()
+        self._forget_ahead()
         if self.stats is not None:
             self.stats.flush()
         return [self._outputs.pop(i) for i in ids]
@@ -396,4 +411,7 @@ class LLM:
         return Trace(token_ids=chosen, logits=kept[:len(chosen)].clone())
 
     def close(self) -> None:
+        self.last_logits = None
+        self._ahead = None
+        self._ahead_failed = None
         self.runner.graphs = None

@@ -96,6 +96,7 @@ class StepPlan:
     # For a step planned ahead (`Scheduler.schedule_ahead`): portion i continues the request of portion
     # `feeds[i]` of the step before, whose drawn token is not known to the host yet.
     feeds: Optional[Tuple[int, ...]] = None
+    gave_way: bool = False     # a request gave way while this step was planned
 
     @property
     def num_tokens(self) -> int:
@@ -244,12 +245,14 @@ class Scheduler:
                 self._leave(request, None)
 
     # ------------------------------------------------------------- planning a step
-    def _seat_arrivals(self, draft: _Draft) -> None:
+    def _seat_arrivals(self, draft: _Draft, spare_each: int = 0) -> None:
+        """`spare_each`: pages that must stay free for every request already seated."""
         while self._queue and len(self._seated) < self.max_seqs and draft.left > 0:
             request = self._queue[0]
             # seated by the pages of everything known of it (scheduler.py:196-211), though only the pages
             # of the portion that runs now are taken
-            if self.cache.slots.num_free < 1 or not self.cache.can_reserve(request.request_id, request.num_tokens):
+            if self.cache.slots.num_free < 1 or not self.cache.can_reserve(
+                    request.request_id, request.num_tokens, spare=spare_each * len(self._seated)):
                 return
             count = min(request.num_tokens, draft.left)
             self._queue.popleft()
@@ -282,7 +285,7 @@ class Scheduler:
                 draft.put(request, request.num_computed, count)
         if not someone_gave_way:          # else whoever gave way would come straight back
             self._seat_arrivals(draft)
-        return StepPlan(tuple(draft.portions))
+        return StepPlan(tuple(draft.portions), gave_way=someone_gave_way)
 
     def schedule_ahead(self, plan: StepPlan) -> Optional[StepPlan]:
         """The step after `plan` (launched, not yet completed), planned before `plan`'s tokens are
@@ -292,7 +295,10 @@ class Scheduler:
         their places in `plan`; those that reach their length with the pending token are left out);
         the next portions of prompts that `plan` has not finished; and queued requests for which a
         seat, a state slot and pages are free now (the seat of a request that ends with the pending
-        token is free one step later). Nobody gives way for it: if a page is missing the answer is
+        token is free one step later, and a page must stay free for every request already seated, so that
+        an arrival does not take the page an older request needs at its next page boundary; none is seated
+        behind a step in which somebody gave way, or whoever gave way would come straight back and give way
+        again). Nobody gives way for it: if a page is missing the answer is
         None and the plain schedule decides. A request that turns out to have ended with the pending
         token (end of sequence, cancelled) has a row of the next step computed for nothing;
         `complete` skips it."""
@@ -320,7 +326,8 @@ class Scheduler:
                 return None
             self.cache.reserve(request.request_id, count)
             draft.put(request, portion.end, count)
-        self._seat_arrivals(draft)
+        if not plan.gave_way:
+            self._seat_arrivals(draft, spare_each=1)
         if not draft.portions:
             return None
         return StepPlan(tuple(draft.portions), feeds=tuple(draft.feeds))

@@ -1,3 +1,3 @@
-from .interface import BatchMeta, GroupMeta, Ops
+from .interface import BatchMeta, GroupMeta, Ops, ScoreExtras
 
-__all__ = ["BatchMeta", "GroupMeta", "Ops"]
+__all__ = ["BatchMeta", "GroupMeta", "Ops", "ScoreExtras"]

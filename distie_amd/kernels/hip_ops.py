@@ -54,7 +54,27 @@ def _check(status: int, name: str) -> None:
     raise KernelError(f"{name}: launch failed with HIP error {status}")
 
 
-class PartialSums:
+def _written(t: torch.Tensor):
+    """How often `t` has been written in place, as far as anyone can know: torch's own count (every in-place
+    torch operation on the tensor or on a view of it) and the count of this module's kernels that write their
+    argument (`_mark_written`)."""
+    return (t._version, getattr(t, "_distie_version", 0))
+
+
+def _mark_written(t: torch.Tensor) -> None:
+    t._distie_version = getattr(t, "_distie_version", 0) + 1
+
+
+class _NotATensorYet:
+    """What `HipOps` hands out in place of a tensor. Anything asked of it that only a tensor has raises
+    with the way out, instead of an AttributeError far from the cause."""
+
+    def __getattr__(self, name):
+        raise KernelError(f"{type(self).__name__} is a result of the HIP kernels that is not a tensor yet (asked for "
+                          f".{name}): a part that computes on the values itself calls ops.dense(value) first")
+
+
+class PartialSums(_NotATensorYet):
     """The result of a matrix product whose reduction was cut into slices: float32
     [slices, rows, columns], to be added in order by whoever reads it. `linear` returns it for
     small batches (a sum across workgroups inside the product would cost more than the product);
@@ -72,10 +92,12 @@ class PartialSums:
         return self.data.shape[0]
 
 
-class PendingNorm:
+class PendingNorm(_NotATensorYet):
     """rmsnorm(residual) * weight, not computed yet: for steps of few rows the product that reads it computes
     it itself, in front of its own work (`distie_decode_norm_product`); anything else sees the finished
-    tensor through `HipOps.dense`. Valid as long as the residual it was made from is unchanged."""
+    tensor through `HipOps.dense`. Valid as long as the residual it was made from is unchanged: a write in
+    place by torch (also through a view) or by one of this module's kernels between `rmsnorm` and the use is
+    found out and raises, instead of a norm of the wrong values."""
 
     def __init__(self, residual: torch.Tensor, weight: torch.Tensor, eps: float, dtype: torch.dtype) -> None:
         self.residual = residual
@@ -84,14 +106,14 @@ class PendingNorm:
         self.dtype = dtype
         self.shape = residual.shape
         self.device = residual.device
-        self.version = getattr(residual, "_distie_version", 0)
+        self.version = _written(residual)
 
     def check(self) -> None:
-        if getattr(self.residual, "_distie_version", 0) != self.version:
+        if _written(self.residual) != self.version:
             raise KernelError("a normed value was used after the residual stream it was made from had changed")
 
 
-class PendingProduct:
+class PendingProduct(_NotATensorYet):
     """x W^T + bias for few rows of x, not computed yet: if the next thing that happens to it is the sum into
     the residual stream, the product adds itself to the stream in place (`distie_decode_product_residual`) and
     never exists as a tensor; anything else sees the finished tensor through `HipOps.dense`."""
@@ -257,7 +279,7 @@ class HipOps(Ops):
                 raise KernelError(f"attention kernels take even head sizes up to 256, not {head_dim}")
             lib = ctypes.CDLL(str(build.ensure(f"attn_d{head_dim}")))
             lib.distie_attention_generic.argtypes = [_P, _I, _L, _P, _P, _I, _P, _P, _P, _I, _P, _P,
-                                                     _I, _I, _I, _I, _F, _I, _P]
+                                                     _I, _I, _I, _I, _F, _I, _P, _F, _P]
             lib.distie_attention_prefill_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I,
                                                           _F, _I, _I, _P, _P, _P, _I, _P]
             lib.distie_attention_prefill_f32.argtypes = lib.distie_attention_prefill_bf16.argtypes
@@ -292,6 +314,7 @@ class HipOps(Ops):
             raise KernelError("scatter_int32 takes int32 tensors, one value for each index")
         _check(self._ops.distie_scatter_i32(table.data_ptr(), index.data_ptr(), value.data_ptr(), index.numel(),
                                             table.numel(), self._stream()), "scatter_i32")
+        _mark_written(table)
 
     def embed(self, ids, table):
         self._own(ids, table)
@@ -343,7 +366,7 @@ class HipOps(Ops):
         _check(self._ops.distie_rmsnorm(residual.data_ptr(), delta.data_ptr(), _code(delta), slices,
                                         weight.data_ptr(), _code(weight), out.data_ptr(), _CODES[out_dtype],
                                         residual.shape[0], residual.shape[1], eps, self._stream()), "add_rmsnorm")
-        residual._distie_version = getattr(residual, "_distie_version", 0) + 1
+        _mark_written(residual)
         return out
 
     def _product_into_residual(self, product: PendingProduct, residual: torch.Tensor) -> None:
@@ -356,7 +379,7 @@ class HipOps(Ops):
         _check(self._ops.distie_decode_product_residual(
             x.data_ptr(), packed.data_ptr(), bias.data_ptr() if bias is not None else None, residual.data_ptr(),
             M, N, K, self._stream()), "decode_product_residual")
-        residual._distie_version = getattr(residual, "_distie_version", 0) + 1
+        _mark_written(residual)
 
     def dense(self, x):
         """The finished tensor of a value that an operation here returned in a form of its own (partial sums,
@@ -556,6 +579,8 @@ class HipOps(Ops):
             lib.distie_lib_linear.restype = ctypes.c_int
             lib.distie_lib_counts.argtypes = [ctypes.POINTER(ctypes.c_long), ctypes.POINTER(ctypes.c_long)]
             lib.distie_lib_counts.restype = None
+            lib.distie_lib_more_counts.argtypes = [ctypes.POINTER(ctypes.c_long)] * 3
+            lib.distie_lib_more_counts.restype = None
             with torch.cuda.device(self.device):
                 _check(lib.distie_lib_init(self._device_index), "lib_init")
             self._lib = lib
@@ -566,6 +591,14 @@ class HipOps(Ops):
         made, timed = ctypes.c_long(0), ctypes.c_long(0)
         self._library().distie_lib_counts(ctypes.byref(made), ctypes.byref(timed))
         return made.value, timed.value
+
+    def library_counts(self) -> dict:
+        """`held`: shapes the library holds a plan for now; `asked`: how often it was asked to rank its kernels
+        (row counts of one class of 32 share a choice); `refused`: timed candidates dropped because their
+        result differed from that of the library's first choice."""
+        held, asked, refused = ctypes.c_long(0), ctypes.c_long(0), ctypes.c_long(0)
+        self._library().distie_lib_more_counts(ctypes.byref(held), ctypes.byref(asked), ctypes.byref(refused))
+        return {"held": held.value, "asked": asked.value, "refused": refused.value}
 
     LIBRARY_UNSUPPORTED = -3
 
@@ -750,10 +783,13 @@ class HipOps(Ops):
             slots.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _code(k_cache),
             inv_freq.data_ptr() if inv_freq is not None else None, pairs, T, num_heads, num_kv_heads, head_dim,
             meta.block_size, 1 if write else 0, self._stream()), "rope_kv_write")
+        _mark_written(out)
         return out
 
     def paged_attention(self, qkv, meta: BatchMeta, group, k_cache, v_cache, num_heads, num_kv_heads, head_dim,
-                        scale, window):
+                        scale, window, extras=None):
+        """The matrix-core kernels and the tiled float32 kernel compute plain attention; a step with
+        `extras` goes to the wave-per-token kernel, which takes slopes and a cap (any types and sizes)."""
         if not scale > 0:
             raise KernelError(f"paged_attention: the scale of the scores must be positive, not {scale}")
         qkv = self.dense(qkv)
@@ -768,8 +804,14 @@ class HipOps(Ops):
             raise KernelError("paged_attention: tensors do not match the batch")
         rows_ptr = rows.data_ptr() if rows is not None else None
         out = torch.empty((T, num_heads * head_dim), dtype=qkv.dtype, device=self.device)
+        plain = extras is None or extras.plain
+        slopes, cap = (None, 0.0) if plain else (extras.head_slopes, float(extras.score_cap or 0.0))
+        if slopes is not None:
+            self._own(slopes)
+            if slopes.dtype != torch.float32 or tuple(slopes.shape) != (num_heads,):
+                raise KernelError("paged_attention: head_slopes must be float32 [num_heads]")
         bf16 = qkv.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16
-        if bf16 and meta.block_size % 16 == 0 and head_dim % 16 == 0:
+        if plain and bf16 and meta.block_size % 16 == 0 and head_dim % 16 == 0:
             # how the step is launched, and its buffers for partial results, are the same for every layer
             # with these sizes: worked out once per step (the layers run one after the other, so they can
             # share the buffers)
@@ -797,7 +839,7 @@ class HipOps(Ops):
                     "attention_prefill_bf16")
             return out
         f32 = qkv.dtype == torch.float32 and k_cache.dtype == torch.float32
-        if f32 and meta.max_q >= self.PREFILL_F32_MIN_TOKENS and meta.block_size % 16 == 0 and \
+        if plain and f32 and meta.max_q >= self.PREFILL_F32_MIN_TOKENS and meta.block_size % 16 == 0 and \
                 qkv.shape[1] % 4 == 0 and lib.distie_attention_prefill_f32_fits():
             # portions of prompts in float32: the tiled kernel on float32 matrix products takes the whole step
             key = ("attention_f32", int(window or 0), num_heads, head_dim, meta.max_kv, self.PREFILL_PARTS,
@@ -817,7 +859,7 @@ class HipOps(Ops):
             qkv.data_ptr(), _code(qkv), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), _code(k_cache),
             meta.positions.data_ptr(), meta.token_request.data_ptr(), table.data_ptr(), table.shape[1], rows_ptr,
             out.data_ptr(), T, num_heads, num_kv_heads, meta.block_size, float(scale), int(window or 0),
-            self._stream()), "attention_generic")
+            slopes.data_ptr() if slopes is not None else None, cap, self._stream()), "attention_generic")
         return out
 
     def _attention_plan(self, lib, meta: BatchMeta, T, num_heads, num_kv_heads, head_dim, window) -> dict:

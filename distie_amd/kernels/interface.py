@@ -56,6 +56,28 @@ class BatchMeta:
     scratch: dict = field(default_factory=dict)   # what an implementation computes once per step (cos/sin tables)
 
 
+@dataclass(frozen=True)
+class ScoreExtras:
+    """What a variant of attention does to a score beyond scale, causal mask and window; everything None
+    for plain attention. An implementation's kernel that does not take a field that is set refuses the call
+    (it never ignores it), so a new variant is a kernel added behind this argument, not a changed signature.
+
+    score(i, j) = q_i . k_j * scale; with `score_cap` c: c * tanh(score / c); with `head_slopes` s:
+    + s[h] * (j - i), a bias by the distance to the key with a slope of the head's own (a position
+    encoding that needs no rotation)."""
+
+    head_slopes: Optional[torch.Tensor] = None      # float32 [H] on the device
+    score_cap: Optional[float] = None               # > 0
+
+    def __post_init__(self):
+        if self.score_cap is not None and not self.score_cap > 0:
+            raise ValueError("score_cap must be positive")
+
+    @property
+    def plain(self) -> bool:
+        return self.head_slopes is None and self.score_cap is None
+
+
 class Ops(abc.ABC):
     device: torch.device
     # True while the engine warms or records a captured step: launches then cost the host nothing when the
@@ -78,7 +100,15 @@ class Ops(abc.ABC):
 
     @abc.abstractmethod
     def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
-        """float32 [T, C] -> out_dtype [T, C]; statistics in float32."""
+        """float32 [T, C] -> out_dtype [T, C]; statistics in float32.
+
+        As with `linear`, an implementation may return the result in a form of its own that only its own
+        operations read (the HIP kernels leave the norm of few rows to the product that reads it: the value
+        is then not computed yet, and stays valid only until `x` is next written in place, which the
+        implementation finds out and refuses). A part hands the result on to `linear`, `linear_silu_mul`,
+        `linear_rope_kv_write`, `linear_f32out` or `gather_rows`; a part that computes on the values itself
+        (indexing, `.float()`, any torch operation) calls `ops.dense(result)` first. The same holds for
+        `add_rmsnorm`."""
 
     @abc.abstractmethod
     def add_rmsnorm(self, residual: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor,
@@ -91,12 +121,15 @@ class Ops(abc.ABC):
 
         An implementation may return the product in a form of its own that only its
         `add_rmsnorm`, `silu_mul`, `rope_kv_write`, `linear`, `paged_attention` and `gather_rows`
-        read (the HIP kernels return partial sums over slices of K for small batches); parts
-        hand the result on to those operations and do nothing else with it."""
+        read (the HIP kernels return partial sums over slices of K for small batches, or, for few
+        rows, a product not yet computed that adds itself to the residual stream if `add_rmsnorm`
+        is what comes next); parts hand the result on to those operations, or as the `delta` of a
+        `ResidualStream`, and do nothing else with it. A part that computes on the values itself
+        calls `ops.dense(result)` first."""
 
     def dense(self, x):
-        """The plain tensor of a result that `linear` returned in a form of its own; any other
-        tensor as it is. For parts that compute on a product's values themselves."""
+        """The plain tensor of a result that `linear`, `rmsnorm` or `add_rmsnorm` returned in a form of
+        its own; any other tensor as it is. For parts that compute on the values themselves."""
         return x
 
     def prepare_linear(self, weight: torch.Tensor, gated: bool = False, rotary=None, role: Optional[str] = None) -> None:
@@ -137,9 +170,10 @@ class Ops(abc.ABC):
     @abc.abstractmethod
     def paged_attention(self, qkv: torch.Tensor, meta: BatchMeta, group: int, k_cache: torch.Tensor,
                         v_cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
-                        scale: float, window: Optional[int]) -> torch.Tensor:
+                        scale: float, window: Optional[int], extras: Optional[ScoreExtras] = None) -> torch.Tensor:
         """softmax(q k^T * scale) v over the cached keys 0..position of each token (the last
-        `window` of them on a windowed layer), read through the block table -> act [T, H*D]."""
+        `window` of them on a windowed layer), read through the block table -> act [T, H*D].
+        `extras`: what a variant adds to the scores (`ScoreExtras`); None for plain attention."""
 
     @abc.abstractmethod
     def silu_mul(self, gate_up: torch.Tensor) -> torch.Tensor:

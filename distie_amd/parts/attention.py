@@ -18,6 +18,7 @@ from typing import Optional, Tuple
 import torch
 
 from ..config.model_config import PartSpec
+from ..kernels.interface import ScoreExtras
 from .base import PAGE, Mixer, PagedTensors, ParamSpec, TensorDecl, build_part, register_part
 
 
@@ -58,10 +59,12 @@ class Attention(Mixer):
         self.out_bias = bool(p.get("out_bias", False))
         self.window = p.get("window")
         self.scale = float(p.get("scale", self.head_dim ** -0.5))
+        self.score_cap = p.get("score_cap")        # None for this architecture: scores are not bent
         if self.num_heads % self.num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
         self.position = build_part("position", p.get("position") or PartSpec("none"))
         self.qkv_weight = self.qkv_bias_t = self.out_weight = self.out_bias_t = None
+        self.extras = None                         # what the position encoding or a cap adds to the scores
 
     def cache_requirement(self):
         return PagedKV(self.num_kv_heads, self.head_dim, self.window)
@@ -92,6 +95,11 @@ class Attention(Mixer):
         if self.out_bias:
             self.out_bias_t = tensors["o_proj.bias"].float().contiguous()
         self.position.to_device(self.out_weight.device)
+        slopes = self.position.head_slopes(self.num_heads)
+        if slopes is not None or self.score_cap is not None:
+            if slopes is not None:
+                slopes = slopes.to(device=self.out_weight.device, dtype=torch.float32).contiguous()
+            self.extras = ScoreExtras(slopes, None if self.score_cap is None else float(self.score_cap))
 
     def prepare(self, ops) -> None:
         ops.prepare_linear(self.qkv_weight, rotary=(self.num_heads, self.num_kv_heads, self.head_dim),
@@ -112,7 +120,7 @@ class Attention(Mixer):
                                        self.position.rotary(), self.num_heads, self.num_kv_heads, self.head_dim,
                                        writes_cache)
         mixed = ops.paged_attention(qkv, ctx.meta, cache.group, k_cache, v_cache, self.num_heads,
-                                    self.num_kv_heads, self.head_dim, self.scale, self.window)
+                                    self.num_kv_heads, self.head_dim, self.scale, self.window, self.extras)
         return ops.linear(mixed, self.out_weight, self.out_bias_t)
 
 

@@ -7,7 +7,8 @@ them through `load`, and computes through the kernel surface (`Ops`).
 Families and their interfaces, in short:
 
 * `embedding`: `Embedding.forward(ops, ids, meta)` -> float32 [T, C], the start of the residual stream;
-* `position`: `PositionEncoding.rotary()` -> inverse frequencies for the fused rotation (or None) and
+* `position`: `PositionEncoding.rotary()` -> inverse frequencies for the fused rotation (or None),
+  `head_slopes(num_heads)` -> per-head slopes of a bias by distance inside attention (or None), and
   `on_embedding(ops, hidden, meta)` for encodings that act on the embeddings;
 * `norm`: `Norm.apply(ops, x_f32, out_dtype)` and `Norm.add_apply(ops, residual_f32, delta, out_dtype)`;
 * `mixer`: `Mixer.cache_requirement()` -> `PagedTensors` | `FixedState` | None,
@@ -170,6 +171,11 @@ class PositionEncoding(Part):
     def rotary(self) -> Optional[torch.Tensor]:
         """float32 [rotary_dim / 2] inverse frequencies for the rotation fused into the
         cache write, or None if this encoding does not rotate."""
+        return None
+
+    def head_slopes(self, num_heads: int) -> Optional[torch.Tensor]:
+        """float32 [num_heads] for an encoding that biases every score by the distance to the key,
+        score += slope[h] * (key position - query position) (`ScoreExtras.head_slopes`); None otherwise."""
         return None
 
     def on_embedding(self, ops, hidden: torch.Tensor, meta) -> None:

@@ -18,6 +18,7 @@ from typing import Dict, Iterator, List, Mapping, Tuple
 
 import torch
 
+from .random_init import standard_normal
 from .safetensors_io import SafetensorsFile, model_files, write_safetensors
 
 
@@ -83,26 +84,30 @@ def load_into(model, model_dir, device, engine_dtype: torch.dtype) -> None:
             f.close()
 
 
-def random_tensor(name: str, spec, generator: torch.Generator, std: float, device) -> torch.Tensor:
-    """Matrices, embeddings and biases ~ N(0, std); norm weights 1; zeros where asked.
-    Always drawn in float32 so that every precision sees the same numbers."""
+def random_tensor(name: str, spec, seed: int, std: float, device) -> torch.Tensor:
+    """Matrices, embeddings and biases ~ N(0, std); norm weights 1; zeros where asked. Always float32, and a
+    function of (seed, name, element) alone (`random_init`): the same bits on the CPU and on the device, in
+    any order of drawing, so that every user of the random-weights mode sees one model for one seed."""
     if spec.init == "ones":
         return torch.ones(spec.shape, dtype=torch.float32, device=device)
     if spec.init == "zeros":
         return torch.zeros(spec.shape, dtype=torch.float32, device=device)
     if spec.init == "int":
         return torch.zeros(spec.shape, dtype=torch.int32, device=device)
-    return torch.randn(spec.shape, generator=generator, dtype=torch.float32, device=device) * std
+    count = 1
+    for n in spec.shape:
+        count *= int(n)
+    return torch.mul(standard_normal(seed, name, count, device), std).view(tuple(spec.shape))
 
 
 def random_into(model, seed: int, device, engine_dtype: torch.dtype, std: float = 0.02) -> None:
-    """Random weights straight into the parts, drawn on `device` (no file)."""
-    generator = torch.Generator(device=device).manual_seed(seed)
+    """Random weights straight into the parts, drawn on `device` (no file): tensor for tensor what
+    `write_random_model` writes for the same seed, stored in the engine's precision."""
     specs = model.param_specs()
     store = torch.bfloat16 if engine_dtype == torch.bfloat16 else torch.float32
 
     def fetch(name: str) -> torch.Tensor:
-        tensor = random_tensor(name, specs[name], generator, std, device)
+        tensor = random_tensor(name, specs[name], seed, std, device)
         return tensor if not tensor.dtype.is_floating_point else tensor.to(store)
 
     model.load_tensors(fetch)
@@ -110,8 +115,7 @@ def random_into(model, seed: int, device, engine_dtype: torch.dtype, std: float 
 
 def write_random_model(config, out_dir, seed: int, dtype: str = "float32", std: float = 0.02) -> Path:
     """Random-weights mode: write a model folder (config.json, model.safetensors) from a
-    typed configuration and a seed. Tensors are drawn in name order of the model's
-    declaration, in float32, then stored as `dtype`."""
+    typed configuration and a seed. Tensors are drawn in float32 (`random_tensor`), then stored as `dtype`."""
     from ..engine.model import Model  # local import: weights <-> engine
 
     store = {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype]
@@ -121,14 +125,13 @@ def write_random_model(config, out_dir, seed: int, dtype: str = "float32", std: 
     config_json["torch_dtype"] = dtype
     (out_dir / "config.json").write_text(json.dumps(config_json, indent=1))
     specs = Model.declare(config.model_spec())
-    generator = torch.Generator().manual_seed(seed)
 
     def dtype_of(spec) -> torch.dtype:
         return torch.int32 if spec.init == "int" else store
 
     def tensors() -> Iterator[Tuple[str, torch.Tensor]]:
         for name, spec in specs.items():
-            yield name, random_tensor(name, spec, generator, std, "cpu").to(dtype_of(spec))
+            yield name, random_tensor(name, spec, seed, std, "cpu").to(dtype_of(spec))
 
     write_safetensors(out_dir / "model.safetensors",
                       [(n, dtype_of(s), tuple(s.shape)) for n, s in specs.items()],

@@ -147,3 +147,65 @@ def check_generation(weights, cfg, prompt, token_ids, temperature=0.0, seed=0, t
                 near += 1
         ids.append(int(token))
     return near
+
+
+def run_and_keep_logits(llm, prompts, params):
+    """`LLM.generate`, keeping the logits every token was drawn from: -> (outputs, {request: [(position, row)]})."""
+    kept = {}
+    seen = {}
+    sample = llm.sampler.sample_device
+    complete = llm.scheduler.complete
+
+    def spy_sample(logits, *args):
+        seen["logits"] = logits.clone()             # queued behind the step, ahead of whatever overwrites its buffer
+        return sample(logits, *args)
+
+    def spy_complete(plan, drawn):
+        rows = [p for p in plan.portions if p.samples]
+        for i, portion in enumerate(rows):
+            kept.setdefault(portion.request.request_id, []).append((portion.end - 1, seen["logits"][i]))
+        return complete(plan, drawn)
+
+    llm.sampler.sample_device = spy_sample
+    llm.scheduler.complete = spy_complete
+    try:
+        outs = llm.generate(prompts, params)
+    finally:
+        llm.sampler.sample_device = sample
+        llm.scheduler.complete = complete
+    return outs, kept
+
+
+def check_generation_in_two_halves(weights, cfg, prompt, token_ids, rows, dtype, temperature=0.0, seed=0):
+    """For a precision whose logits are too far from the oracle's to judge a draw by them: (1) the logits the
+    engine drew from (`rows`: [(position, float32 row)], in the order of the tokens) are the oracle's for the
+    tokens the engine saw, within the bounds of `check_logits`; (2) every token is the plain draw from the
+    engine's own row: its argmax (lowest index among equals), or the first index whose cumulative softmax
+    weight exceeds the request's n-th uniform number. A request that gave way and recomputed has drawn some
+    tokens twice; the rows of the last time count."""
+    ids = list(prompt) + list(token_ids[:-1])
+    last = {}
+    for position, row in rows:
+        last[position] = row
+    positions = list(range(len(prompt) - 1, len(ids)))
+    assert sorted(last) == positions, "a token was drawn from a row at another place"
+    got = torch.stack([last[p] for p in positions]).float().cpu()
+    want = oracle(weights, cfg, ids)[positions]
+    diff = got - want
+    scale = want.abs().max().item()
+    if dtype == torch.float32:
+        assert diff.abs().max().item() < FP32_TOL
+    else:
+        assert diff.abs().max().item() < scale / 16 and diff.pow(2).mean().sqrt().item() < scale / 64
+    for n, token in enumerate(token_ids):
+        row = got[n].double()
+        if temperature <= 0:
+            assert token == int(row.argmax()), f"token {n}: {token} is not the largest of the engine's own logits"
+            continue
+        w = torch.exp((row - row.max()) / temperature)
+        c = torch.cumsum(w, 0) / w.sum()
+        u = plain_uniform(seed, n)
+        pick = int((c > u).nonzero()[0])
+        if token != pick:          # float32 sums of the kernel against float64 here: only at an interval's very edge
+            below = float(c[token - 1]) if token else 0.0
+            assert below - 1e-5 <= u <= float(c[token]) + 1e-5, f"token {n}: {token} drawn, the plain draw is {pick}"

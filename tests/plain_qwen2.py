@@ -81,7 +81,7 @@ def rope_cos_sin(positions: torch.Tensor, head_dim: int, theta: float, dtype=tor
     :103), and only the results take the dtype of the activations (:105): at position 2,000 a
     float32 angle is off by up to 1e-4 rad, which is part of what the reference computes.
     (`angle_dtype=float64` is for tests of the formula itself.)"""
-    freqs = positions.to(angle_dtype)[:, None] * rope_inv_freq(head_dim, theta, angle_dtype)[None, :]
+    freqs = positions.to(angle_dtype)[:, None] * rope_inv_freq(head_dim, theta, angle_dtype).to(positions.device)[None, :]
     emb = torch.cat((freqs, freqs), dim=-1)
     return emb.cos().to(dtype), emb.sin().to(dtype)
 
@@ -105,11 +105,11 @@ def repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
     return x[:, :, None, :].expand(t, kh, n_rep, d).reshape(t, kh * n_rep, d)
 
 
-def visibility(q_len: int, window) -> torch.Tensor:
+def visibility(q_len: int, window, device=None) -> torch.Tensor:
     """[q, k] bool: key k visible to query q iff k <= q (worker/src/inference/qwen2/model.py:128-135)
     and, on a windowed layer, q - k < window (this build's rule)."""
-    q = torch.arange(q_len)[:, None]
-    k = torch.arange(q_len)[None, :]
+    q = torch.arange(q_len, device=device)[:, None]
+    k = torch.arange(q_len, device=device)[None, :]
     seen = k <= q
     if window is not None:
         seen = seen & (q - k < window)
@@ -124,7 +124,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window=None) ->
     k = repeat_kv(k, n_rep)
     v = repeat_kv(v, n_rep)
     scores = torch.einsum("qhd,khd->hqk", q, k) * (d ** -0.5)
-    scores = scores.masked_fill(~visibility(t, window)[None], float("-inf"))
+    scores = scores.masked_fill(~visibility(t, window, q.device)[None], float("-inf"))
     weights = torch.softmax(scores, dim=-1)
     return torch.einsum("hqk,khd->qhd", weights, v)
 
@@ -168,15 +168,21 @@ def decoder_layer(x, w: dict, index: int, positions, cfg: dict, window, angle_dt
 
 
 def forward(w: dict, cfg: dict, ids, dtype=torch.float32, first_position: int = 0,
-            angle_dtype=torch.float32) -> torch.Tensor:
+            angle_dtype=torch.float32, rows=None) -> torch.Tensor:
     """Token ids [T] -> logits [T, vocab] of one whole sequence:
-    worker/src/inference/qwen2/model.py:305-314 (tied head: :302-303)."""
+    worker/src/inference/qwen2/model.py:305-314 (tied head: :302-303). It runs where the weights
+    lie. `rows`: only these positions go through the final norm and the head (the reference's batched
+    forward selects rows before the head too: model.py:376-379), so that a long sequence against a large
+    vocabulary fits in memory."""
     w = {k: v.to(dtype) for k, v in w.items()}
-    ids = torch.as_tensor(ids, dtype=torch.long)
+    device = w["model.embed_tokens.weight"].device
+    ids = torch.as_tensor(ids, dtype=torch.long, device=device)
     x = w["model.embed_tokens.weight"][ids]
-    positions = torch.arange(first_position, first_position + ids.shape[0])
+    positions = torch.arange(first_position, first_position + ids.shape[0], device=device)
     for index, window in enumerate(layer_windows(cfg)):
         x = decoder_layer(x, w, index, positions, cfg, window, angle_dtype)
+    if rows is not None:
+        x = x[torch.as_tensor(rows, dtype=torch.long, device=device)]
     x = rms_norm(x, w["model.norm.weight"], float(cfg["rms_norm_eps"]))
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
     return x @ head.T

@@ -257,3 +257,70 @@ def test_a_half_precision_file(tmp_path):
         assert torch.equal(model.embedding, weights["model.embed_tokens.weight"].to(engine_dtype))
         assert torch.equal(model.blocks[1].feed_forward.down_weight,
                            weights["model.layers.1.mlp.down_proj.weight"].to(engine_dtype))
+
+
+def test_random_values_are_a_function_of_seed_name_and_index():
+    """The bits behind the random weights, written out again with numpy's unsigned integers: splitmix64 of
+    base + index * golden ratio, top 16 bits an interval of the normal quantiles, next 24 a place in it."""
+    import numpy as np
+
+    from distie_amd.weights import random_init as ri
+
+    base = ri.stream_base(7, "model.layers.0.mlp.down_proj.weight")
+    with np.errstate(over="ignore"):
+        u = np.uint64
+        z = np.arange(5, 5 + 1000, dtype=np.uint64) * u(0x9E3779B97F4A7C15) + u(base)
+        z = (z ^ (z >> u(30))) * u(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> u(27))) * u(0x94D049BB133111EB)
+        z = z ^ (z >> u(31))
+    got = ri.mixed_bits(base, 5, 1000, "cpu").numpy().view(np.uint64)
+    assert np.array_equal(got, z)
+    # a value is its interval's lower edge plus the place times the width, each rounded once
+    values = ri.standard_normal(7, "model.layers.0.mlp.down_proj.weight", 1005, "cpu")[5:].numpy()
+    lower, width = (t.numpy() for t in ri._tables("cpu"))
+    interval = (z >> u(48)).astype(np.int64)
+    place = ((z >> u(24)) & u(0xFFFFFF)).astype(np.float32) * np.float32(2.0 ** -24)
+    assert np.array_equal(values, lower[interval] + (width[interval] * place).astype(np.float32))
+    # chunks change nothing, names and seeds do
+    old = ri.CPU_CHUNK
+    try:
+        ri.CPU_CHUNK = 97
+        assert np.array_equal(ri.standard_normal(7, "model.layers.0.mlp.down_proj.weight", 1005, "cpu")[5:].numpy(), values)
+    finally:
+        ri.CPU_CHUNK = old
+    assert not np.array_equal(ri.standard_normal(8, "model.layers.0.mlp.down_proj.weight", 1005, "cpu")[5:].numpy(), values)
+    assert not np.array_equal(ri.standard_normal(7, "model.layers.1.mlp.down_proj.weight", 1005, "cpu")[5:].numpy(), values)
+
+
+def test_random_values_are_normal():
+    from distie_amd.weights import random_init as ri
+
+    x = ri.standard_normal(1, "w", 2_000_000, "cpu").double()
+    assert abs(x.mean().item()) < 3e-3
+    assert abs(x.std().item() - 1.0) < 3e-3
+    assert abs((x ** 3).mean().item()) < 1e-2                     # symmetric
+    assert abs((x ** 4).mean().item() - 3.0) < 3e-2               # the normal's fourth moment
+    assert abs((x.abs() > 1.959964).double().mean().item() - 0.05) < 1e-3
+    assert x.abs().max().item() < 4.9 and x.abs().max().item() > 4.0
+    # neighbours in a tensor are not correlated
+    assert abs((x[1:] * x[:-1]).mean().item()) < 3e-3
+
+
+def test_an_engine_with_random_weights_is_the_model_of_the_written_folder(tmp_path):
+    """One generator: `LLM(config=..., random_weights=True, seed=s)` holds tensor for tensor what
+    `write_random_model(config, dir, s)` writes, so the plain implementation reading the folder is the
+    oracle of the engine that never saw it."""
+    from distie_amd import LLM, StepEntry
+    from torch_ops import TorchOps
+
+    for cfg in (plain.TINY_A, plain.TINY_B):
+        config = config_from_dict(cfg)
+        folder = write_random_model(config, tmp_path / f"m{cfg['hidden_size']}", seed=11, dtype="float32", std=0.1)
+        weights = plain.read_weights(folder)
+        llm = LLM(config=config, random_weights=True, seed=11, weights_std=0.1, dtype="fp32", ops=TorchOps(), block_size=4, num_blocks=32)
+        ids = [3, 1, 4, 1, 5, 9, 2, 6, 5, 3]
+        got = llm.step([StepEntry("a", ids, list(range(len(ids))))])
+        want = plain.forward(weights, cfg, ids, torch.float64).float()
+        assert (got - want).abs().max().item() < 1e-4
+        from_folder = LLM(folder, dtype="fp32", ops=TorchOps(), block_size=4, num_blocks=32)
+        assert torch.equal(from_folder.step([StepEntry("a", ids, list(range(len(ids))))]), got)

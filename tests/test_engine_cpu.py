@@ -114,19 +114,33 @@ def test_wanted_rows_and_empty_want(setup):
     assert (logits[2] - wb[11]).abs().max() < FP32_TOL
 
 
-def test_filling_a_step_does_not_grow_with_the_contexts():
-    """64 requests that decode: what the host does to describe the step is the same at 2,000 and at 32,000
-    cached tokens a request, since the block tables live on the device and only changed entries travel."""
-    import time
+class _CountingTable(list):
+    """A request's block table that counts the entries anyone looks at."""
 
+    touched = 0
+
+    def __getitem__(self, key):
+        got = super().__getitem__(key)
+        _CountingTable.touched += len(got) if isinstance(key, slice) else 1
+        return got
+
+    def __iter__(self):
+        _CountingTable.touched += len(self)
+        return super().__iter__()
+
+
+def test_filling_a_step_does_not_grow_with_the_contexts():
+    """64 requests, decoding or with a portion of 40 tokens: what the host looks at to describe the step is the
+    same at 2,000 and at 32,000 cached tokens a request, since the block tables live on the device and only
+    changed entries travel. Counted in table entries touched and entries sent, not in seconds."""
     import numpy as np
 
     from distie_amd.cache import CacheManager
     from distie_amd.engine.batch import BatchBuilder
     from distie_amd.parts import PagedKV
 
-    def seconds(context):
-        cache = CacheManager([PagedKV(1, 16), PagedKV(1, 16, 4096)], 16, 64 * (context // 16 + 2), 64, device="cpu",
+    def work(context, new):
+        cache = CacheManager([PagedKV(1, 16), PagedKV(1, 16, 4096)], 16, 64 * (context // 16 + 8), 64, device="cpu",
                              allocate=False)
         builder = BatchBuilder(cache, 40000, "cpu", 100)
         entries = []
@@ -134,18 +148,84 @@ def test_filling_a_step_does_not_grow_with_the_contexts():
             cache.add(r)
             cache.reserve(r, context)
             cache.commit(r, context)
-            cache.reserve(r, 1)
-            entries.append(StepEntry(r, [1], [0]))
+            entries.append(StepEntry(r, [1] * new, [0]))
         builder.flush_tables()
-        host = np.empty(int(builder.layout(64, 64, 64)[-1]), dtype=np.int32)
-        best = 1e9
-        for _ in range(5):
-            began = time.perf_counter()
-            for _ in range(20):
-                builder.fill(host, entries)
-                builder.flush_tables()
-            best = min(best, time.perf_counter() - began)
-        return best
+        for r in range(64):
+            cache.reserve(r, new)
+            state = cache.request(r)
+            state.tables = [_CountingTable(t) for t in state.tables]
+        host = np.empty(int(builder.layout(64 * new, 64, 64)[-1]), dtype=np.int32)
+        sent = sum(len(cache.groups[g].changed) for g in range(2))
+        _CountingTable.touched = 0
+        builder.fill(host, entries)
+        builder.flush_tables()
+        return _CountingTable.touched, sent
 
-    short, long = seconds(2000), seconds(32000)
-    assert long < 1.5 * short + 1e-3, (short, long)
+    for new in (1, 40):
+        short, long = work(2000 - 8, new), work(32000 - 8, new)
+        assert short == long, (new, short, long)
+        touched, sent = short
+        assert touched <= 64 * 2 * (new // 16 + 2) and sent <= 64 * 2 * (new // 16 + 1)
+
+
+def test_the_fields_of_a_step_as_numbers():
+    """The reference's vector of its batch description (worker/tests/test_qwen2_batch.py:50-59): two requests
+    at pages of 4 tokens, "a" with 2 new tokens behind none in pages [3, 0], "b" with 1 new token behind 5
+    in pages [1, 5] -> positions [0, 1, 5], slots [12, 13, 21], prefix sums [0, 2, 3], tables [[3, 0], [1, 5]],
+    last rows [1, 2], longest portion 2, longest context 6. Here the cached lengths travel as they are
+    ([2, 6]; the reference sends their prefix sums [0, 2, 8]) and the tables are rows of the device table
+    named by each request's state slot."""
+    import numpy as np
+
+    from distie_amd.cache import CacheManager
+    from distie_amd.engine.batch import BatchBuilder
+    from distie_amd.parts import PagedKV
+
+    cache = CacheManager([PagedKV(2, 8), PagedKV(2, 8)], 4, 8, 4, device="cpu")
+    builder = BatchBuilder(cache, 16, "cpu", 100)
+    assert builder.table_width == 4
+    (group,) = cache.groups
+    held = group.pool.allocate(8)                       # every page is taken, so the chosen ones are held
+    group.pool.free([p for p in held if p not in (3, 0, 1, 5)])
+    a, b = cache.add("a"), cache.add("b")
+    for entry, pages, cached in ((a, [3, 0], 0), (b, [1, 5], 5)):
+        entry.tables[0] = list(pages)
+        entry.num_cached = cached
+        for i, page in enumerate(pages):
+            cache._note(group, entry.slot, i, page)
+    cache.check()
+    entries = [StepEntry("a", [7, 8], [1]), StepEntry("b", [9], [0])]
+    host = np.full(64, -7, dtype=np.int32)
+    offsets, T, B, R, max_q, max_kv, cu_q, past = builder.fill(host, entries)
+    assert (T, B, R, max_q, max_kv) == (3, 2, 2, 2, 6)
+    field = lambda i: host[offsets[i]:offsets[i + 1]].tolist()
+    assert field(0) == [7, 8, 9]                        # token ids
+    assert field(1) == [0, 1, 5]                        # positions
+    assert field(2) == [0, 0, 1]                        # request of each token
+    assert field(3) == [0, 2, 3]                        # prefix sums of the new tokens
+    assert field(4) == [2, 6]                           # cached after the step
+    assert field(5) == [a.slot, b.slot]                 # state slots = rows of the device tables
+    assert field(6) == [1, 2]                           # rows whose logits are wanted: the last of each
+    assert field(7) == [12, 13, 21]                     # page * 4 + place in the page
+    assert cu_q.tolist() == [0, 2, 3] and past.tolist() == [0, 5]
+    assert int(offsets[-1]) == 3 * 3 + 3 + 2 + 2 + 2 + 3
+    # the device tables: the changed entries go along, rows by state slot, -1 where nothing is held
+    ids, meta, want = builder.build(entries)
+    table = meta.groups[0].block_table
+    assert table[a.slot].tolist() == [3, 0, -1, -1] and table[b.slot].tolist() == [1, 5, -1, -1]
+    assert table[cache.sink_slot, 0] == group.sink_page == 8
+    assert meta.table_rows.tolist() == [a.slot, b.slot] and want.tolist() == [1, 2]
+    assert meta.positions.tolist() == [0, 1, 5] and meta.groups[0].slots.tolist() == [12, 13, 21]
+    assert (meta.max_q, meta.max_kv, meta.all_decode) == (2, 6, False)
+    # two rows of padding, as a captured step of four would have: position 0 of the sink page and slot
+    offsets, T, B, R, *_ = builder.fill(host, [StepEntry("b", [9], [0])], pad_requests=2, want_all=True)
+    field = lambda i: host[offsets[i]:offsets[i + 1]].tolist()
+    assert (T, B, R) == (3, 3, 3)
+    assert field(1) == [5, 0, 0] and field(3) == [0, 1, 2, 3] and field(4) == [6, 1, 1]
+    assert field(5) == [b.slot, 4, 4] and field(6) == [0, 1, 2] and field(7) == [21, 32, 32]
+    # what the reference refuses (test_qwen2_batch.py:61-68): a table too short for the new tokens, an empty step
+    b.tables[0] = [1]
+    with pytest.raises(ValueError):
+        builder.fill(host, [StepEntry("b", [9], [0])])
+    with pytest.raises(ValueError):
+        builder.fill(host, [])

@@ -11,7 +11,8 @@ import torch
 import plain_qwen2 as plain
 from distie_amd import LLM, SamplingParams
 from distie_amd.engine.batch import StepEntry
-from engine_util import build_runner, check_generation, check_logits, make_model_dir, random_ids
+from engine_util import (build_runner, check_generation, check_generation_in_two_halves, check_logits, make_model_dir,
+                         random_ids, run_and_keep_logits)
 
 pytestmark = pytest.mark.gpu
 
@@ -51,6 +52,43 @@ def test_greedy_and_temperature_mixed_in_one_batch(tmp_path, name, graphs, looka
         assert llm.runner.graphs.captured and llm.runner.graphs.failures == 0
     llm.cache.check()
     assert all(f == 48 for f in llm.cache.free_pages())
+
+
+BF16_WORKLOADS = {
+    "B": (plain.TINY_B, 8, (1, 9, 23, 40), 12, 7),
+    "C": (plain.TINY_C, 16, (3, 30, 70, 18, 44), 20, 33),
+}
+
+
+@pytest.mark.parametrize("name", sorted(BF16_WORKLOADS))
+@pytest.mark.parametrize("graphs,lookahead,pages", [(False, False, 48), (True, True, 48), (True, True, None)])
+def test_bfloat16_generation_through_the_scheduler(tmp_path, name, graphs, lookahead, pages):
+    """The serving precision through the whole loop: greedy and temperature requests in one batch, prompts in
+    portions, captured steps launched ahead, and (pages=None) a pool so tight that requests give way and
+    recompute. bfloat16 logits lie too far from the oracle's to judge a draw by the oracle's logits, so the
+    check has two halves: the logits each token was drawn from are the oracle's for the tokens the engine saw,
+    within the bfloat16 bounds, and each token is the plain draw from the engine's own logits, exactly."""
+    cfg, block, lengths, new, budget = BF16_WORKLOADS[name]
+    folder, weights = make_model_dir(tmp_path, cfg, seed=45, dtype=torch.bfloat16)
+    prompts = [random_ids(cfg, n, 300 + n) for n in lengths]
+    params = [SamplingParams(max_new_tokens=new, temperature=0.7 if i % 2 == 0 else 0.0, seed=200 + i)
+              for i in range(len(prompts))]
+    tight = pages is None
+    if tight:                       # the two longest requests fit, all of them do not
+        pages = sum(-(-(n + new) // block) for n in sorted(lengths)[-2:]) + 1
+    llm = LLM(folder, dtype="bf16", block_size=block, num_blocks=pages, token_budget=budget, use_graphs=graphs,
+              lookahead=lookahead)
+    outs, kept = run_and_keep_logits(llm, prompts, params)
+    for prompt, sp, out in zip(prompts, params, outs):
+        assert len(out.token_ids) == new and out.finish_reason == "length"
+        check_generation_in_two_halves(weights, cfg, prompt, out.token_ids, kept[out.request_id], torch.bfloat16,
+                                       sp.temperature, sp.seed)
+    assert (sum(o.preemptions for o in outs) > 0) == tight
+    assert (llm.steps_ahead > 0) == lookahead
+    if graphs:
+        assert llm.runner.graphs.captured and llm.runner.graphs.failures == 0
+    llm.cache.check()
+    assert all(f == pages for f in llm.cache.free_pages()) and llm.cache.slots.num_free == llm.cache.num_slots
 
 
 def test_a_tight_pool_makes_requests_give_way_and_changes_nothing(tmp_path):

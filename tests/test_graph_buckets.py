@@ -15,6 +15,24 @@ def test_decode_buckets():
         decode_buckets(0)
 
 
+def test_chosen_buckets_replace_the_rule():
+    assert decode_buckets(32, (8, 1, 8, 64)) == (1, 8)            # sorted, once each, none above the maximum
+    assert decode_buckets(4, (16, 32)) == (4,)                      # nothing left: the maximum alone
+    with pytest.raises(ValueError):
+        decode_buckets(32, (0, 4))
+    with pytest.raises(ValueError):
+        decode_buckets(32, ())
+
+
+def test_engine_config_holds_the_buckets():
+    from distie_amd.config import EngineConfig
+
+    assert EngineConfig().graph_buckets is None
+    assert EngineConfig(graph_buckets=[16, 2, 2]).graph_buckets == (2, 16)
+    with pytest.raises(ValueError):
+        EngineConfig(graph_buckets=[0])
+
+
 def test_bucket_for():
     buckets = decode_buckets(32)
     assert [bucket_for(buckets, n) for n in (1, 3, 8, 9, 17, 32)] == [1, 4, 8, 16, 24, 32]

@@ -164,6 +164,7 @@ def test_steps_planned_ahead_change_nothing(tiny):
         ahead = engine(folder, **options)
         got = ahead.generate(prompts, params)
         assert ahead.steps_ahead > 0
+        assert ahead._ahead is None and ahead._ahead_failed is None      # nothing is kept of a step launched for nothing
         assert [o.token_ids for o in got] == [o.token_ids for o in want]
         assert [o.finish_reason for o in got] == [o.finish_reason for o in want]
         assert got[1].finish_reason == "stop" and got[0].finish_reason == "length"
@@ -293,3 +294,46 @@ def test_step_stats_and_forgotten_records(tiny):
     assert all(row["host"] >= row["launch"] > 0 for row in summary.values())
     assert "device" not in summary["decode"]                       # no GPU here: host parts only
     assert "host=" in llm.stats.format()
+
+
+def test_nothing_is_kept_of_a_step_launched_for_nothing(tiny):
+    """The only request stops at an end-of-sequence token while the step after is already launched: the loop
+    ends without another turn, and the engine lets go of that step's plan and logits all the same."""
+    cfg, folder, weights = tiny
+    prompt = random_ids(cfg, 9, 5)
+    stop = plain_greedy(weights, cfg, prompt, 6)[4]
+    llm = engine(folder)
+    (out,) = llm.generate([prompt], SamplingParams(max_new_tokens=12, eos_id=stop))
+    assert out.finish_reason == "stop" and llm.steps_ahead > 0
+    assert llm._ahead is None
+    emitted = list(llm.stream([prompt], SamplingParams(max_new_tokens=12, eos_id=stop)))
+    assert emitted[-1].finished and llm._ahead is None
+    llm.add_request(prompt, SamplingParams(max_new_tokens=12))
+    for _ in range(3):
+        llm.run_step()
+    assert llm._ahead is not None
+    llm.close()
+    assert llm._ahead is None
+
+
+def test_tokens_are_the_plain_draws_from_the_logits_they_were_drawn_from(tiny):
+    """The check in two halves that the bfloat16 runs on the GPU use, here on the test double: the logits each
+    token was drawn from are the oracle's for the tokens the engine saw, and each token is the plain draw from
+    those logits; also for requests that gave way and recomputed."""
+    from engine_util import check_generation_in_two_halves, run_and_keep_logits
+
+    cfg, folder, weights = tiny
+    prompts = [random_ids(cfg, n, 90 + n) for n in (5, 11, 17, 8)]
+    params = [SamplingParams(max_new_tokens=10, temperature=0.7 if i % 2 else 0.0, seed=40 + i) for i in range(4)]
+    for options in ({}, {"num_blocks": 8}):
+        llm = engine(folder, **options)
+        outs, kept = run_and_keep_logits(llm, prompts, params)
+        assert (sum(o.preemptions for o in outs) > 0) == bool(options)
+        for prompt, sp, out in zip(prompts, params, outs):
+            check_generation_in_two_halves(weights, cfg, prompt, out.token_ids, kept[out.request_id], torch.float32,
+                                           sp.temperature, sp.seed)
+    # the check notices a wrong token
+    with pytest.raises(AssertionError):
+        wrong = list(outs[0].token_ids)
+        wrong[3] = (wrong[3] + 1) % cfg["vocab_size"]
+        check_generation_in_two_halves(weights, cfg, prompts[0], wrong, kept[outs[0].request_id], torch.float32, 0.0, 40)

@@ -15,8 +15,8 @@ from distie_amd.config import LayerCall, LayerSpec, ModelSpec, PartSpec, registe
 from distie_amd.engine.batch import BatchBuilder, StepEntry
 from distie_amd.engine.model import Model
 from distie_amd.engine.runner import ModelRunner
-from distie_amd.parts import (FeedForward, FixedState, Mixer, PagedKV, PagedTensors, ParamSpec, ResidualStream, StepContext, build_part,
-                              register_part)
+from distie_amd.parts import (FeedForward, FixedState, Mixer, PagedKV, PagedTensors, ParamSpec, PositionEncoding, ResidualStream,
+                              StepContext, build_part, register_part)
 from torch_ops import TorchOps
 
 
@@ -172,7 +172,7 @@ class DecayMixer(Mixer):
 
     def forward(self, ops, x, ctx, cache, writes_cache):
         meta = ctx.meta
-        u = x.float() @ self.weight.T
+        u = ops.dense(x).float() @ self.weight.T        # computes on the values itself: the finished tensor first
         out = torch.empty_like(u)
         slots = meta.state_slots.tolist()
         cu = meta.cu_q.tolist()
@@ -315,13 +315,115 @@ def test_toy_architecture_with_a_state_mixer_is_registered_built_and_stepped(ops
     assert (got - want_b).abs().max() < 1e-4
 
 
+@pytest.mark.gpu
+def test_toy_state_mixer_in_bfloat16_on_the_hip_kernels():
+    """The same toy in the serving precision, where a step of few rows hands a mixer values that are not
+    tensors yet (the norm is left to the product that reads it): the toy asks for the finished tensor with
+    `ops.dense`, as the interface says, and one that does not is told so."""
+    from distie_amd.config import config_from_dict
+    from distie_amd.kernels.hip_ops import HipOps, KernelError
+
+    ops = HipOps("cuda:0")
+    register_part("mixer", "test_decay", DecayMixer)
+    register_architecture("ToyForCausalLM", ToyConfig)
+    cfg = config_from_dict({"architectures": ["ToyForCausalLM"], "hidden": 32, "vocab": 70, "decay": 0.8})
+    model = Model(cfg.model_spec())
+    gen = torch.Generator().manual_seed(3)
+    weights = {n: (torch.ones(s.shape) if s.init == "ones" else torch.randn(s.shape, generator=gen) * 0.2).bfloat16().float()
+               for n, s in model.param_specs().items()}
+    model.load_tensors(lambda name: weights[name].to(ops.device).bfloat16())
+    cache = CacheManager(model.cache_requirements(), 16, 16, 4, device=ops.device, dtype=torch.bfloat16)
+    runner = ModelRunner(model, cache, ops, torch.bfloat16, 256)
+    a = torch.randint(0, 70, (40,), generator=gen).tolist()
+    want = toy_plain(weights, cfg, a).float()
+    rows = [runner.step([StepEntry("a", a[:20], list(range(20)))])]            # 20 rows: tensors all the way
+    rows += [runner.step([StepEntry("a", a[i:i + 1], [0])]) for i in range(20, 40)]      # 1 row: pending values
+    got = torch.cat(rows).float().cpu()
+    scale = want.abs().max().item()
+    assert (got - want).abs().max().item() < scale / 16 and (got - want).pow(2).mean().sqrt().item() < scale / 64
+    runner.finish("a")
+
+    class Careless(DecayMixer):
+        def forward(self, ops, x, ctx, cache, writes_cache):
+            return x.float().to(torch.bfloat16)
+
+    register_part("mixer", "test_decay", Careless)
+    try:
+        careless = Model(cfg.model_spec())
+        careless.load_tensors(lambda name: weights[name].to(ops.device).bfloat16())
+        runner = ModelRunner(careless, cache, ops, torch.bfloat16, 256)
+        with pytest.raises(KernelError, match="ops.dense"):
+            runner.step([StepEntry("b", a[:1], [0])])
+    finally:
+        register_part("mixer", "test_decay", DecayMixer)
+
+
+# ---------------------------------------------------------------------------------------------
+# a position encoding that lives inside attention: a bias on every score by the distance to the key, with a
+# slope per head, and scores bent by a cap; both reach the kernels as `ScoreExtras`
+# ---------------------------------------------------------------------------------------------
+class DistanceBias(PositionEncoding):
+    def head_slopes(self, num_heads):
+        return torch.tensor([2.0 ** (-8.0 * (h + 1) / num_heads) for h in range(num_heads)])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv_heads,dim,window,cap", [(4, 2, 16, None, 3.0), (3, 1, 32, 6, None), (8, 2, 128, None, 5.0)])
+def test_attention_with_a_bias_by_distance_and_capped_scores(ops, heads, kv_heads, dim, window, cap, dtype):
+    if dtype == torch.bfloat16 and ops.device.type != "cuda":
+        pytest.skip("the test double is run in float32")
+    register_part("position", "test_distance_bias", DistanceBias)
+    hidden = 48
+    spec = PartSpec("attention", "a.", {"hidden_size": hidden, "num_heads": heads, "num_kv_heads": kv_heads, "head_dim": dim,
+                                        "qkv_bias": True, "window": window, "score_cap": cap,
+                                        "position": PartSpec("test_distance_bias")})
+    part = build_part("mixer", spec)
+    w = {name: rnd(*pspec.shape, seed=40 + i, scale=0.5 if "q_proj" in name or "k_proj" in name else 0.2)
+         for i, (name, pspec) in enumerate(part.param_specs().items())}
+    w = {k: v.to(dtype).float() for k, v in w.items()}
+    part.load({k: v.to(ops.device).to(dtype if v.dim() == 2 else torch.float32) for k, v in w.items()})
+    part.prepare(ops)
+    assert part.extras is not None and part.extras.score_cap == cap and part.extras.head_slopes.shape == (heads,)
+    lengths = [70, 1, 20]          # 70: beyond one chunk of 64 keys
+    cache, meta = context(ops, [part.cache_requirement()], lengths, block=16, dtype=dtype)
+    x = rnd(sum(lengths), hidden, seed=6).to(dtype)
+    got = dense(ops, part.forward(ops, x.to(ops.device), StepContext(meta, dtype), cache.layer(0)["mixer"], True)).float().cpu()
+    slopes = DistanceBias(PartSpec("test_distance_bias")).head_slopes(heads).double()
+    at = 0
+    for n in lengths:
+        xs = x[at:at + n].double()
+        q = (xs @ w["q_proj.weight"].double().T + w["q_proj.bias"].double()).view(n, heads, dim)
+        k = (xs @ w["k_proj.weight"].double().T + w["k_proj.bias"].double()).view(n, kv_heads, dim)
+        v = (xs @ w["v_proj.weight"].double().T + w["v_proj.bias"].double()).view(n, kv_heads, dim)
+        if dtype == torch.bfloat16:                 # what the cache holds
+            q, k, v = (t.to(dtype).double() for t in (q, k, v))
+        k, v = plain.repeat_kv(k, heads // kv_heads), plain.repeat_kv(v, heads // kv_heads)
+        s = torch.einsum("ihd,jhd->hij", q, k) * dim ** -0.5
+        if cap is not None:
+            s = cap * torch.tanh(s / cap)
+        i, j = torch.arange(n)[:, None], torch.arange(n)[None, :]
+        s = s + slopes[:, None, None] * (j - i).double()
+        seen = (j <= i) if window is None else (j <= i) & (i - j < window)
+        s = s.masked_fill(~seen, float("-inf"))
+        mixed = torch.einsum("hij,jhd->ihd", torch.softmax(s, -1), v).reshape(n, heads * dim)
+        if dtype == torch.bfloat16:
+            mixed = mixed.to(dtype).double()
+        want = mixed @ w["o_proj.weight"].double().T
+        err = (got[at:at + n].double() - want).abs().max().item()
+        size = want.abs().max().item()               # float32: 1e-5 of the largest value, which is well above 1 here
+        assert err < (1e-5 * max(size, 1.0) if dtype == torch.float32 else 0.02 * size + 1e-3), (n, err, size)
+        at += n
+    # the slopes matter: without them the result is another
+    part.extras = None
+    plain_scores = dense(ops, part.forward(ops, x.to(ops.device), StepContext(meta, dtype), cache.layer(0)["mixer"], True)).float().cpu()
+    assert (plain_scores - got).abs().max().item() > 1e-2
+
+
 # ---------------------------------------------------------------------------------------------
 # a second toy architecture: positions learned and added to the embeddings (attention without rotation),
 # and in one layer a routed feed-forward (the best of three experts of different widths, scaled by its
 # router weight) beside a dense one in the other: chosen layer by layer by the configuration
 # ---------------------------------------------------------------------------------------------
-from distie_amd.parts import PositionEncoding   # noqa: E402
-
 
 class LearnedPositions(PositionEncoding):
     def __init__(self, spec):

@@ -1,0 +1,175 @@
+"""The regime that the benchmark times, checked against the plain implementation: the layer sizes of the
+1.5B model, contexts beyond 2,048 tokens, 8 and 64 requests, prompts fed in portions of the token budget,
+decoding through captured steps that are launched ahead of the host (worker/tests/test_model_runner.py:72-80
+holds the graph path against the eager one at tiny sizes; here the sizes are the benchmark's and the judge
+is the plain model). Also: what two ways of cutting the same tokens leave in the cache
+(worker/tests/test_qwen2_batch.py:106-109, 185-189), and the random-weights mode on the device."""
+
+import pytest
+import torch
+
+import plain_qwen2 as plain
+from distie_amd import LLM, SamplingParams, StepEntry
+from engine_util import build_runner, make_model_dir, random_ids, run_and_keep_logits
+
+pytestmark = pytest.mark.gpu
+
+SIZES_1_5B = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 2, "hidden_size": 1536,
+              "num_attention_heads": 12, "num_key_value_heads": 2, "head_dim": 128, "intermediate_size": 8960,
+              "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
+              "max_position_embeddings": 4096, "hidden_act": "silu"}
+NEW_TOKENS = 41          # the token drawn from the prompt's last row, then 40 decode steps
+
+
+@pytest.fixture(scope="module")
+def model_1_5b(tmp_path_factory):
+    folder, weights = make_model_dir(tmp_path_factory.mktemp("regime"), SIZES_1_5B, seed=29, std=0.03, dtype=torch.bfloat16)
+    on_device = {k: v.to("cuda", torch.float64) for k, v in weights.items()}
+    return folder, on_device
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+def test_the_regime_the_benchmark_times(model_1_5b, dtype):
+    folder, weights = model_1_5b
+    llm = LLM(folder, dtype=dtype, block_size=16, num_blocks=64 * 136 + 8, max_seqs=64, token_budget=2048,
+              max_model_len=4096, use_graphs=True, lookahead=True)
+    graphs = llm.runner.graphs
+    assert graphs is not None
+    for batch in (8, 64):
+        replays, ahead = graphs.replays, llm.steps_ahead
+        # prompts of 2,048 tokens and a few more: no portion ends where a prompt ends, steps hold the end of one
+        # prompt beside the start of the next, and requests that were admitted early decode beside them
+        prompts = [random_ids(SIZES_1_5B, 2048 + (5 * i) % 13, 100 * batch + i) for i in range(batch)]
+        params = [SamplingParams(max_new_tokens=NEW_TOKENS, ignore_eos=True, temperature=0.9 if i % 4 == 3 else 0.0,
+                                 seed=i) for i in range(batch)]
+        outs, kept = run_and_keep_logits(llm, prompts, params)
+        torch.cuda.synchronize()
+        assert graphs.failures == 0 and graphs.replays > replays + 30, "decode steps did not run captured"
+        assert llm.steps_ahead > ahead + 30, "decode steps were not launched ahead"
+        assert (batch, 3072) in graphs.captured_contexts, graphs.captured_contexts
+        for prompt, out, asked in zip(prompts, outs, params):
+            assert out.finish_reason == "length" and len(out.token_ids) == NEW_TOKENS
+            ids = prompt + out.token_ids[:-1]            # the tokens the engine saw, whatever it drew
+            rows = list(range(len(prompt) - 1, len(ids)))
+            want = plain.forward(weights, SIZES_1_5B, ids, torch.float64, rows=rows).float()
+            mine = kept[out.request_id]
+            assert [position for position, _ in mine] == rows
+            got = torch.stack([row for _, row in mine])
+            diff = got - want
+            scale = want.abs().max().item()
+            if dtype == "fp32":
+                assert diff.abs().max().item() < 1e-4 * max(1.0, scale), (batch, out.request_id, diff.abs().max().item())
+            else:
+                assert diff.abs().max().item() < scale / 16, (batch, out.request_id, diff.abs().max().item(), scale)
+                assert diff.pow(2).mean().sqrt().item() < scale / 64, (batch, out.request_id)
+            if asked.temperature == 0.0:
+                # greedy picks: the engine's token is the oracle's best, or within the engine's rounding of it
+                for step, token in enumerate(out.token_ids):
+                    assert want[step, token] >= want[step].max() - 2 * diff.abs().max().item(), (batch, out.request_id, step)
+        llm.cache.check()
+        assert llm.cache.slots.num_free == llm.cache.num_slots
+    llm.close()
+
+
+def slabs_at(cache, request_id):
+    """{(tensor, layer): the request's pages of that tensor, in the order of its positions}"""
+    entry = cache.request(request_id)
+    out = {}
+    for g, group in enumerate(cache.groups):
+        pages = torch.tensor([p for p in entry.tables[g] if p >= 0], device=cache.device)
+        for name, slab in group.tensors.items():
+            for member in range(slab.shape[0]):
+                out[(g, name, member)] = slab[member][pages].clone()
+    return out
+
+
+@pytest.mark.parametrize("name,dtype", [("A", torch.float32), ("B", torch.float32), ("C", torch.float32),
+                                        ("B", torch.bfloat16), ("C", torch.bfloat16)])
+def test_the_cache_holds_the_same_however_the_tokens_were_cut(tmp_path, name, dtype):
+    """The same tokens as one mixed step (a whole prompt beside single tokens of two requests that decode) and
+    as steps of one request each: every layer's keys and values at the pages each run holds are equal, in
+    float32 within 1e-5. In bfloat16 they are equal bit for bit where both runs took the same kernels (the
+    whole prompt: a step of 21 rows and one of 23 go through the same products and the same attention, whose
+    sums do not depend on what else is in the batch); a single token takes other kernels alone (one row: the
+    norm inside the product, sums cut differently) than among 23 rows, so its float32 sums differ in the last
+    bit and a key may round to the neighbouring bfloat16 value, and in deeper layers so may its input: there
+    the bound is four steps of the largest value's 8 bits, and one step on average over a page."""
+    from distie_amd.kernels.hip_ops import HipOps
+
+    cfg, block = {"A": (plain.TINY_A, 4), "B": (plain.TINY_B, 8), "C": (plain.TINY_C, 16)}[name]
+    folder, _ = make_model_dir(tmp_path, cfg, seed=37, dtype=dtype)
+    ops = HipOps("cuda:0")
+    prompts = [random_ids(cfg, n, 60 + n) for n in (21, 22, 9)]
+    nxt = [7, 9]
+    single = build_runner(folder, ops, dtype, block_size=block, num_blocks=24)
+    batched = build_runner(folder, ops, dtype, block_size=block, num_blocks=24)
+    for runner in (single, batched):
+        for slab in (t for group in runner.cache.groups for t in group.tensors.values()):
+            slab.fill_(float("nan"))                    # what is compared was written, by this run
+    # requests 1 and 2 have their prompts cached (request 1 in two portions in the one run, whole in the other)
+    single.step([StepEntry(1, prompts[1], [])])
+    single.step([StepEntry(2, prompts[2], [])])
+    batched.step([StepEntry(2, prompts[2][:4], []), StepEntry(1, prompts[1][:15], [])])
+    batched.step([StepEntry(1, prompts[1][15:], []), StepEntry(2, prompts[2][4:], [])])
+    # one by one ...
+    want = [single.step([StepEntry(0, prompts[0], [len(prompts[0]) - 1])]),
+            single.step([StepEntry(1, [nxt[0]], [0])]), single.step([StepEntry(2, [nxt[1]], [0])])]
+    # ... and as one step
+    got = batched.step([StepEntry(0, prompts[0], [len(prompts[0]) - 1]), StepEntry(1, [nxt[0]], [0]),
+                        StepEntry(2, [nxt[1]], [0])])
+    tol = 1e-4 if dtype == torch.float32 else None
+    for request in (0, 1, 2):
+        a, b = slabs_at(single.cache, request), slabs_at(batched.cache, request)
+        assert a.keys() == b.keys() and len(a) >= 2 * cfg["num_hidden_layers"]
+        held = single.cache.request(request).num_cached
+        for key in a:
+            # positions beyond what the request holds lie in the last page and were never written: NaN in both
+            x, y = a[key].float(), b[key].float()
+            assert torch.equal(torch.isnan(x), torch.isnan(y)), key
+            written = ~torch.isnan(x)
+            assert int(written.sum()) > 0
+            if dtype == torch.float32:
+                assert (x[written] - y[written]).abs().max().item() < 1e-5, (request, key)
+            elif request == 0:
+                assert torch.equal(x[written], y[written]), (request, key)
+            else:
+                size = x[written].abs().max().item()
+                assert (x[written] - y[written]).abs().max().item() <= size * 2.0 ** -6, (request, key)
+                assert (x[written] - y[written]).abs().mean().item() <= size * 2.0 ** -10, (request, key)
+        assert held == batched.cache.request(request).num_cached
+    if tol is not None:
+        assert (torch.cat(want) - got).abs().max().item() < tol
+
+
+def test_random_weights_on_the_device_are_those_of_the_written_folder(tmp_path):
+    """One generator: drawn on the device, tensor for tensor the bits that `write_random_model` draws on the CPU;
+    an engine made from a configuration and a seed gives the logits of the engine that loads the folder, and
+    the plain implementation reading the folder is the oracle of both."""
+    from distie_amd.config import config_from_dict
+    from distie_amd.weights import random_init, write_random_model
+
+    for name, count in (("model.embed_tokens.weight", 1_000_003), ("x", 70_000_001)):
+        on_cpu = random_init.standard_normal(5, name, min(count, 3_000_000), "cpu")
+        on_device = random_init.standard_normal(5, name, count, "cuda")
+        assert torch.equal(on_device[:on_cpu.shape[0]].cpu(), on_cpu)
+        tail = random_init.standard_normal(5, name, count, "cpu")[-1000:] if count < 2_000_000 else None
+        if tail is not None:
+            assert torch.equal(on_device[-1000:].cpu(), tail)
+    for cfg, dtype in ((plain.TINY_A, "fp32"), (plain.TINY_B, "bf16"), (plain.TINY_C, "bf16")):
+        config = config_from_dict(cfg)
+        stored = "float32" if dtype == "fp32" else "bfloat16"
+        folder = write_random_model(config, tmp_path / f"m{cfg['hidden_size']}", seed=13, dtype=stored, std=0.1)
+        weights = plain.read_weights(folder)
+        drawn = LLM(config=config, random_weights=True, seed=13, weights_std=0.1, dtype=dtype, block_size=16, num_blocks=16)
+        loaded = LLM(folder, dtype=dtype, block_size=16, num_blocks=16)
+        for a, b in zip(drawn.model.parts(), loaded.model.parts()):
+            for key, t in vars(a).items():
+                if isinstance(t, torch.Tensor):
+                    assert torch.equal(t, getattr(b, key)), (type(a).__name__, key)
+        ids = random_ids(cfg, 50, 3)
+        entry = [StepEntry("a", ids, list(range(len(ids))))]
+        got = drawn.step(entry)
+        assert torch.equal(got, loaded.step(entry))
+        want = plain.forward(weights, cfg, ids, torch.float64).float()
+        diff = (got.cpu() - want).abs().max().item()
+        assert diff < (1e-4 if dtype == "fp32" else want.abs().max().item() / 16)

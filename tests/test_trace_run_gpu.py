@@ -25,6 +25,7 @@ class Replay:
              "--out", str(out), "--max-tokens", str(max_tokens)],
             stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
         self.step = 0
+        self.rows = {}          # step -> what its sidecar says of the rows of its logits
 
     def run(self, entries, end=()):
         record = {"step": self.step, "entries": entries, "end": list(end)}
@@ -39,11 +40,16 @@ class Replay:
             assert not path.exists()
             return None
         data = np.fromfile(path, dtype="<f4")
+        self.rows[self.step - 1] = json.loads((self.out / f"{self.step - 1}.json").read_text())
         return torch.from_numpy(data.reshape(wanted, -1))
 
     def close(self):
         self.proc.stdin.close()
         assert self.proc.wait(timeout=60) == 0
+        # the index of the whole run repeats the sidecars
+        index = json.loads((self.out / "index.json").read_text())
+        assert index["steps"] == {str(step): side["rows"] for step, side in self.rows.items()}
+        assert all(side["vocab"] == index["vocab"] and side["step"] == step for step, side in self.rows.items())
 
 
 @pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("B", "bfloat16"), ("C", "bfloat16")])
@@ -70,6 +76,9 @@ def test_replay_mixed_trace(tmp_path, name, dtype):
             want = list(range(n)) if r != "q" else [n - 1]
             entries.append({"id": r, "tokens": reqs[r][at[r]:at[r] + n], "want": want})
         logits = replay.run(entries, end=[e["id"] for e in entries if at[e["id"]] + len(e["tokens"]) == len(reqs[e["id"]])])
+        # the index names (request, position) of every row, in the order of the entries and of `want`
+        assert replay.rows[replay.step - 1]["rows"] == [[e["id"], at[e["id"]] + w] for e in entries for w in e["want"]]
+        assert replay.rows[replay.step - 1]["vocab"] == cfg["vocab_size"]
         row = 0
         for e in entries:
             r, n = e["id"], len(e["tokens"])
@@ -99,6 +108,7 @@ def test_replay_step_without_wanted_rows_and_a_pause(tmp_path):
     logits = replay.run([{"id": "a", "tokens": ids[7:], "want": [0, 12]}], end=["a"])
     want = oracle(weights, cfg, ids)
     assert (logits - want[[7, 19]]).abs().max() < 1e-4
+    assert replay.rows[2]["rows"] == [["a", 7], ["a", 19]] and 0 not in replay.rows
     # a name that was given back names a new request; a request may be ended by a step it sits out
     replay.run([{"id": "a", "tokens": other[:4], "want": []}, {"id": "c", "tokens": ids[:3], "want": []}])
     again = replay.run([{"id": "a", "tokens": other[4:], "want": [1]}], end=["c"])

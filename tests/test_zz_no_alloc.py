@@ -18,6 +18,7 @@ def _library():
     lib.distie_argmax_parts.argtypes = [I, I]
     lib.distie_argmax_static.argtypes = [P, P, I, I, P]
     lib.distie_argmax_static_limits.argtypes = [ctypes.POINTER(I), ctypes.POINTER(I)]
+    lib.distie_argmax_static_prepare.argtypes = []
     return lib
 
 
@@ -74,3 +75,31 @@ def test_sizes_beyond_the_maximum_are_refused():
     assert lib.distie_argmax_static(logits.data_ptr(), out.data_ptr(), max_rows.value + 1, 64, stream) == -2
     assert lib.distie_argmax_static(logits.data_ptr(), out.data_ptr(), 4, 0, stream) == -1
     assert lib.distie_argmax_static(logits.data_ptr(), out.data_ptr(), 0, 64, stream) == 0
+
+
+def test_recorded_into_a_graph_after_the_device_was_prepared():
+    """The callers the entry point is for: the array's address is looked up outside the capture
+    (`distie_argmax_static_prepare`), the launches are recorded, and every replay picks what the eager entry
+    point picks for the logits that lie in the buffer then, with eager work and waits between the replays."""
+    lib = _library()
+    assert lib.distie_argmax_static_prepare() == 0
+    gen = torch.Generator().manual_seed(6)
+    logits = torch.randn((24, 151_936), generator=gen).cuda()
+    out = torch.full((24,), -7, dtype=torch.int32, device="cuda")
+    assert lib.distie_argmax_parts(24, 151_936) > 1
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        status = lib.distie_argmax_static(logits.data_ptr(), out.data_ptr(), 24, 151_936,
+                                          torch.cuda.current_stream().cuda_stream)
+    assert status == 0
+    for round_ in range(4):
+        fresh = torch.randn((24, 151_936), generator=gen)
+        fresh[round_, 151_935 - round_] = 40.0
+        logits.copy_(fresh.cuda())
+        out.fill_(-7)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        _, want, _ = _both(lib, logits)                 # eager work on the same array between the replays
+        assert torch.equal(out.cpu(), want)
+        assert torch.equal(out.cpu().long(), fresh.argmax(dim=1))

@@ -60,7 +60,7 @@ class TorchOps(Ops):
         return qkv
 
     def paged_attention(self, qkv, meta, group, k_cache, v_cache, num_heads, num_kv_heads, head_dim,
-                        scale, window):
+                        scale, window, extras=None):
         T = qkv.shape[0]
         P = k_cache.shape[2]
         q_all = qkv.view(T, num_heads + 2 * num_kv_heads, head_dim)[:, :num_heads].float()
@@ -82,6 +82,10 @@ class TorchOps(Ops):
                 k = k.repeat_interleave(rep, dim=1)
                 v = v.repeat_interleave(rep, dim=1)
                 s = torch.einsum("hd,nhd->hn", q_all[t], k) * scale
+                if extras is not None and extras.score_cap is not None:
+                    s = extras.score_cap * torch.tanh(s / extras.score_cap)
+                if extras is not None and extras.head_slopes is not None:
+                    s = s + extras.head_slopes.float()[:, None] * (keys - pos).float()[None, :]
                 out[t] = torch.einsum("hn,nhd->hd", torch.softmax(s, -1), v)
         return out.view(T, num_heads * head_dim).to(qkv.dtype)
 
