@@ -74,8 +74,11 @@ def test_bfloat16_generation_through_the_scheduler(tmp_path, name, graphs, looka
     params = [SamplingParams(max_new_tokens=new, temperature=0.7 if i % 2 == 0 else 0.0, seed=200 + i)
               for i in range(len(prompts))]
     tight = pages is None
-    if tight:                       # the two longest requests fit, all of them do not
-        pages = sum(-(-(n + new) // block) for n in sorted(lengths)[-2:]) + 1
+    if tight:
+        # every request is seated (by the pages of what is known of it then), and they cannot all grow to their
+        # length: B's draw 30 tokens each on 11 pages of 8, C's 20 each on 11 pages of 16
+        pages, new = 11, {"B": 30, "C": 20}[name]
+        params = [SamplingParams(max_new_tokens=new, temperature=p.temperature, seed=p.seed) for p in params]
     llm = LLM(folder, dtype="bf16", block_size=block, num_blocks=pages, token_budget=budget, use_graphs=graphs,
               lookahead=lookahead)
     outs, kept = run_and_keep_logits(llm, prompts, params)
