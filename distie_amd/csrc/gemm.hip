@@ -509,18 +509,29 @@ extern "C" int distie_gemm_packed_bf16(const void* x, const void* w_packed, cons
 }
 
 // ---------------------------------------------------------------- packed weights, 17 to 64 rows of x a pass
-// A workgroup of four waves owns four row blocks (one a wave) and one slice of K. Per k-step of 128 the
-// weights go straight into registers, four k-steps ahead; the x tile ([16 MB rows, 128 k], the same for
-// all four waves) is fetched four k-steps ahead as well, into registers, and put into LDS (two stages)
-// right before it is used, so that x is read from the L2 once per workgroup and not once per wave.
+// A workgroup of WAVES waves owns as many row blocks (one a wave) and one slice of K. Per k-step of 128 the
+// weights go straight into registers, some k-steps ahead; the x tile ([16 MB rows, 128 k], the same for
+// all waves) is fetched as far ahead, into registers, and put into LDS (two stages) right before it is used,
+// so that x is read from the L2 once per workgroup and not once per wave.
 // Epilogues as in gemm_packed_kernel, for every block of 16 rows of x.
-constexpr int WD_STAGES = 4;
+//
+//
+// WAVES is two for up to 32 rows of x in all, else four. What streams the weights fastest here is many small
+// workgroups, spread evenly over the compute units (the same loop with x left out, gate+up of the 1.5B shape,
+// 55 MB: 13.0 us with one wave a workgroup, 13.7 with two, 15.8 with four, of which there are 280 for 256 compute
+// units); but a smaller workgroup reads x more often. At 32 rows two waves are best (15.8 us against 18.3 with
+// four and 17.2 with one; the decode step at batch 24 and 32 is 6 and 5 % faster); from 48 rows on, and with the
+// rows taken in two passes, four are (batch 64: 3 % slower with two, a portion of 200 tokens 8 %).
+// How far ahead the loads run matters little beside that (four, six or eight k-steps: the same time), as long as
+// the wave never waits for all of them at once.
+template <int MB, int WAVES>
+constexpr int wd_stages() { return WAVES == 2 && MB == 1 ? 8 : 4; }    // (k-steps under way; eight with four waves filled the registers so far that fewer workgroups fit a compute unit)
 // elements of an x row in LDS: a stride of 32 bytes more than a multiple of 64 keeps the reads (lane (r, g):
 // row r, byte 16 g) free of bank conflicts; with 16 bytes more every read costs twice (measured)
 constexpr int WD_XROW = SK_KSTEP + 16;
 
-template <typename Y, int MODE, int MB>
-__global__ __launch_bounds__(256, 2) void gemm_packed_wide_kernel(const bf16_t* __restrict__ x,
+template <typename Y, int MODE, int MB, int WD_WAVES>
+__global__ __launch_bounds__(64 * WD_WAVES) void gemm_packed_wide_kernel(const bf16_t* __restrict__ x,
                                                                const bf16_t* __restrict__ w,
                                                                const float* __restrict__ bias, Y* __restrict__ y,
                                                                int M, int N, int K, int row_blocks, int tiles_per_slice,
@@ -533,6 +544,7 @@ __global__ __launch_bounds__(256, 2) void gemm_packed_wide_kernel(const bf16_t* 
   x += static_cast<int64_t>(m0) * K;
   y += static_cast<int64_t>(m0) * (MODE == PK_GATED ? N / 2 : N);
   M = min(m_group, M - m0);
+  constexpr int WD_STAGES = wd_stages<MB, WD_WAVES>();
   const int tid = threadIdx.x;
   const int lane = tid % 64;
   const int wave = tid / 64;
@@ -542,27 +554,32 @@ __global__ __launch_bounds__(256, 2) void gemm_packed_wide_kernel(const bf16_t* 
   const int s_begin = blockIdx.y * tiles_per_slice;
   const int s_end = min(k_tiles, s_begin + tiles_per_slice);
   const int steps = (s_end - s_begin + 3) / 4;
-  const int block = blockIdx.x * 4 + wave;
+  const int block = blockIdx.x * WD_WAVES + wave;
   const bool active = block < row_blocks;                       // a wave without a row block still carries x
   const bf16_t* wp = w + static_cast<int64_t>(min(block, row_blocks - 1)) * k_tiles * PK_TILE + lane * 8;
-  // this thread's part of an x tile: rows 16 p + tid / 16 (p < MB), k 8 (tid % 16) .. + 7 of the step
+  // this thread's part of an x tile: rows XROWS p + tid / 16 (p < XP), k 8 (tid % 16) .. + 7 of the step
   const int x_row = tid / 16;
   const int x_chunk = tid % 16;
-  const bf16_t* xsrc[MB];
+  constexpr int XP = MB * 4 / WD_WAVES;                          // pieces of an x tile a thread carries
+  constexpr int XROWS = 4 * WD_WAVES;                           // rows of the tile the threads cover at once
+  const bf16_t* xsrc[XP];
 #pragma unroll
-  for (int p = 0; p < MB; ++p) xsrc[p] = x + static_cast<int64_t>(min(16 * p + x_row, M - 1)) * K;
+  for (int p = 0; p < XP; ++p) xsrc[p] = x + static_cast<int64_t>(min(XROWS * p + x_row, M - 1)) * K;
 
   bf16x8 a[WD_STAGES][4];
-  uint4 xr[WD_STAGES][MB];
+  uint4 xr[WD_STAGES][XP];
   floatx4 acc[MB];
 #pragma unroll
   for (int b = 0; b < MB; ++b) acc[b] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  // Loads are unconditional and nothing touches their results before the k-step that uses them: a load
-  // under a branch, or a select right behind it, would make the wave wait for every load in flight.
-  // Addresses are clamped into the buffers instead. A weight tile past the slice's end is read from the
+  // Loads are unconditional, and nothing but arithmetic stands between a load and its use, in the same order in
+  // every path into the loop: only then does the compiler count how many younger loads may stay in flight at each
+  // use (a load under a branch, a select that it turns into one, or paths that issue different loads, and it
+  // waits for all of them instead: measured, one trip to memory per WD_STAGES k-steps with nothing else under
+  // way). Addresses are clamped into the buffers instead. A weight tile past the slice's end is read from the
   // slice's last tile (the same rows, so whatever it holds reaches no output it would not reach anyway) and
-  // meets zeros in x: x past the slice or past K is replaced by zeros when it is put into LDS.
+  // meets zeros in x: x past the slice or past K is masked to zeros when it is put into LDS. A wave without a
+  // row block computes on the last block's weights and writes nothing.
   auto x_inside = [&](int step) {
     const int t0 = s_begin + 4 * step;
     return 32 * t0 + 8 * x_chunk < K && t0 + x_chunk / 4 < s_end;
@@ -574,35 +591,32 @@ __global__ __launch_bounds__(256, 2) void gemm_packed_wide_kernel(const bf16_t* 
       a[slot][j] = *reinterpret_cast<const bf16x8*>(wp + static_cast<int64_t>(min(t0 + j, s_end - 1)) * PK_TILE);
     const int k = x_inside(step) ? 32 * t0 + 8 * x_chunk : 0;
 #pragma unroll
-    for (int p = 0; p < MB; ++p) xr[slot][p] = *reinterpret_cast<const uint4*>(xsrc[p] + k);
+    for (int p = 0; p < XP; ++p) xr[slot][p] = *reinterpret_cast<const uint4*>(xsrc[p] + k);
   };
 
 #pragma unroll
-  for (int slot = 0; slot < WD_STAGES; ++slot)
-    if (slot < steps) fetch(slot, slot);
+  for (int slot = 0; slot < WD_STAGES; ++slot) fetch(slot, slot);         // (beyond the last step: clamped, unused)
 
   // One k-step: x of this step into LDS, barrier, products. Stage `slot % 2` was last read two k-steps ago;
   // every wave has passed the barrier of the k-step in between, so all of them are done with it.
   auto k_step = [&](int step, int slot) {
     const int stage = slot % 2;
-    const bool inside = x_inside(step);
+    const uint32_t keep = x_inside(step) ? 0xffffffffu : 0u;
 #pragma unroll
-    for (int p = 0; p < MB; ++p)
-      *reinterpret_cast<uint4*>(&xs[stage][16 * p + x_row][8 * x_chunk]) = inside ? xr[slot][p] : uint4{0u, 0u, 0u, 0u};
-    __syncthreads();
-    if (active) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int b = 0; b < MB; ++b) {
-          const bf16x8 xb = *reinterpret_cast<const bf16x8*>(&xs[stage][16 * b + r][32 * j + 8 * g]);
-          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[slot][j], xb, acc[b], 0, 0, 0);
-        }
+    for (int p = 0; p < XP; ++p) {
+      const uint4 v = xr[slot][p];
+      *reinterpret_cast<uint4*>(&xs[stage][XROWS * p + x_row][8 * x_chunk]) = uint4{v.x & keep, v.y & keep, v.z & keep, v.w & keep};
     }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        const bf16x8 xb = *reinterpret_cast<const bf16x8*>(&xs[stage][16 * b + r][32 * j + 8 * g]);
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[slot][j], xb, acc[b], 0, 0, 0);
+      }
   };
   int s = 0;
-  // the steady state has no branch between the loads and their use, so the waits the compiler places let
-  // the loads of the three k-steps ahead stay in flight
   for (; s + 2 * WD_STAGES <= steps; s += WD_STAGES) {
 #pragma unroll
     for (int slot = 0; slot < WD_STAGES; ++slot) {
@@ -610,13 +624,17 @@ __global__ __launch_bounds__(256, 2) void gemm_packed_wide_kernel(const bf16_t* 
       fetch(s + slot + WD_STAGES, slot);
     }
   }
-  for (; s < steps; s += WD_STAGES) {
+  // the last k-steps: what they need is under way already
+#pragma unroll
+  for (int round = 0; round < 2; ++round) {
 #pragma unroll
     for (int slot = 0; slot < WD_STAGES; ++slot) {
       if (s + slot >= steps) break;
       k_step(s + slot, slot);
-      if (s + slot + WD_STAGES < steps) fetch(s + slot + WD_STAGES, slot);
+      if (round == 0 && s + slot + WD_STAGES < steps) fetch(s + slot + WD_STAGES, slot);
     }
+    s += WD_STAGES;
+    if (s >= steps) break;
   }
   if (!active) return;
 
@@ -656,13 +674,14 @@ __global__ __launch_bounds__(256, 2) void gemm_packed_wide_kernel(const bf16_t* 
   }
 }
 
-// Slices of K for the wide kernel: enough workgroups for the chip, slices of whole k-steps, at least two
+// Slices of K for the wide kernel: enough waves for the chip (a thousand), slices of whole k-steps, at least two
 // k-steps long.
 static void wide_plan(int row_blocks, int K, int* slices, int* tiles_per_slice) {
-  const int groups = (row_blocks + 3) / 4;
+  constexpr int WD_WAVES = 4;             // (the cut does not depend on the workgroups' size: the caller sizes its buffer by it)
+  const int groups = (row_blocks + WD_WAVES - 1) / WD_WAVES;
   const int steps = (K + SK_KSTEP - 1) / SK_KSTEP;
   int want = 1;
-  while (want < 64 && groups * want < 256 && steps / (want * 2) >= 2) want *= 2;
+  while (want < 64 && groups * want * WD_WAVES < 1024 && steps / (want * 2) >= 2) want *= 2;
   int per = (steps + want - 1) / want;
   *tiles_per_slice = 4 * per;
   *slices = (steps + per - 1) / per;
@@ -688,17 +707,21 @@ static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bia
   // 15.4 us, gate+up 22.4 -> 21.3 us; a weight of 270 MB gets slower, being fetched from memory twice).
   const int m_group = (pass_blocks >= 1 && pass_blocks <= 4) ? 16 * pass_blocks : 64;
   const int groups = (M + m_group - 1) / m_group;
-  dim3 grid((row_blocks + 3) / 4, slices, groups);
   const int mb = (std::min(M, m_group) + 15) / 16;
-#define WIDE(MODE, MB)                                                                                   \
-  DISTIE_DISPATCH(y_dtype, Y, (gemm_packed_wide_kernel<Y, MODE, MB><<<grid, 256, 0, stream>>>(           \
+  const int waves = M <= 32 ? 2 : 4;
+  dim3 grid((row_blocks + waves - 1) / waves, slices, groups);
+#define WIDE(MODE, MB, WAVES)                                                                                   \
+  DISTIE_DISPATCH(y_dtype, Y, (gemm_packed_wide_kernel<Y, MODE, MB, WAVES><<<grid, 64 * WAVES, 0, stream>>>(    \
                                   x, w, bias, static_cast<Y*>(y), M, N, K, row_blocks, tiles_per_slice, m_group)))
-#define WIDE_MB(MODE)                    \
-  switch (mb) {                          \
-    case 1: WIDE(MODE, 1); break;        \
-    case 2: WIDE(MODE, 2); break;        \
-    case 3: WIDE(MODE, 3); break;        \
-    default: WIDE(MODE, 4); break;       \
+#define WIDE_MB(MODE)                                   \
+  switch (mb) {                                         \
+    case 1: WIDE(MODE, 1, 2); break;                    \
+    case 2:                                             \
+      if (waves == 2) WIDE(MODE, 2, 2);                 \
+      else WIDE(MODE, 2, 4);                            \
+      break;                                            \
+    case 3: WIDE(MODE, 3, 4); break;                    \
+    default: WIDE(MODE, 4, 4); break;                   \
   }
   if (mode == PK_GATED) {
     WIDE_MB(PK_GATED);
