@@ -200,6 +200,8 @@ def main() -> int:
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--context", type=int, default=None,
                         help="tokens behind every request when decoding starts (the shape's own: 2,048 or 8,192)")
+    parser.add_argument("--prefill", type=int, default=None,
+                        help="tokens of the timed prompt (the shape's own: 2,048 or 8,192), run in portions of the token budget")
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     parser.add_argument("--no-points", action="store_true", help="skip the other batch sizes")
     parser.add_argument("--no-tune", action="store_true",
@@ -222,7 +224,7 @@ def main() -> int:
     layers = shape["num_hidden_layers"]
     layers_run = args.layers or layers
     shape["num_hidden_layers"] = layers_run
-    context, prefill_tokens = args.context or preset["context"], preset["prefill"]
+    context, prefill_tokens = args.context or preset["context"], args.prefill or preset["prefill"]
     points_at = () if args.no_points or args.serve else preset["points"]
     max_batch = SERVE["requests"] if args.serve else max((args.batch,) + tuple(points_at))
     tokens_per_request = context + args.warmup + args.steps + early_tokens(max_batch, context)
