@@ -177,7 +177,7 @@ class CacheManager:
         self.table_width = int(width)
         for group in self.groups:
             table = torch.full((self.num_slots + 1, self.table_width), GONE, dtype=torch.int32)
-            table[self.sink_slot, 0] = group.sink_page
+            table[self.sink_slot, :] = group.sink_page       # every position of a padding request lies in the sink page
             group.table = table.to(self.device) if self.device is not None else table
             group.changed.clear()
             # what requests hold already goes along with the next step

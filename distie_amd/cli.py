@@ -34,6 +34,9 @@ def _engine_options(parser: argparse.ArgumentParser) -> None:
     parser.add_argument("--graph-buckets", default=None, metavar="SIZES",
                         help="batch sizes that get a captured decode step, comma-separated (default: 1,2,4,8, then "
                              "every multiple of 8 up to --max-seqs)")
+    parser.add_argument("--graph-tokens", type=int, default=None, metavar="N",
+                        help="steps that hold a portion of a prompt replay a captured step too if they bring at most "
+                             "N tokens (default 96; 0: only decode steps are captured)")
     parser.add_argument("--step-stats", type=int, default=None, help="log a time breakdown every N steps")
     parser.add_argument("--no-packed-weights", action="store_true",
                         help="no second copy of the weights in the matrix cores' order (half the weight memory, "
@@ -55,7 +58,7 @@ def _build(args):
         dtype=args.dtype, block_size=args.block_size, num_blocks=args.num_blocks, max_seqs=args.max_seqs,
         token_budget=args.token_budget, use_graphs=False if args.no_decode_graphs else None,
         graph_buckets=tuple(int(b) for b in args.graph_buckets.split(",") if b) if args.graph_buckets else None,
-        step_stats=args.step_stats, seed=args.seed, packed_weights=False if args.no_packed_weights else (
+        graph_tokens=args.graph_tokens, step_stats=args.step_stats, seed=args.seed, packed_weights=False if args.no_packed_weights else (
             tuple(r for r in args.packed_weights.split(",") if r) if args.packed_weights else None),
         gpu_mem_fraction=args.gpu_mem_fraction,
         tune_products=True if args.tune_products else None)

@@ -47,6 +47,11 @@ class EngineConfig:
     # batch sizes that get a captured decode step of their own; None = 1, 2, 4, 8, then every multiple of 8 up to
     # max_seqs (a step is padded up to the next size; one with more rows than the largest runs uncaptured)
     graph_buckets: Optional[Tuple[int, ...]] = None
+    # mixed steps (portions of prompts beside single tokens) of up to so many tokens replay graphs as well, padded
+    # to 16, 24, 32, 48, 64, 96, ... tokens: launched kernel by kernel such a step costs the host about as long as
+    # the device, replayed a sixth of that. 0: only decode steps are captured. (Up to 96 tokens a step runs on this
+    # engine's own kernels alone; every bucket of tokens, requests and context length is a graph of its own.)
+    graph_tokens: int = 96
     # a second copy of the weights in the matrix cores' order, for decode: True, False, or the roles that get one.
     # A role is whatever name a part gives its product in `Ops.prepare_linear(role=...)`; the parts of the Qwen2
     # decoder name "qkv", "attn_out", "gate_up", "down" and "head", another part may name others
@@ -69,6 +74,8 @@ class EngineConfig:
             if not buckets or buckets[0] < 1:
                 raise ValueError("graph_buckets must be batch sizes >= 1")
             object.__setattr__(self, "graph_buckets", buckets)
+        if self.graph_tokens < 0:
+            raise ValueError("graph_tokens must be >= 0")
         if not isinstance(self.packed_weights, bool):
             object.__setattr__(self, "packed_weights", tuple(self.packed_weights))
 
@@ -116,6 +123,9 @@ class EngineConfig:
         raw = os.getenv("WORKER_GRAPH_BUCKETS", "").strip()
         if raw:
             env["graph_buckets"] = tuple(int(b) for b in raw.split(","))
+        raw = os.getenv("WORKER_GRAPH_TOKENS", "").strip()
+        if raw:
+            env["graph_tokens"] = int(raw)
         raw = os.getenv("WORKER_GPU_MEM_FRACTION", "").strip()
         if raw:
             env["gpu_mem_fraction"] = float(raw)

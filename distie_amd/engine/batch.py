@@ -72,21 +72,26 @@ class BatchBuilder:
                 dev = torch.from_numpy(both).to(group.table.device)
                 group.table.view(-1)[dev[0].long()] = dev[1]
 
-    def fill(self, host: np.ndarray, entries: Sequence[StepEntry], pad_requests: int = 0, want_all: bool = False):
+    def fill(self, host: np.ndarray, entries: Sequence[StepEntry], pad_requests: int = 0, want_all: bool = False,
+             pad_tokens: int = 0, want_last: bool = False):
         """Write the step into `host` (int32, at least layout(...)[-1] long).
         -> (offsets, T, B, R, max_q, max_kv, host_cu_q, host_past)
 
         Pages for the new tokens must have been reserved. `pad_requests` appends that many
-        one-token rows that write to the sink page and the sink slot (for captured steps of
-        fixed size). `want_all`: every row is wanted, whatever the entries say."""
+        requests that write to the sink page and the sink slot (for captured steps of
+        fixed size): one token each, the first of them `pad_tokens` more (positions 0, 1, ...). `want_all`:
+        every row is wanted, whatever the entries say. `want_last`: one row a request, its last (also of
+        the padding requests), whatever the entries say."""
         if not entries:
             raise ValueError("a step needs at least one entry")
+        if pad_tokens and not pad_requests:
+            raise ValueError("padding tokens need a padding request to belong to")
         cache = self.cache
         P = cache.block_size
         G = len(cache.groups)
         B = len(entries) + pad_requests
-        T = sum(len(e.tokens) for e in entries) + pad_requests
-        R = T if want_all else sum(len(e.want) for e in entries)
+        T = sum(len(e.tokens) for e in entries) + pad_requests + pad_tokens
+        R = T if want_all else (B if want_last else sum(len(e.want) for e in entries))
         if len({e.request_id for e in entries}) != len(entries):
             raise ValueError("a request may appear once in a step")
         offsets = self.layout(T, B, R)
@@ -146,7 +151,9 @@ class BatchBuilder:
                     if (pages < 0).any():
                         raise AssertionError("a new token would be written to a page that was given back")
                     slots[g][t0:t0 + n] = pages * P + pos % P
-            if not want_all:
+            if want_last:
+                want_rows[b] = t0 + n - 1
+            elif not want_all:
                 for w in entry.want:
                     if not 0 <= int(w) < n:
                         raise ValueError(f"request {entry.request_id!r}: wanted place {w} is outside its {n} tokens")
@@ -155,21 +162,27 @@ class BatchBuilder:
             t0 += n
             max_q = max(max_q, n)
             max_kv = max(max_kv, past + n)
-        for b in range(len(entries), B):           # padding rows
-            positions[t0] = 0
-            token_request[t0] = b
-            cu_q[b + 1] = t0 + 1
-            kv_len[b] = 1
+        for b in range(len(entries), B):           # padding requests
+            n = 1 + (pad_tokens if b == len(entries) else 0)
+            pos = np.arange(n, dtype=np.int64)
+            positions[t0:t0 + n] = pos
+            token_request[t0:t0 + n] = b
+            cu_q[b + 1] = t0 + n
+            kv_len[b] = n
             slots_state[b] = cache.sink_slot
             for g, group in enumerate(cache.groups):
-                slots[g][t0] = group.sink_page * P
-            t0 += 1
+                slots[g][t0:t0 + n] = group.sink_page * P + pos % P
+            if want_last:
+                want_rows[b] = t0 + n - 1
+            t0 += n
+            max_q = max(max_q, n)
+            max_kv = max(max_kv, n)
         if want_all:
             want_rows[:] = np.arange(T)
         return offsets, T, B, R, int(max_q), int(max_kv), cu_q.copy(), host_past
 
     def meta_of(self, dev: torch.Tensor, offsets, T: int, B: int, R: int, max_q: int, max_kv: int,
-                host_cu_q=None, host_past=None):
+                host_cu_q=None, host_past=None, singles_bound=None):
         """Views into the device copy `dev` of a packed buffer -> (ids, BatchMeta, want_rows)."""
         dcut = lambda i: dev[int(offsets[i]):int(offsets[i + 1])]
         meta = BatchMeta(
@@ -178,6 +191,7 @@ class BatchBuilder:
             max_q=max_q, max_kv=max_kv, block_size=self.cache.block_size,
             groups=[GroupMeta(block_table=group.table, slots=dcut(7 + g)) for g, group in enumerate(self.cache.groups)],
             host_cu_q=host_cu_q, host_past=host_past, all_decode=(max_q == 1), table_rows=dcut(5),
+            singles_bound=singles_bound,
         )
         return dcut(0), meta, (dcut(6) if R else None)
 

@@ -61,9 +61,12 @@ def bucket_for(buckets: Sequence[int], rows: int) -> int:
 
 
 class _Bucket:
-    def __init__(self, size: int, builder, device) -> None:
-        self.size = size
-        self.offsets = builder.layout(size, size, size)
+    def __init__(self, tokens: int, requests: int, builder, device) -> None:
+        self.tokens = tokens
+        self.requests = requests
+        self.mixed = tokens != requests
+        self.rows = requests if self.mixed else tokens        # of the logits: one a request, or every token
+        self.offsets = builder.layout(tokens, requests, self.rows)
         words = int(self.offsets[-1])
         self.host = torch.zeros(words, dtype=torch.int32, pin_memory=True)
         self.host_np = self.host.numpy()
@@ -73,17 +76,35 @@ class _Bucket:
         self.copied = torch.cuda.Event()
 
 
+def token_buckets(most: int) -> Tuple[int, ...]:
+    """Token counts that captured mixed steps are made for: 16, 32, 48, 64, 96, 128, ... up to `most`."""
+    sizes, step = [], 16
+    while True:
+        for k in (2, 3):
+            size = step * k // 2
+            if size > most:
+                return tuple(sizes) if sizes else ((most,) if most > 1 else ())
+            sizes.append(size)
+        step *= 2
+
+
 class DecodeGraphs:
     RETRY_AFTER_STEPS = 512     # after a failure, steps run uncaptured for so long before a capture is tried again
     MAX_FAILURES = 3            # ... and after so many failures for good
+    MAX_MIXED_GRAPHS = 64       # captured mixed steps kept at most; a shape beyond that runs kernel by kernel
 
-    def __init__(self, runner, max_batch: int, buckets: Optional[Sequence[int]] = None) -> None:
+    def __init__(self, runner, max_batch: int, buckets: Optional[Sequence[int]] = None, mixed_tokens: int = 0) -> None:
         self.runner = runner
         self.buckets = decode_buckets(max_batch, buckets)
         self.max_batch = self.buckets[-1]
-        self._made: Dict[int, _Bucket] = {}
+        # a mixed step that is padded needs a request more than it holds
+        self.mixed_tokens = int(mixed_tokens)
+        self.token_buckets = token_buckets(self.mixed_tokens) if self.mixed_tokens > 1 else ()
+        self.request_buckets = decode_buckets(max_batch + 1, None if buckets is None else list(buckets) + [max_batch + 1])
+        self._made: Dict[Tuple[int, int], _Bucket] = {}
         self._pool = None
         self.replays = 0
+        self.mixed_replays = 0
         self.failures = 0           # captures or replays that raised
         self._resting = 0           # decode steps still to run uncaptured after a failure
 
@@ -94,13 +115,18 @@ class DecodeGraphs:
 
     @property
     def captured(self) -> List[int]:
-        """Batch sizes that have a graph."""
-        return sorted(size for size, b in self._made.items() if b.graphs)
+        """Batch sizes that have a graph of a decode step."""
+        return sorted(b.tokens for b in self._made.values() if b.graphs and not b.mixed)
 
     @property
     def captured_contexts(self) -> List[Tuple[int, int]]:
-        """(batch size, context class) of every graph."""
-        return sorted((size, limit) for size, b in self._made.items() for limit in b.graphs)
+        """(batch size, context class) of every graph of a decode step."""
+        return sorted((b.tokens, limit) for b in self._made.values() if not b.mixed for limit in b.graphs)
+
+    @property
+    def captured_mixed(self) -> List[Tuple[int, int, int]]:
+        """(tokens, requests, context class) of every graph of a mixed step."""
+        return sorted((b.tokens, b.requests, limit) for b in self._made.values() if b.mixed for limit in b.graphs)
 
     def drop(self) -> None:
         """Forget every graph *and* the memory pool they were captured into. The two go together: graphs
@@ -110,35 +136,64 @@ class DecodeGraphs:
         self._made.clear()
         self._pool = None
 
+    def _mixed_bucket(self, entries: Sequence[StepEntry]) -> Optional[Tuple[int, int]]:
+        """(tokens, requests) of the captured step that takes these entries, or None."""
+        tokens = sum(len(e.tokens) for e in entries)
+        if not self.token_buckets or tokens > self.token_buckets[-1] or len(entries) > self.max_batch:
+            return None
+        for e in entries:
+            if len(e.want) > 1 or (len(e.want) == 1 and int(e.want[0]) != len(e.tokens) - 1):
+                return None
+        for size in self.token_buckets:
+            if size < tokens:
+                continue
+            if size == tokens:
+                requests = bucket_for(self.request_buckets, len(entries))
+            else:
+                requests = bucket_for(self.request_buckets, len(entries) + 1)
+            # every padding request brings a token; what is left of the bucket goes to the first of them
+            if size - tokens >= requests - len(entries) and (size > tokens or requests == len(entries)):
+                return size, requests
+        return None
+
     def try_run(self, entries: Sequence[StepEntry], feed: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Logits [wanted, vocab] if this step went through a graph, None if it must run the
-        ordinary way (not a pure decode step, too many rows, or captured steps are switched off).
+        ordinary way (no bucket takes it, or captured steps are switched off).
         What is wrong with the entries themselves (a token id out of range, pages not reserved) raises
         as it does in an ordinary step and switches nothing off."""
-        if len(entries) > self.max_batch or any(len(e.tokens) != 1 for e in entries):
+        if len(entries) > self.max_batch or self.failures >= self.MAX_FAILURES:
             return None
-        if self.failures >= self.MAX_FAILURES:
-            return None
+        if all(len(e.tokens) == 1 for e in entries):
+            size = bucket_for(self.buckets, len(entries))
+            key = (size, size)
+        else:
+            key = self._mixed_bucket(entries)
+            if key is None:
+                return None
         if self._resting > 0:
             self._resting -= 1
             return None
         runner = self.runner
-        size = bucket_for(self.buckets, len(entries))
-        bucket = self._made.get(size)
+        bucket = self._made.get(key)
         if bucket is None:
-            bucket = self._made[size] = _Bucket(size, runner.builder, runner.ops.device)
+            if key[0] != key[1] and sum(len(b.graphs) for b in self._made.values() if b.mixed) >= self.MAX_MIXED_GRAPHS:
+                return None
+            bucket = self._made[key] = _Bucket(key[0], key[1], runner.builder, runner.ops.device)
         bucket.copied.synchronize()                      # the previous copy out of the pinned buffer is done
-        max_kv = runner.builder.fill(bucket.host_np, entries, pad_requests=size - len(entries), want_all=True)[5]
+        pad_requests = bucket.requests - len(entries)
+        pad_tokens = bucket.tokens - sum(len(e.tokens) for e in entries) - pad_requests
+        max_kv = runner.builder.fill(bucket.host_np, entries, pad_requests=pad_requests, pad_tokens=pad_tokens,
+                                     want_all=not bucket.mixed, want_last=bucket.mixed)[5]
         try:
             return self._run(bucket, entries, feed, max_kv)
         except Exception:  # noqa: BLE001 - the ordinary path rewrites the same slots
             self.failures += 1
             self._resting = self.RETRY_AFTER_STEPS
             self.drop()
-            _log.exception("captured decode step failed (failure %d of %d allowed): graphs and their memory pool "
+            _log.exception("captured step failed (failure %d of %d allowed): graphs and their memory pool "
                            "are dropped, steps run uncaptured %s", self.failures, self.MAX_FAILURES,
                            "from now on" if self.failures >= self.MAX_FAILURES
-                           else f"for the next {self.RETRY_AFTER_STEPS} decode steps")
+                           else f"for the next {self.RETRY_AFTER_STEPS} steps that a graph would take")
             return None
 
     def _run(self, bucket: _Bucket, entries: Sequence[StepEntry], feed: Optional[torch.Tensor],
@@ -159,6 +214,8 @@ class DecodeGraphs:
             made[0].replay()
             logits = made[1]
             self.replays += 1
+        if bucket.mixed:
+            self.mixed_replays += 1
         rows = [i for i, e in enumerate(entries) if len(e.want)]
         if not rows:
             return logits[:0]
@@ -168,11 +225,15 @@ class DecodeGraphs:
 
     def _forward(self, bucket: _Bucket, limit: int) -> torch.Tensor:
         runner = self.runner
-        n = bucket.size
-        ids, meta, want = runner.builder.meta_of(bucket.dev, bucket.offsets, n, n, n, 1, limit)
+        T, B = bucket.tokens, bucket.requests
+        if bucket.mixed:
+            ids, meta, want = runner.builder.meta_of(bucket.dev, bucket.offsets, T, B, B, T, limit, singles_bound=B)
+        else:
+            ids, meta, want = runner.builder.meta_of(bucket.dev, bucket.offsets, T, T, T, 1, limit)
         runner.ops.captured = True
         try:
-            return runner.model.forward(runner.ops, ids, meta, runner.cache, runner.act_dtype, want, every_row=True)
+            return runner.model.forward(runner.ops, ids, meta, runner.cache, runner.act_dtype, want,
+                                        every_row=not bucket.mixed)
         finally:
             runner.ops.captured = False
 

@@ -123,7 +123,7 @@ class LLM:
             if self.model.capturable:
                 from .graphs import DecodeGraphs
 
-                self.runner.graphs = DecodeGraphs(self.runner, ec.max_seqs, ec.graph_buckets)
+                self.runner.graphs = DecodeGraphs(self.runner, ec.max_seqs, ec.graph_buckets, ec.graph_tokens)
             else:
                 names = sorted({type(p).__name__ for p in self.model.parts() if not p.capturable})
                 _log.info("decode steps are not captured: %s cannot be recorded into a graph", ", ".join(names))

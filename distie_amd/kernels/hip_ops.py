@@ -816,7 +816,7 @@ class HipOps(Ops):
             # with these sizes: worked out once per step (the layers run one after the other, so they can
             # share the buffers)
             key = ("attention", int(window or 0), num_heads, num_kv_heads, head_dim, meta.max_kv, meta.all_decode,
-                   self.PREFILL_PARTS, self.PREFILL_WORKGROUPS, self.DECODE_WAVES, self.DECODE_MAX_RUNS)
+                   meta.singles_bound, self.PREFILL_PARTS, self.PREFILL_WORKGROUPS, self.DECODE_WAVES, self.DECODE_MAX_RUNS)
             plan = meta.scratch.get(key)
             if plan is None or plan["cu_q"] is not meta.host_cu_q:
                 plan = meta.scratch[key] = self._attention_plan(lib, meta, T, num_heads, num_kv_heads, head_dim, window)
@@ -865,7 +865,11 @@ class HipOps(Ops):
     def _attention_plan(self, lib, meta: BatchMeta, T, num_heads, num_kv_heads, head_dim, window) -> dict:
         group = num_heads // num_kv_heads
         singles = meta.num_requests if meta.all_decode else 0
-        if not meta.all_decode and meta.host_cu_q is not None:
+        if not meta.all_decode and meta.singles_bound is not None:
+            # a captured step of portions and single tokens: which requests bring one token is known on the device
+            # only; both kernels are launched for as many as there may be, and each leaves the other's requests alone
+            singles = meta.singles_bound
+        elif not meta.all_decode and meta.host_cu_q is not None:
             singles = int((meta.host_cu_q[1:] - meta.host_cu_q[:-1] == 1).sum())
         plan = {"cu_q": meta.host_cu_q, "decode": singles > 0 and group <= lib.distie_attention_decode_columns()}
         if plan["decode"]:
@@ -882,7 +886,8 @@ class HipOps(Ops):
                                            device=self.device)
             plan["decode_ml"] = torch.empty((meta.num_requests, num_heads, max_splits, 2), dtype=torch.float32,
                                             device=self.device)
-        plan["prefill"] = singles < meta.num_requests or not plan["decode"]
+        plan["prefill"] = singles < meta.num_requests or not plan["decode"] or \
+            (meta.singles_bound is not None and not meta.all_decode)
         if plan["prefill"]:
             plan.update(self._prefill_parts(meta, T, num_heads, head_dim, window))
         return plan

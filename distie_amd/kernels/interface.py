@@ -53,6 +53,10 @@ class BatchMeta:
     host_past: Optional[object] = None
     all_decode: bool = False           # every request brings exactly one token
     table_rows: Optional[torch.Tensor] = None    # int32 [B]: each request's row of the groups' block tables
+    # In a captured step no launch may depend on how the step's tokens are spread over its requests (that is
+    # known on the device only): `max_q` and `max_kv` are then bounds, and so is this, the most requests that
+    # bring exactly one token (None: an implementation may count them from `host_cu_q`).
+    singles_bound: Optional[int] = None
     scratch: dict = field(default_factory=dict)   # what an implementation computes once per step (cos/sin tables)
 
 

@@ -223,6 +223,18 @@ def test_the_fields_of_a_step_as_numbers():
     assert (T, B, R) == (3, 3, 3)
     assert field(1) == [5, 0, 0] and field(3) == [0, 1, 2, 3] and field(4) == [6, 1, 1]
     assert field(5) == [b.slot, 4, 4] and field(6) == [0, 1, 2] and field(7) == [21, 32, 32]
+    # a mixed step padded to 8 tokens and 4 requests, the last row of every request wanted: the first padding
+    # request takes the tokens that are left, at positions 0.. of the sink page
+    b.tables[0] = [1, 5]
+    offsets, T, B, R, max_q, max_kv, *_ = builder.fill(host, [StepEntry("b", [9], [0]), StepEntry("a", [7, 8], [])],
+                                                       pad_requests=2, pad_tokens=3, want_last=True)
+    field = lambda i: host[offsets[i]:offsets[i + 1]].tolist()
+    assert (T, B, R, max_q, max_kv) == (8, 4, 4, 4, 6)
+    assert field(1) == [5, 0, 1, 0, 1, 2, 3, 0] and field(2) == [0, 1, 1, 2, 2, 2, 2, 3]
+    assert field(3) == [0, 1, 3, 7, 8] and field(4) == [6, 2, 4, 1] and field(5) == [b.slot, a.slot, 4, 4]
+    assert field(6) == [0, 2, 6, 7] and field(7) == [21, 12, 13, 32, 33, 34, 35, 32]
+    with pytest.raises(ValueError):
+        builder.fill(host, [StepEntry("b", [9], [0])], pad_tokens=2)
     # what the reference refuses (test_qwen2_batch.py:61-68): a table too short for the new tokens, an empty step
     b.tables[0] = [1]
     with pytest.raises(ValueError):

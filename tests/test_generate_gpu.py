@@ -50,6 +50,8 @@ def test_greedy_and_temperature_mixed_in_one_batch(tmp_path, name, graphs, looka
     assert (llm.steps_ahead > 0) == lookahead
     if graphs:
         assert llm.runner.graphs.captured and llm.runner.graphs.failures == 0
+        # the steps that hold a portion of a prompt are short enough to replay graphs as well
+        assert llm.runner.graphs.captured_mixed and llm.runner.graphs.mixed_replays > 0
     llm.cache.check()
     assert all(f == 48 for f in llm.cache.free_pages())
 
@@ -90,6 +92,7 @@ def test_bfloat16_generation_through_the_scheduler(tmp_path, name, graphs, looka
     assert (llm.steps_ahead > 0) == lookahead
     if graphs:
         assert llm.runner.graphs.captured and llm.runner.graphs.failures == 0
+        assert llm.runner.graphs.captured_mixed and llm.runner.graphs.mixed_replays > 0
     llm.cache.check()
     assert all(f == pages for f in llm.cache.free_pages()) and llm.cache.slots.num_free == llm.cache.num_slots
 

@@ -2,7 +2,8 @@
 
 import pytest
 
-from distie_amd.engine.graphs import bucket_for, decode_buckets
+from distie_amd.engine.batch import StepEntry
+from distie_amd.engine.graphs import DecodeGraphs, bucket_for, decode_buckets, token_buckets
 from distie_amd.parts.attention import context_classes
 
 
@@ -33,6 +34,18 @@ def test_engine_config_holds_the_buckets():
         EngineConfig(graph_buckets=[0])
 
 
+def test_engine_config_reads_the_graph_options_from_the_environment(monkeypatch):
+    from distie_amd.config import EngineConfig
+
+    monkeypatch.setenv("WORKER_GRAPH_BUCKETS", "4,1,32")
+    monkeypatch.setenv("WORKER_GRAPH_TOKENS", "48")
+    config = EngineConfig.from_env()
+    assert config.graph_buckets == (1, 4, 32) and config.graph_tokens == 48
+    assert EngineConfig.from_env(graph_tokens=0).graph_tokens == 0          # an option given wins, zero too
+    with pytest.raises(ValueError):
+        EngineConfig(graph_tokens=-1)
+
+
 def test_bucket_for():
     buckets = decode_buckets(32)
     assert [bucket_for(buckets, n) for n in (1, 3, 8, 9, 17, 32)] == [1, 4, 8, 16, 24, 32]
@@ -52,3 +65,31 @@ def test_context_classes():
     assert all(b <= 1.5 * a for a, b in zip(classes, classes[1:]))
     with pytest.raises(ValueError):
         context_classes(0)
+
+
+def test_token_buckets():
+    assert token_buckets(96) == (16, 24, 32, 48, 64, 96)
+    assert token_buckets(512) == (16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512)
+    assert token_buckets(100) == (16, 24, 32, 48, 64, 96)
+    assert token_buckets(10) == (10,) and token_buckets(1) == ()
+
+
+def test_which_captured_step_takes_a_mixed_step():
+    """(tokens, requests) of the bucket: the smallest token bucket that holds the step and leaves every padding
+    request a token; a step is padded with at least one request unless it fills its token bucket exactly."""
+    graphs = DecodeGraphs(None, 8, mixed_tokens=96)
+    assert graphs.request_buckets == (1, 2, 4, 8, 9)
+    entry = lambda n, want=None: StepEntry(object(), [1] * n, [n - 1] if want is None else want)
+    pick = graphs._mixed_bucket
+    assert pick([entry(5)]) == (16, 2)                      # 11 tokens of padding in one request
+    assert pick([entry(16)]) == (16, 1)                     # fills the bucket: no padding
+    assert pick([entry(15), entry(1)]) == (16, 2)
+    assert pick([entry(14), entry(1), entry(1)]) == (24, 4) # 16 would need a request of padding without a token
+    assert pick([entry(13), entry(1), entry(1)]) == (16, 4)
+    assert pick([entry(40), entry(1)] + [entry(1)] * 6) == (48, 9)
+    assert pick([entry(90), entry(7)]) is None              # more than the largest bucket
+    assert pick([entry(5, want=[0])]) is None               # wants a row that is not its last
+    assert pick([entry(5, want=[3, 4])]) is None
+    assert pick([entry(5, want=[]), entry(3)]) == (16, 4)   # nothing wanted is fine
+    assert DecodeGraphs(None, 8)._mixed_bucket([entry(5)]) is None      # switched off
+    assert DecodeGraphs(None, 8).request_buckets == (1, 2, 4, 8, 9)
