@@ -1,5 +1,6 @@
-"""Captured decode steps: a step in which every request brings exactly one token replays
-a HIP graph of the whole forward instead of launching its kernels one by one.
+"""Captured steps: a step in which every request brings exactly one token, and a short step that
+holds portions of prompts as well, replays a HIP graph of the whole forward instead of launching its
+kernels one by one.
 
 As in the reference (worker/src/inference/qwen2/batch_decode.py:42-211): batch sizes are
 rounded up to a bucket (1, 2, 4, 8, then steps of 8, and the maximum); each bucket has its
@@ -19,6 +20,13 @@ One number of the step is frozen into a graph all the same: the longest context 
 (`Part.capture_context`; attention answers with classes of length, since it cuts the keys into runs
 by that number): a bucket keeps one graph per answer of the model, each captured when a step first
 needs it.
+
+Short mixed steps (the reference captures decode steps only): a step of at most `mixed_tokens` tokens in
+which every request wants the logits of its last token or none is padded to a bucket of tokens and a
+bucket of requests; the requests added write to the sink page, and the first of them takes whatever
+tokens are left over. Which request brings one token is then a fact of the device's buffers, not of the
+graph: the kernels are launched for as many single tokens as there may be (`BatchMeta.singles_bound`).
+The logits buffer of such a graph has one row a request.
 """
 
 from __future__ import annotations

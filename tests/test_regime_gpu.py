@@ -189,3 +189,81 @@ def test_random_weights_on_the_device_are_those_of_the_written_folder(tmp_path):
         want = plain.forward(weights, cfg, ids, torch.float64).float()
         diff = (got.cpu() - want).abs().max().item()
         assert diff < (1e-4 if dtype == "fp32" else want.abs().max().item() / 16)
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "fp32"), ("B", "fp32"), ("C", "fp32"), ("B", "bf16"), ("C", "bf16")])
+def test_short_mixed_steps_replay_graphs_and_give_the_plain_logits(tmp_path, name, dtype):
+    """Steps that hold portions of prompts, short enough to be captured: up to four live requests, portions of 2
+    to 20 tokens beside single tokens, requests that sit a step out, want their last row or nothing, end and
+    give their pages to the next. Every such step goes through a graph (a first use captures, a second
+    replays: the same buckets come again with other requests, lengths and pages), none falls back, and every
+    row is the plain model's."""
+    import random
+
+    cfg, block = {"A": (plain.TINY_A, 4), "B": (plain.TINY_B, 8), "C": (plain.TINY_C, 16)}[name]
+    act = torch.float32 if dtype == "fp32" else torch.bfloat16
+    folder, weights = make_model_dir(tmp_path, cfg, seed=53, dtype=act)
+    lengths = [70, 45, 90, 33, 58, 64, 21, 80]
+    pages = 2 * (-(-90 // block)) + 4              # two of the longest and a little: pages come back and go out again
+    llm = LLM(folder, dtype=dtype, block_size=block, num_blocks=pages, max_seqs=4, graph_tokens=48, lookahead=False)
+    graphs = llm.runner.graphs
+    rng = random.Random(7)
+    waiting = [(f"r{i}", random_ids(cfg, n, 500 + n)) for i, n in enumerate(lengths)]
+    live, at, rows = {}, {}, {}
+    mixed = decode = 0
+    while waiting or live:
+        while waiting and len(live) < 4 and \
+                sum(-(-len(ids) // block) for ids in live.values()) + -(-len(waiting[0][1]) // block) <= pages:
+            rid, ids = waiting.pop(0)
+            live[rid], at[rid], rows[rid] = ids, 0, []
+        entries, budget = [], 48
+        for rid, ids in live.items():
+            left = len(ids) - at[rid]
+            if rng.random() < 0.15 or budget < 2:
+                continue                                                    # sits this step out
+            if at[rid] > 0 and rng.random() < 0.5:
+                n = 1
+            else:
+                n = min(left, budget, rng.choice((2, 2, 3, 5, 8, 13, 20)))
+            want = [] if rng.random() < 0.2 else [n - 1]
+            entries.append((rid, n, want))
+            budget -= n
+        if not entries:
+            continue
+        entries.sort(key=lambda e: e[1] != 1)                              # single tokens lead a step
+        step = [StepEntry(rid, live[rid][at[rid]:at[rid] + n], want) for rid, n, want in entries]
+        before = graphs.mixed_replays, graphs.replays
+        out = llm.step(step)                                             # None if no row was wanted
+        logits = out.float().cpu() if out is not None else torch.zeros(0, cfg["vocab_size"])
+        if all(n == 1 for _, n, _ in entries):
+            decode += 1
+        else:
+            mixed += 1
+            assert graphs.mixed_replays == before[0] + 1, [(n, want) for _, n, want in entries]
+        row = 0
+        for rid, n, want in entries:
+            at[rid] += n
+            if want:
+                rows[rid].append((at[rid] - 1, logits[row]))
+                row += 1
+        assert row == logits.shape[0]
+        for rid in [r for r in live if at[r] == len(live[r])]:
+            ids = live.pop(rid)
+            llm.finish(rid)
+            want = plain.forward(weights, cfg, ids, torch.float64).float()
+            places = [p for p, _ in rows[rid]]
+            assert len(places) >= 2
+            diff = torch.stack([r for _, r in rows[rid]]) - want[places]
+            scale = want.abs().max().item()
+            if dtype == "fp32":
+                assert diff.abs().max().item() < 1e-4, (rid, diff.abs().max().item())
+            else:
+                assert diff.abs().max().item() < scale / 16, (rid, diff.abs().max().item(), scale)
+                assert diff.pow(2).mean().sqrt().item() < scale / 64, rid
+    assert graphs.failures == 0 and mixed >= 30 and graphs.mixed_replays == mixed
+    shapes = graphs.captured_mixed
+    assert len({(tokens, requests) for tokens, requests, _ in shapes}) >= 5, shapes
+    assert graphs.mixed_replays >= len(shapes) + 10            # many steps replayed a graph made by an earlier one
+    llm.cache.check()
+    assert all(f == pages for f in llm.cache.free_pages()) and llm.cache.slots.num_free == llm.cache.num_slots
+    llm.close()
