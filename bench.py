@@ -206,6 +206,8 @@ def main() -> int:
     parser.add_argument("--no-points", action="store_true", help="skip the other batch sizes")
     parser.add_argument("--no-tune", action="store_true",
                         help="leave the choice of the library's product kernels (prefill) to the library's defaults")
+    parser.add_argument("--step-stats", action="store_true",
+                        help="with --serve: add the mean time of a step on the host and on the device, by kind of step")
     parser.add_argument("--gpu-mem-fraction", type=float, default=None,
                         help="size the cache from free memory (the default for --shape 32b and --serve: 0.9)")
     parser.add_argument("--packed-weights", default=None, metavar="ROLES",
@@ -241,7 +243,7 @@ def main() -> int:
         packed = False if args.packed_weights == "none" else tuple(r for r in args.packed_weights.split(",") if r)
     llm = LLM(config=shape, random_weights=True, seed=0, dtype=args.dtype, block_size=BLOCK_SIZE, num_blocks=pages,
               gpu_mem_fraction=fraction, max_seqs=max_batch, token_budget=TOKEN_BUDGET, use_graphs=True,
-              packed_weights=packed, tune_products=not args.no_tune)
+              packed_weights=packed, tune_products=not args.no_tune, step_stats=10 ** 9 if args.step_stats else 0)
     vocab = shape["vocab_size"]
     elem = 2 if args.dtype == "bf16" else 4
     body, head = linear_params(shape)
@@ -258,6 +260,8 @@ def main() -> int:
 
     if args.serve:
         served = serve_run(llm, vocab, seed=7)             # the first pass captures the graphs and warms the library
+        if llm.stats is not None:
+            llm.stats.flush()                              # forget the first pass
         served = serve_run(llm, vocab, seed=7)
         config.update({"global_batch": SERVE["requests"], "seq_len": "prompts U[128,2048], outputs U[32,256]",
                        "prefill_tokens": served["prompt_tokens"]})
@@ -278,6 +282,10 @@ def main() -> int:
                 "e2e_latency_ms": {k: round(v, 1) for k, v in served["e2e_latency_ms"].items()},
             },
         }
+        if llm.stats is not None:
+            llm.stats._read(keep=0)
+            line["serve"]["step_ms"] = {kind: {k: round(v, 3) for k, v in row.items()}
+                                        for kind, row in llm.stats.summary().items()}
         print(json.dumps(line), flush=True)
         return 0
 
