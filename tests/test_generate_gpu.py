@@ -56,6 +56,33 @@ def test_greedy_and_temperature_mixed_in_one_batch(tmp_path, name, graphs, looka
     assert all(f == 48 for f in llm.cache.free_pages())
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_the_two_tiny_workloads_at_their_named_sizes_and_spread(tmp_path, name):
+    """The two tiny workloads exactly as they are named for this engine: Tiny B with a feed-forward width of 256
+    and a vocabulary of 320 (the other tests give it 250 and 323, which end inside a tile), weights and biases
+    drawn from N(0, 0.02) and norm weights of one (the other tests spread the weights further and move the norms,
+    so that a fault shows in the logits; here the logits of a row lie close together, so the check has two halves:
+    the row every token was drawn from is the oracle's within the float32 bound, and the token is the plain draw
+    from that row)."""
+    cfg, block, lengths, new, budget = WORKLOADS[name]
+    if name == "B":
+        cfg = dict(cfg, intermediate_size=256, vocab_size=320)
+    weights = plain.random_weights(cfg, seed=91, std=0.02, norm_jitter=0.0)
+    folder = tmp_path / "model"
+    plain.write_model_dir(folder, cfg, weights)
+    prompts = [random_ids(cfg, n, 700 + n) for n in lengths]
+    params = [SamplingParams(max_new_tokens=new, temperature=0.7 if name == "B" and i % 2 == 0 else 0.0, seed=300 + i)
+              for i in range(len(prompts))]
+    llm = LLM(folder, dtype="fp32", block_size=block, num_blocks=48, token_budget=budget)
+    outs, kept = run_and_keep_logits(llm, prompts, params)
+    for prompt, sp, out in zip(prompts, params, outs):
+        assert len(out.token_ids) == new and out.finish_reason == "length"
+        check_generation_in_two_halves(weights, cfg, prompt, out.token_ids, kept[out.request_id], torch.float32,
+                                       sp.temperature, sp.seed)
+    llm.cache.check()
+    assert all(f == 48 for f in llm.cache.free_pages())
+
+
 BF16_WORKLOADS = {
     "B": (plain.TINY_B, 8, (1, 9, 23, 40), 12, 7),
     "C": (plain.TINY_C, 16, (3, 30, 70, 18, 44), 20, 33),
