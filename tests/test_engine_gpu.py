@@ -162,18 +162,30 @@ def test_a_file_in_32_bit_under_a_bfloat16_engine(tmp_path, ops):
     check_logits(replay_cut(runner, "a", ids, [50, 20, 3]), weights, cfg, ids, torch.bfloat16, folder)
 
 
-def test_layer_sizes_of_the_1_5b_model(tmp_path, ops):
-    """Two layers with the sizes the benchmark runs (width 1,536, 12 heads over 2 kv heads of 128, feed-forward
-    8,960, vocabulary 151,936, tied head): sizes the tiny configurations do not reach (products cut along
-    8,960, rows of the head beyond 2^17, head size 128). One file in bfloat16 serves both engines, since the
-    float32 engine keeps every tensor in 32-bit whatever the file holds."""
-    cfg = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 2, "hidden_size": 1536,
-           "num_attention_heads": 12, "num_key_value_heads": 2, "head_dim": 128, "intermediate_size": 8960,
-           "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
-           "max_position_embeddings": 4096, "hidden_act": "silu"}
-    folder, weights = make_model_dir(tmp_path, cfg, seed=19, std=0.03, dtype=torch.bfloat16)
+LAYER_SIZES = {
+    "1.5b": dict(hidden_size=1536, num_attention_heads=12, num_key_value_heads=2, intermediate_size=8960,
+                 vocab_size=151936, tie_word_embeddings=True),
+    "7b": dict(hidden_size=3584, num_attention_heads=28, num_key_value_heads=4, intermediate_size=18944,
+               vocab_size=152064, tie_word_embeddings=False),
+}
+
+
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("shape", sorted(LAYER_SIZES))
+def test_layer_sizes_of_the_models_the_benchmark_runs(tmp_path, ops, shape):
+    """Two layers with the sizes the benchmark runs: width 1,536, 12 heads over 2 kv heads of 128, feed-forward
+    8,960, vocabulary 151,936, tied head; and width 3,584, 28 heads over 4 kv heads (seven to a kv head),
+    feed-forward 18,944, vocabulary 152,064, a head of its own. Sizes the tiny configurations do not reach
+    (products cut along 8,960 and 18,944, rows of the head beyond 2^17, head size 128). One file in bfloat16
+    serves both engines, since the float32 engine keeps every tensor in 32-bit whatever the file holds."""
+    cfg = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 2, "head_dim": 128,
+           "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "max_position_embeddings": 4096, "hidden_act": "silu",
+           **LAYER_SIZES[shape]}
+    folder, weights = make_model_dir(tmp_path, cfg, seed=19, std=0.03 if shape == "1.5b" else 0.02, dtype=torch.bfloat16)
     seqs = {"a": random_ids(cfg, 120, 1), "b": random_ids(cfg, 45, 2)}
-    want = {name: plain.forward(weights, cfg, ids, torch.float64).float() for name, ids in seqs.items()}
+    on_device = {k: v.to("cuda", torch.float64) for k, v in weights.items()}
+    want = {name: plain.forward(on_device, cfg, ids, torch.float64).float().cpu() for name, ids in seqs.items()}
+    del on_device
     for dtype in (torch.float32, torch.bfloat16):
         runner = build_runner(folder, ops, dtype, block_size=16, num_blocks=24, max_model_len=4096)
         got = {name: [] for name in seqs}
