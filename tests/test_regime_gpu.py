@@ -1,5 +1,6 @@
 """The regime that the benchmark times, checked against the plain implementation: the layer sizes of the
-1.5B model, contexts beyond 2,048 tokens, 8 and 64 requests, prompts fed in portions of the token budget,
+1.5B model (and, in bfloat16, of the 7B model: seven query heads to a kv head, products cut along 18,944),
+contexts beyond 2,048 tokens, 8 and 64 requests, prompts fed in portions of the token budget,
 decoding through captured steps that are launched ahead of the host (worker/tests/test_model_runner.py:72-80
 holds the graph path against the eager one at tiny sizes; here the sizes are the benchmark's and the judge
 is the plain model). Also: what two ways of cutting the same tokens leave in the cache
@@ -18,20 +19,31 @@ SIZES_1_5B = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num
               "num_attention_heads": 12, "num_key_value_heads": 2, "head_dim": 128, "intermediate_size": 8960,
               "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
               "max_position_embeddings": 4096, "hidden_act": "silu"}
+SIZES_7B = dict(SIZES_1_5B, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4, intermediate_size=18944,
+                vocab_size=152064, tie_word_embeddings=False, max_position_embeddings=8192)
 NEW_TOKENS = 41          # the token drawn from the prompt's last row, then 40 decode steps
 
 
 @pytest.fixture(scope="module")
-def model_1_5b(tmp_path_factory):
-    folder, weights = make_model_dir(tmp_path_factory.mktemp("regime"), SIZES_1_5B, seed=29, std=0.03, dtype=torch.bfloat16)
-    on_device = {k: v.to("cuda", torch.float64) for k, v in weights.items()}
-    return folder, on_device
+def models(tmp_path_factory):
+    """shape -> (folder, float64 weights on the device, sizes), made when first asked for and dropped with the module."""
+    made = {}
+
+    def get(shape):
+        if shape not in made:
+            sizes, std = {"1.5b": (SIZES_1_5B, 0.03), "7b": (SIZES_7B, 0.02)}[shape]
+            made.clear()                    # one set of float64 weights on the device at a time
+            folder, weights = make_model_dir(tmp_path_factory.mktemp("regime"), sizes, seed=29, std=std, dtype=torch.bfloat16)
+            made[shape] = (folder, {k: v.to("cuda", torch.float64) for k, v in weights.items()}, sizes)
+        return made[shape]
+
+    return get
 
 
 @pytest.mark.timeout(900)
-@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
-def test_the_regime_the_benchmark_times(model_1_5b, dtype):
-    folder, weights = model_1_5b
+@pytest.mark.parametrize("shape,dtype", [("1.5b", "bf16"), ("1.5b", "fp32"), ("7b", "bf16")])
+def test_the_regime_the_benchmark_times(models, shape, dtype):
+    folder, weights, SIZES = models(shape)
     llm = LLM(folder, dtype=dtype, block_size=16, num_blocks=64 * 144 + 8, max_seqs=64, token_budget=2048,
               max_model_len=4096, use_graphs=True, lookahead=True)
     graphs = llm.runner.graphs
@@ -40,7 +52,7 @@ def test_the_regime_the_benchmark_times(model_1_5b, dtype):
         replays, ahead = graphs.replays, llm.steps_ahead
         # prompts of 2,048 tokens and a few more: no portion ends where a prompt ends, steps hold the end of one
         # prompt beside the start of the next, and requests that were admitted early decode beside them
-        prompts = [random_ids(SIZES_1_5B, 2048 + (5 * i) % 13, 100 * batch + i) for i in range(batch)]
+        prompts = [random_ids(SIZES, 2048 + (5 * i) % 13, 100 * batch + i) for i in range(batch)]
         # a request that is admitted early decodes while the prompts of the others are run, a portion or two a
         # step: every request gets so many tokens more that its last 41 are drawn with all of them decoding
         new = NEW_TOKENS + 2 * batch + 8
@@ -55,7 +67,7 @@ def test_the_regime_the_benchmark_times(model_1_5b, dtype):
             assert out.finish_reason == "length" and len(out.token_ids) == new
             ids = prompt + out.token_ids[:-1]            # the tokens the engine saw, whatever it drew
             rows = list(range(len(ids) - NEW_TOKENS, len(ids)))
-            want = plain.forward(weights, SIZES_1_5B, ids, torch.float64, rows=rows).float()
+            want = plain.forward(weights, SIZES, ids, torch.float64, rows=rows).float()
             mine = kept[out.request_id]
             assert [position for position, _ in mine] == list(range(len(prompt) - 1, len(ids)))
             got = torch.stack([row for _, row in mine[-NEW_TOKENS:]])
