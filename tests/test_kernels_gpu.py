@@ -628,6 +628,18 @@ def test_paged_attention_keys_walked_in_parts(ops, dtype, heads, kv_heads, dim, 
                                             dim ** -0.5, window)
     got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
     close(got, want, dtype, scale=want.abs().max().item())
+    # The merge reads only what the kernel before it wrote in this call: whatever the buffers between the two
+    # kernels held before (here: NaN everywhere), the result is the same.
+    filled = 0
+    for plan in meta.scratch.values():
+        for name in ("prefill_o", "prefill_ml"):
+            if isinstance(plan, dict) and name in plan:
+                plan[name].fill_(float("nan"))
+                filled += 1
+    tiled = dtype == torch.bfloat16 or (dim % 32 == 0 and dim <= 128)       # else: the wave-per-token kernel, no parts
+    assert (filled >= 2) == tiled
+    again = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
+    assert torch.equal(again, got)
     meta.host_cu_q = None                      # the tiled kernel takes the single tokens too
     got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, window)
     close(got, want, dtype, scale=want.abs().max().item())
