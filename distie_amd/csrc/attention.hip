@@ -1236,7 +1236,7 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
 // of requests that the kernel skipped (fewer than min_q_len tokens) are skipped here as well.
 constexpr int PF_MAX_SPLITS = 16;
 
-template <typename OUT>
+template <typename OUT, int MOST>
 __global__ void attn_prefill_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                           const int32_t* __restrict__ token_request, const int32_t* __restrict__ cu_q,
                                           OUT* __restrict__ out, int tokens, int heads, int min_q_len, int splits) {
@@ -1248,17 +1248,18 @@ __global__ void attn_prefill_merge_kernel(const float* __restrict__ part_o, cons
     const int head = i / (D / 4);
     const int d = 4 * (i % (D / 4));
     const int64_t row = token * heads + head;
-    float2 ml[PF_MAX_SPLITS];
-    float4 o[PF_MAX_SPLITS];
+    float2 ml[MOST];
+    float4 o[MOST];
     float m = -INFINITY;
 #pragma unroll
-    for (int s = 0; s < PF_MAX_SPLITS; ++s) {
+    for (int s = 0; s < MOST; ++s) {
       ml[s] = float2{-INFINITY, 0.f};
       o[s] = float4{0.f, 0.f, 0.f, 0.f};
       if (s < splits) ml[s] = *reinterpret_cast<const float2*>(part_ml + 2 * (s * part + row));
       // a part without a key for this token has l = 0; what it left in part_o is not read (for a prompt
       // without a past that is a third of all reads: asking for them anyway, to save the second trip to
-      // memory, made this kernel slower where it runs, 12.2 -> 14.7 us)
+      // memory, made this kernel slower where it runs, 12.2 -> 14.7 us, and 10.0 -> 10.5 once the registers of
+      // the parts that are not there no longer held waves back)
       if (s < splits && ml[s].y > 0.f) {
         o[s] = *reinterpret_cast<const float4*>(part_o + (s * part + row) * D + d);
         m = fmaxf(m, ml[s].x);
@@ -1267,7 +1268,7 @@ __global__ void attn_prefill_merge_kernel(const float* __restrict__ part_o, cons
     float l = 0.f;
     float4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int s = 0; s < PF_MAX_SPLITS; ++s) {
+    for (int s = 0; s < MOST; ++s) {
       const float w = ml[s].y > 0.f ? fast_exp2(ml[s].x - m) : 0.f;
       l += w * ml[s].y;
       sum.x += w * o[s].x;
@@ -1286,6 +1287,24 @@ __global__ void attn_prefill_merge_kernel(const float* __restrict__ part_o, cons
       *reinterpret_cast<uint2*>(out + row * D + d) = uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
     }
   }
+}
+
+// The merge holds every part's maximum, sum and four outputs in registers: compiled for at most 4, 8 and 16 parts,
+// so that few parts leave room for more waves on a compute unit.
+template <typename OUT>
+static void launch_merge(const float* part_o, const float* part_ml, const int32_t* token_request, const int32_t* cu_q,
+                         OUT* out, int tokens, int heads, int min_q_len, int splits, hipStream_t stream) {
+  const int work = heads * (D / 4);
+  const int threads = work >= 512 ? 512 : (work >= 256 ? 256 : 64);
+  if (splits <= 4)
+    attn_prefill_merge_kernel<OUT, 4><<<tokens, threads, 0, stream>>>(part_o, part_ml, token_request, cu_q, out, tokens,
+                                                                       heads, min_q_len, splits);
+  else if (splits <= 8)
+    attn_prefill_merge_kernel<OUT, 8><<<tokens, threads, 0, stream>>>(part_o, part_ml, token_request, cu_q, out, tokens,
+                                                                       heads, min_q_len, splits);
+  else
+    attn_prefill_merge_kernel<OUT, PF_MAX_SPLITS><<<tokens, threads, 0, stream>>>(part_o, part_ml, token_request, cu_q, out,
+                                                                                   tokens, heads, min_q_len, splits);
 }
 
 // Portions of prompts (and whole mixed steps). bfloat16 only; block_size must be a multiple of 16. Requests that
@@ -1311,9 +1330,7 @@ extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, 
       kv_heads, block_size, scale, window, min_q_len);
   int status = launch_status();
   if (status != 0 || splits == 1) return status;
-  const int work = heads * (D / 4);
-  attn_prefill_merge_kernel<bf16_t><<<tokens, work >= 512 ? 512 : (work >= 256 ? 256 : 64), 0, stream>>>(
-      part_o, part_ml, token_request, cu_q, static_cast<bf16_t*>(out), tokens, heads, min_q_len, splits);
+  launch_merge(part_o, part_ml, token_request, cu_q, static_cast<bf16_t*>(out), tokens, heads, min_q_len, splits, stream);
   return launch_status();
 }
 
@@ -1600,9 +1617,7 @@ extern "C" int distie_attention_prefill_f32(const void* qkv, int64_t q_stride, c
       heads, kv_heads, block_size, scale, window, min_q_len);
   int status = launch_status();
   if (status != 0 || splits == 1) return status;
-  const int work = heads * (D / 4);
-  attn_prefill_merge_kernel<float><<<tokens, work >= 512 ? 512 : (work >= 256 ? 256 : 64), 0, stream>>>(
-      part_o, part_ml, token_request, cu_q, static_cast<float*>(out), tokens, heads, min_q_len, splits);
+  launch_merge(part_o, part_ml, token_request, cu_q, static_cast<float*>(out), tokens, heads, min_q_len, splits, stream);
   return launch_status();
 #else
   return DISTIE_BAD_ARGUMENT;
