@@ -309,12 +309,53 @@ static __device__ __forceinline__ uint4 pack8(const float v[8]) {
   return uint4{w[0], w[1], w[2], w[3]};
 }
 
+// Blocks 0 .. tokens - 1 turn q and k of one token each and write k into the cache; the blocks behind them write v
+// into the cache for 16 tokens each: the cache keeps v with the key index innermost, so one token's values lie
+// block_size elements apart, and 16 tokens that follow one another inside a page fill 32 bytes in a row, written
+// by one thread as two 16-byte stores instead of 16 stores of 2 bytes from 16 blocks.
+constexpr int V_GROUP = 16;
+
 __global__ void rope_kv_write_bf16_kernel(const bf16_t* in, bf16_t* out, const float2* __restrict__ table,
                                           const int32_t* __restrict__ slots, bf16_t* __restrict__ k_cache,
-                                          bf16_t* __restrict__ v_cache, int heads, int kv_heads, int dim,
+                                          bf16_t* __restrict__ v_cache, int tokens, int heads, int kv_heads, int dim,
                                           int block_size, int write) {
-  const int64_t t = blockIdx.x;
   const int64_t width = static_cast<int64_t>(heads + 2 * kv_heads) * dim;
+  if (static_cast<int>(blockIdx.x) >= tokens) {
+    const int t0 = (static_cast<int>(blockIdx.x) - tokens) * V_GROUP;
+    const int n = min(V_GROUP, tokens - t0);
+    const int64_t slot0 = slots[t0];
+    // one run inside a page, a whole group, at a place where 16-byte stores are aligned?
+    bool together = n == V_GROUP && block_size % 8 == 0 && slot0 % block_size % 8 == 0 &&
+                    slot0 % block_size + V_GROUP <= block_size;
+#pragma unroll
+    for (int i = 1; i < V_GROUP; ++i) together = together && slots[min(t0 + i, tokens - 1)] == slot0 + i;
+    const uint16_t* src = reinterpret_cast<const uint16_t*>(in) + static_cast<int64_t>(heads + kv_heads) * dim;
+    uint16_t* cache = reinterpret_cast<uint16_t*>(v_cache);
+    for (int item = threadIdx.x; item < kv_heads * dim; item += blockDim.x) {
+      const int head = item / dim;
+      const int d = item % dim;
+      uint32_t v[V_GROUP];
+#pragma unroll
+      for (int i = 0; i < V_GROUP; ++i) v[i] = src[min(t0 + i, tokens - 1) * width + item];
+      if (together) {
+        const int64_t page = slot0 / block_size;
+        uint16_t* dst = cache + ((page * kv_heads + head) * dim + d) * block_size + slot0 % block_size;
+        *reinterpret_cast<uint4*>(dst) = uint4{v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16)};
+        *reinterpret_cast<uint4*>(dst + 8) =
+            uint4{v[8] | (v[9] << 16), v[10] | (v[11] << 16), v[12] | (v[13] << 16), v[14] | (v[15] << 16)};
+      } else {
+#pragma unroll
+        for (int i = 0; i < V_GROUP; ++i) {
+          if (i >= n) break;
+          const int64_t slot = slots[t0 + i];
+          const int64_t page = slot / block_size;
+          cache[((page * kv_heads + head) * dim + d) * block_size + slot % block_size] = static_cast<uint16_t>(v[i]);
+        }
+      }
+    }
+    return;
+  }
+  const int64_t t = blockIdx.x;
   const bf16_t* src = in + t * width;
   bf16_t* row = out + t * width;
   const int64_t slot = write ? slots[t] : 0;
@@ -352,22 +393,12 @@ __global__ void rope_kv_write_bf16_kernel(const bf16_t* in, bf16_t* out, const f
       *reinterpret_cast<uint4*>(at + half) = pb;
     }
   }
-  // v: copied (nothing to do in place), and written into the cache with the key index innermost
+  // v: copied (nothing to do in place); the blocks behind the tokens' write it into the cache
+  if (row == src) return;
   const int v_items = kv_heads * (dim / 8);
   for (int i = threadIdx.x; i < v_items; i += blockDim.x) {
-    const int head = i / (dim / 8);
-    const int d0 = 8 * (i % (dim / 8));
-    const int64_t at = static_cast<int64_t>(rotated_heads + head) * dim + d0;
-    const uint4 raw = *reinterpret_cast<const uint4*>(src + at);
-    if (row != src) *reinterpret_cast<uint4*>(row + at) = raw;
-    if (!write) continue;
-    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-    uint16_t* dst = reinterpret_cast<uint16_t*>(v_cache) + ((page * kv_heads + head) * dim + d0) * block_size + offset;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      dst[static_cast<int64_t>(2 * e) * block_size] = static_cast<uint16_t>(w[e] & 0xffffu);
-      dst[static_cast<int64_t>(2 * e + 1) * block_size] = static_cast<uint16_t>(w[e] >> 16);
-    }
+    const int64_t at = static_cast<int64_t>(rotated_heads) * dim + 8 * i;
+    *reinterpret_cast<uint4*>(row + at) = *reinterpret_cast<const uint4*>(src + at);
   }
 }
 
@@ -383,12 +414,13 @@ extern "C" int distie_rope_kv_write(const void* in, int in_dtype, int slices, vo
   if (slices == 1 && in_dtype == DISTIE_BF16 && dtype == DISTIE_BF16 && cache_dtype == DISTIE_BF16 && dim % 16 == 0 &&
       2 * pairs == dim && table != nullptr && reinterpret_cast<uintptr_t>(in) % 16 == 0 &&
       reinterpret_cast<uintptr_t>(out) % 16 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(v_cache) % 16 == 0 &&
       reinterpret_cast<uintptr_t>(table) % 16 == 0) {
     const int items = (heads + kv_heads) * (dim / 16) + kv_heads * (dim / 8);
     const int threads = items >= 256 ? 256 : (items >= 128 ? 128 : 64);
-    rope_kv_write_bf16_kernel<<<tokens, threads, 0, stream>>>(
+    rope_kv_write_bf16_kernel<<<tokens + (write ? (tokens + V_GROUP - 1) / V_GROUP : 0), threads, 0, stream>>>(
         static_cast<const bf16_t*>(in), static_cast<bf16_t*>(out), static_cast<const float2*>(table), slots,
-        static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), heads, kv_heads, dim, block_size, write);
+        static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), tokens, heads, kv_heads, dim, block_size, write);
     return launch_status();
   }
   const int work = (heads + kv_heads) * dim / 2;
