@@ -530,12 +530,19 @@ constexpr int wd_stages() { return WAVES == 2 && MB == 1 ? 8 : 4; }    // (k-ste
 // row r, byte 16 g) free of bank conflicts; with 16 bytes more every read costs twice (measured)
 constexpr int WD_XROW = SK_KSTEP + 16;
 
+// MODE PK_ROTARY here: the weight is the ROTARY copy of a stacked q/k/v weight (rotation partners in one block), the
+// result is the plain product, every sum written to the column its row of W has: the rotation needs the whole
+// sum over K, which this kernel cuts into slices, so it is left to the kernel that adds the slices.
+struct HeadRows {
+  int heads, kv_heads, dim;
+};
+
 template <typename Y, int MODE, int MB, int WD_WAVES>
 __global__ __launch_bounds__(64 * WD_WAVES) void gemm_packed_wide_kernel(const bf16_t* __restrict__ x,
                                                                const bf16_t* __restrict__ w,
                                                                const float* __restrict__ bias, Y* __restrict__ y,
                                                                int M, int N, int K, int row_blocks, int tiles_per_slice,
-                                                               int m_group) {
+                                                               int m_group, HeadRows head_rows) {
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][MB * 16][WD_XROW];
   // blockIdx.z: a group of m_group rows of x. The groups run one after the other over the whole weight, so
   // the second reads it from the memory-side cache (if it fits there; the launcher decides).
@@ -663,10 +670,19 @@ __global__ __launch_bounds__(64 * WD_WAVES) void gemm_packed_wide_kernel(const b
     } else {
       Y* out = y + static_cast<int64_t>(blockIdx.y) * m_all * N;
       const bool with_bias = bias != nullptr && blockIdx.y == 0;
+      int64_t n0 = static_cast<int64_t>(block) * 16 + 4 * g;        // the column of the lane's first sum
+      if constexpr (MODE == PK_ROTARY) {
+        // block (head, sub) of a q or k head holds the head's rows 8 sub .. + 7 and dim / 2 + 8 sub .. + 7
+        const int per_head = head_rows.dim / 16;
+        const int head = block / per_head;
+        const int sub = block % per_head;
+        if (head < head_rows.heads + head_rows.kv_heads)
+          n0 = static_cast<int64_t>(head) * head_rows.dim + (g / 2) * (head_rows.dim / 2) + 8 * sub + 4 * (g % 2);
+      }
       if (m < M) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int64_t n = static_cast<int64_t>(block) * 16 + 4 * g + i;
+          const int64_t n = n0 + i;
           if (n < N) out[static_cast<int64_t>(m) * N + n] = from_float<Y>(acc[b][i] + (with_bias ? bias[n] : 0.f));
         }
       }
@@ -696,10 +712,10 @@ extern "C" int distie_gemm_packed_wide_slices(int N, int K) {
 // 17 to 256 rows of x, at most 64 a pass. mode 0: y [M, N] of y_dtype, or float32 [slices, M, N] when the plan cuts K
 // (distie_gemm_packed_wide_slices); 1 (gated): [M, N / 2].
 static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bias, void* y, int y_dtype, int M, int N,
-                              int K, int mode, int pass_blocks, hipStream_t stream) {
+                              int K, int mode, int pass_blocks, hipStream_t stream, HeadRows head_rows = HeadRows{0, 0, 0}) {
   const int row_blocks = mode == PK_GATED ? (N / 2 + 7) / 8 : (N + 15) / 16;
   int slices = 1, tiles_per_slice = 4 * ((K + SK_KSTEP - 1) / SK_KSTEP);
-  if (mode == PK_PLAIN) wide_plan(row_blocks, K, &slices, &tiles_per_slice);
+  if (mode != PK_GATED) wide_plan(row_blocks, K, &slices, &tiles_per_slice);
   if (slices > 1 && y_dtype != DISTIE_F32) return DISTIE_BAD_ARGUMENT;
   // pass_blocks: the rows of x are taken in passes of 16 * pass_blocks rows over the weight (0: all at once),
   // with more workgroups and fewer registers and less LDS each; worth it if the weight fits the memory-side
@@ -712,7 +728,7 @@ static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bia
   dim3 grid((row_blocks + waves - 1) / waves, slices, groups);
 #define WIDE(MODE, MB, WAVES)                                                                                   \
   DISTIE_DISPATCH(y_dtype, Y, (gemm_packed_wide_kernel<Y, MODE, MB, WAVES><<<grid, 64 * WAVES, 0, stream>>>(    \
-                                  x, w, bias, static_cast<Y*>(y), M, N, K, row_blocks, tiles_per_slice, m_group)))
+                                  x, w, bias, static_cast<Y*>(y), M, N, K, row_blocks, tiles_per_slice, m_group, head_rows)))
 #define WIDE_MB(MODE)                                   \
   switch (mb) {                                         \
     case 1: WIDE(MODE, 1, 2); break;                    \
@@ -725,6 +741,8 @@ static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bia
   }
   if (mode == PK_GATED) {
     WIDE_MB(PK_GATED);
+  } else if (mode == PK_ROTARY) {
+    WIDE_MB(PK_ROTARY);
   } else {
     WIDE_MB(PK_PLAIN);
   }
@@ -740,6 +758,20 @@ extern "C" int distie_gemm_packed_wide_bf16(const void* x, const void* w_packed,
   if (M > 256 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
   return packed_wide_launch(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w_packed), bias, y, y_dtype, M, N,
                             K, gated ? PK_GATED : PK_PLAIN, pass_blocks, stream);
+}
+
+// The stacked q/k/v product alone, on the ROTARY copy of its weight, for 17 rows of x and more against a weight large
+// enough for the wide kernel: y as distie_gemm_packed_wide_bf16 writes it (columns in the weight's own order; float32
+// [slices, M, N] when K is cut, distie_gemm_packed_wide_slices(N, K) says), bias on the first slice. Rotation and
+// cache write are the caller's next kernel.
+extern "C" int distie_gemm_packed_wide_qkv_bf16(const void* x, const void* w_packed, const float* bias, void* y,
+                                                int y_dtype, int M, int K, int heads, int kv_heads, int dim,
+                                                int pass_blocks, hipStream_t stream) {
+  if (M <= 0) return 0;
+  if (M > 256 || K <= 0 || K % 8 != 0 || heads < 1 || kv_heads < 1 || dim < 16 || dim % 16 != 0) return DISTIE_BAD_ARGUMENT;
+  const int N = (heads + 2 * kv_heads) * dim;
+  return packed_wide_launch(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w_packed), bias, y, y_dtype, M, N,
+                            K, PK_ROTARY, pass_blocks, stream, HeadRows{heads, kv_heads, dim});
 }
 
 // The stacked q/k/v product with the rotation and the cache write in its epilogue. w_packed: the ROTARY

@@ -244,6 +244,7 @@ class HipOps(Ops):
         o.distie_gemm_packed_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
         o.distie_gemm_packed_wide_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
         o.distie_gemm_packed_wide_slices.argtypes = [_I, _I]
+        o.distie_gemm_packed_wide_qkv_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         o.distie_gemm_packed_rotary_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         o.distie_decode_norm_fits.argtypes = [_I]
         o.distie_decode_product_residual.argtypes = [_P, _P, _P, _P, _I, _I, _I, _P]
@@ -557,6 +558,21 @@ class HipOps(Ops):
         self._check_cache(k_cache, v_cache, num_kv_heads, meta.block_size, head_dim)
         if M != meta.num_tokens or slots.shape[0] != M:
             raise KernelError("linear_rope_kv_write: rows do not match the batch")
+        if M > self.SKINNY_MAX_ROWS and N * K > self.ROW_GROUPS_MAX_ELEMENTS:
+            # more than one group of 16 rows against a weight that fills the chip through the wide kernel: the
+            # epilogue kernel would read the weight once per group, so the product runs wide (weights once, K in
+            # slices) and the rotation with the cache write behind it adds the slices
+            slices = self._ops.distie_gemm_packed_wide_slices(N, K)
+            shape, dtype = ((M, N), torch.bfloat16) if slices == 1 else ((slices, M, N), torch.float32)
+            product = torch.empty(shape, dtype=dtype, device=self.device)
+            _check(self._ops.distie_gemm_packed_wide_qkv_bf16(
+                x.data_ptr(), packed.data_ptr(), bias.data_ptr() if bias is not None else None, product.data_ptr(),
+                _code(product), M, K, num_heads, num_kv_heads, head_dim, self._pass_blocks(M, N * K), self._stream()),
+                "gemm_packed_wide_qkv_bf16")
+            if slices > 1:
+                product = PartialSums(product, torch.bfloat16)
+            return self.rope_kv_write(product, meta, group, k_cache, v_cache, inv_freq, num_heads, num_kv_heads,
+                                      head_dim, write)
         table = self._rope_table(meta, inv_freq)
         out = torch.empty((M, N), dtype=torch.bfloat16, device=self.device)
         _check(self._ops.distie_gemm_packed_rotary_bf16(

@@ -234,11 +234,15 @@ def test_linear_silu_mul_fused(ops, M, I, K):
 
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 45, 64, 70, 96, 129, 224])
 @pytest.mark.parametrize("heads,kv_heads,dim,K,P", [(3, 1, 32, 2048, 4), (12, 2, 128, 1536, 16), (4, 4, 16, 72, 16),
-                                                    (5, 5, 48, 240, 8), (2, 1, 80, 520, 16), (7, 1, 256, 136, 32)])
+                                                    (5, 5, 48, 240, 8), (2, 1, 80, 520, 16), (7, 1, 256, 136, 32),
+                                                    (28, 4, 128, 3584, 16), (10, 2, 64, 5000, 16), (20, 4, 48, 3200, 8)])
 @pytest.mark.parametrize("with_bias,write", [(True, True), (False, True), (True, False)])
 def test_linear_rope_kv_write_fused(ops, M, heads, kv_heads, dim, K, P, with_bias, write):
     """The q/k/v product with rotation and cache write in its epilogue, against product, rotation
-    and write one after the other in plain torch."""
+    and write one after the other in plain torch. The last three weights are large enough for the wide kernel:
+    from 17 rows on the product runs there, on the same copy of the weight (rotation partners side by side, the
+    sums written to the columns the rows have in the weight itself), and rotation and write follow as a kernel
+    of their own that adds the slices of K."""
     N = (heads + 2 * kv_heads) * dim
     x = rand(M, K, dtype=torch.bfloat16, seed=1)
     w = rand(N, K, dtype=torch.bfloat16, seed=6, scale=1.0 / K ** 0.5)
