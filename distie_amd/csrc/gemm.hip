@@ -690,14 +690,15 @@ __global__ __launch_bounds__(64 * WD_WAVES) void gemm_packed_wide_kernel(const b
   }
 }
 
-// Slices of K for the wide kernel: enough waves for the chip (a thousand), slices of whole k-steps, at least two
-// k-steps long.
+// Slices of K for the wide kernel: enough waves for the chip (five hundred and more: with a thousand the 7B
+// shape's down, o and q/k/v products at 48 and 64 rows were 4-10 % slower, the 1.5B shape's the same), slices of
+// whole k-steps, at least two k-steps long.
 static void wide_plan(int row_blocks, int K, int* slices, int* tiles_per_slice) {
   constexpr int WD_WAVES = 4;             // (the cut does not depend on the workgroups' size: the caller sizes its buffer by it)
   const int groups = (row_blocks + WD_WAVES - 1) / WD_WAVES;
   const int steps = (K + SK_KSTEP - 1) / SK_KSTEP;
   int want = 1;
-  while (want < 64 && groups * want * WD_WAVES < 1024 && steps / (want * 2) >= 2) want *= 2;
+  while (want < 64 && groups * want * WD_WAVES < 512 && steps / (want * 2) >= 2) want *= 2;
   int per = (steps + want - 1) / want;
   *tiles_per_slice = 4 * per;
   *slices = (steps + per - 1) / per;
