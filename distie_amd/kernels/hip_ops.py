@@ -154,6 +154,10 @@ class HipOps(Ops):
     # or, for a weight of at most this many elements (too few row blocks to occupy the chip that way),
     # through the one-wave kernel once per 16 rows of x
     ROW_GROUPS_MAX_ELEMENTS = 4 << 20
+    # the q/k/v product with rotation and cache write in its epilogue exists per 16 rows only; from so many rows on a
+    # weight above that size runs on the wide kernel instead, with rotation and cache write as the kernel behind it
+    # (7B shape, decode step: 1.5 % slower at 24 rows, the same at 32 and 48, 2.7 % faster at 64)
+    WIDE_QKV_MIN_ROWS = 49
     # ... and that kernel takes more than 32 rows in two passes of 32 over a weight of at most this many elements
     # (64 MB: the second pass reads it from the memory-side cache; much larger ones would come from memory twice)
     TWO_PASS_MAX_ELEMENTS = 32 << 20
@@ -558,7 +562,7 @@ class HipOps(Ops):
         self._check_cache(k_cache, v_cache, num_kv_heads, meta.block_size, head_dim)
         if M != meta.num_tokens or slots.shape[0] != M:
             raise KernelError("linear_rope_kv_write: rows do not match the batch")
-        if M > self.SKINNY_MAX_ROWS and N * K > self.ROW_GROUPS_MAX_ELEMENTS:
+        if M >= self.WIDE_QKV_MIN_ROWS and N * K > self.ROW_GROUPS_MAX_ELEMENTS:
             # more than one group of 16 rows against a weight that fills the chip through the wide kernel: the
             # epilogue kernel would read the weight once per group, so the product runs wide (weights once, K in
             # slices) and the rotation with the cache write behind it adds the slices

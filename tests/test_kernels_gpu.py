@@ -240,7 +240,7 @@ def test_linear_silu_mul_fused(ops, M, I, K):
 def test_linear_rope_kv_write_fused(ops, M, heads, kv_heads, dim, K, P, with_bias, write):
     """The q/k/v product with rotation and cache write in its epilogue, against product, rotation
     and write one after the other in plain torch. The last three weights are large enough for the wide kernel:
-    from 17 rows on the product runs there, on the same copy of the weight (rotation partners side by side, the
+    from 49 rows on the product runs there, on the same copy of the weight (rotation partners side by side, the
     sums written to the columns the rows have in the weight itself), and rotation and write follow as a kernel
     of their own that adds the slices of K."""
     N = (heads + 2 * kv_heads) * dim
