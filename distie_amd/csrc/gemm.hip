@@ -690,23 +690,25 @@ __global__ __launch_bounds__(64 * WD_WAVES) void gemm_packed_wide_kernel(const b
   }
 }
 
-// Slices of K for the wide kernel: enough waves for the chip (five hundred and more: with a thousand the 7B
-// shape's down, o and q/k/v products at 48 and 64 rows were 4-10 % slower, the 1.5B shape's the same), slices of
-// whole k-steps, at least two k-steps long.
-static void wide_plan(int row_blocks, int K, int* slices, int* tiles_per_slice) {
-  constexpr int WD_WAVES = 4;             // (the cut does not depend on the workgroups' size: the caller sizes its buffer by it)
+// Slices of K for the wide kernel: enough waves for the chip, slices of whole k-steps, at least two k-steps long.
+// With workgroups of four waves (more than 32 rows of x) five hundred waves and more: with a thousand the 7B shape's
+// down, o and q/k/v products at 48 and 64 rows were 4-10 % slower, the 1.5B shape's the same. With workgroups of two
+// waves (up to 32 rows) a thousand: with five hundred the 32B shape's step at 32 rows was 3 % slower.
+static void wide_plan(int row_blocks, int K, int M, int* slices, int* tiles_per_slice) {
+  constexpr int WD_WAVES = 4;
   const int groups = (row_blocks + WD_WAVES - 1) / WD_WAVES;
   const int steps = (K + SK_KSTEP - 1) / SK_KSTEP;
+  const int enough = M <= 32 ? 1024 : 512;
   int want = 1;
-  while (want < 64 && groups * want * WD_WAVES < 512 && steps / (want * 2) >= 2) want *= 2;
+  while (want < 64 && groups * want * WD_WAVES < enough && steps / (want * 2) >= 2) want *= 2;
   int per = (steps + want - 1) / want;
   *tiles_per_slice = 4 * per;
   *slices = (steps + per - 1) / per;
 }
 
-extern "C" int distie_gemm_packed_wide_slices(int N, int K) {
+extern "C" int distie_gemm_packed_wide_slices(int M, int N, int K) {
   int slices, per;
-  wide_plan((N + 15) / 16, K, &slices, &per);
+  wide_plan((N + 15) / 16, K, M, &slices, &per);
   return slices;
 }
 
@@ -716,7 +718,7 @@ static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bia
                               int K, int mode, int pass_blocks, hipStream_t stream, HeadRows head_rows = HeadRows{0, 0, 0}) {
   const int row_blocks = mode == PK_GATED ? (N / 2 + 7) / 8 : (N + 15) / 16;
   int slices = 1, tiles_per_slice = 4 * ((K + SK_KSTEP - 1) / SK_KSTEP);
-  if (mode != PK_GATED) wide_plan(row_blocks, K, &slices, &tiles_per_slice);
+  if (mode != PK_GATED) wide_plan(row_blocks, K, M, &slices, &tiles_per_slice);
   if (slices > 1 && y_dtype != DISTIE_F32) return DISTIE_BAD_ARGUMENT;
   // pass_blocks: the rows of x are taken in passes of 16 * pass_blocks rows over the weight (0: all at once),
   // with more workgroups and fewer registers and less LDS each; worth it if the weight fits the memory-side
@@ -763,7 +765,7 @@ extern "C" int distie_gemm_packed_wide_bf16(const void* x, const void* w_packed,
 
 // The stacked q/k/v product alone, on the ROTARY copy of its weight, for 17 rows of x and more against a weight large
 // enough for the wide kernel: y as distie_gemm_packed_wide_bf16 writes it (columns in the weight's own order; float32
-// [slices, M, N] when K is cut, distie_gemm_packed_wide_slices(N, K) says), bias on the first slice. Rotation and
+// [slices, M, N] when K is cut, distie_gemm_packed_wide_slices(M, N, K) says), bias on the first slice. Rotation and
 // cache write are the caller's next kernel.
 extern "C" int distie_gemm_packed_wide_qkv_bf16(const void* x, const void* w_packed, const float* bias, void* y,
                                                 int y_dtype, int M, int K, int heads, int kv_heads, int dim,
