@@ -516,12 +516,13 @@ extern "C" int distie_gemm_packed_bf16(const void* x, const void* w_packed, cons
 // Epilogues as in gemm_packed_kernel, for every block of 16 rows of x.
 //
 //
-// WAVES is two for up to 32 rows of x in all, else four. What streams the weights fastest here is many small
+// WAVES is two for the gated product of up to 32 rows of x in all, else four. What streams the weights fastest here is many small
 // workgroups, spread evenly over the compute units (the same loop with x left out, gate+up of the 1.5B shape,
 // 55 MB: 13.0 us with one wave a workgroup, 13.7 with two, 15.8 with four, of which there are 280 for 256 compute
 // units); but a smaller workgroup reads x more often. At 32 rows two waves are best (15.8 us against 18.3 with
 // four and 17.2 with one; the decode step at batch 24 and 32 is 6 and 5 % faster); from 48 rows on, and with the
-// rows taken in two passes, four are (batch 64: 3 % slower with two, a portion of 200 tokens 8 %).
+// rows taken in two passes, four are (batch 64: 3 % slower with two, a portion of 200 tokens 8 %). The products whose
+// K is cut into slices (more workgroups already) are faster with four at every number of rows.
 // How far ahead the loads run matters little beside that (four, six or eight k-steps: the same time), as long as
 // the wave never waits for all of them at once.
 template <int MB, int WAVES>
@@ -690,25 +691,23 @@ __global__ __launch_bounds__(64 * WD_WAVES) void gemm_packed_wide_kernel(const b
   }
 }
 
-// Slices of K for the wide kernel: enough waves for the chip, slices of whole k-steps, at least two k-steps long.
-// With workgroups of four waves (more than 32 rows of x) five hundred waves and more: with a thousand the 7B shape's
-// down, o and q/k/v products at 48 and 64 rows were 4-10 % slower, the 1.5B shape's the same. With workgroups of two
-// waves (up to 32 rows) a thousand: with five hundred the 32B shape's step at 32 rows was 3 % slower.
-static void wide_plan(int row_blocks, int K, int M, int* slices, int* tiles_per_slice) {
+// Slices of K for the wide kernel (the products that are cut run in workgroups of four waves): enough waves for the
+// chip, five hundred and more (with a thousand the 7B shape's down, o and q/k/v products at 48 and 64 rows were 4-10 %
+// slower, the 1.5B shape's the same), slices of whole k-steps, at least two k-steps long.
+static void wide_plan(int row_blocks, int K, int* slices, int* tiles_per_slice) {
   constexpr int WD_WAVES = 4;
   const int groups = (row_blocks + WD_WAVES - 1) / WD_WAVES;
   const int steps = (K + SK_KSTEP - 1) / SK_KSTEP;
-  const int enough = M <= 32 ? 1024 : 512;
   int want = 1;
-  while (want < 64 && groups * want * WD_WAVES < enough && steps / (want * 2) >= 2) want *= 2;
+  while (want < 64 && groups * want * WD_WAVES < 512 && steps / (want * 2) >= 2) want *= 2;
   int per = (steps + want - 1) / want;
   *tiles_per_slice = 4 * per;
   *slices = (steps + per - 1) / per;
 }
 
-extern "C" int distie_gemm_packed_wide_slices(int M, int N, int K) {
+extern "C" int distie_gemm_packed_wide_slices(int N, int K) {
   int slices, per;
-  wide_plan((N + 15) / 16, K, M, &slices, &per);
+  wide_plan((N + 15) / 16, K, &slices, &per);
   return slices;
 }
 
@@ -718,7 +717,7 @@ static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bia
                               int K, int mode, int pass_blocks, hipStream_t stream, HeadRows head_rows = HeadRows{0, 0, 0}) {
   const int row_blocks = mode == PK_GATED ? (N / 2 + 7) / 8 : (N + 15) / 16;
   int slices = 1, tiles_per_slice = 4 * ((K + SK_KSTEP - 1) / SK_KSTEP);
-  if (mode != PK_GATED) wide_plan(row_blocks, K, M, &slices, &tiles_per_slice);
+  if (mode != PK_GATED) wide_plan(row_blocks, K, &slices, &tiles_per_slice);
   if (slices > 1 && y_dtype != DISTIE_F32) return DISTIE_BAD_ARGUMENT;
   // pass_blocks: the rows of x are taken in passes of 16 * pass_blocks rows over the weight (0: all at once),
   // with more workgroups and fewer registers and less LDS each; worth it if the weight fits the memory-side
@@ -727,14 +726,20 @@ static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bia
   const int m_group = (pass_blocks >= 1 && pass_blocks <= 4) ? 16 * pass_blocks : 64;
   const int groups = (M + m_group - 1) / m_group;
   const int mb = (std::min(M, m_group) + 15) / 16;
-  const int waves = M <= 32 ? 2 : 4;
+  // two waves a workgroup for the gated product of up to 32 rows; the products whose K is cut are faster with four
+  // at every number of rows (at 32 rows: the 7B shape's o + down 42.5 -> 36.2 us, its head 239 -> 220, the 1.5B shape's
+  // down 9.7 -> 9.1, its head 107 -> 96; gate+up 15.6 with two against 17.1 at the 1.5B shape, 57.3 and 57.4 at the 7B)
+  const int waves = (mode == PK_GATED && M <= 32) ? 2 : 4;
   dim3 grid((row_blocks + waves - 1) / waves, slices, groups);
 #define WIDE(MODE, MB, WAVES)                                                                                   \
   DISTIE_DISPATCH(y_dtype, Y, (gemm_packed_wide_kernel<Y, MODE, MB, WAVES><<<grid, 64 * WAVES, 0, stream>>>(    \
                                   x, w, bias, static_cast<Y*>(y), M, N, K, row_blocks, tiles_per_slice, m_group, head_rows)))
 #define WIDE_MB(MODE)                                   \
   switch (mb) {                                         \
-    case 1: WIDE(MODE, 1, 2); break;                    \
+    case 1:                                             \
+      if (waves == 2) WIDE(MODE, 1, 2);                 \
+      else WIDE(MODE, 1, 4);                            \
+      break;                                            \
     case 2:                                             \
       if (waves == 2) WIDE(MODE, 2, 2);                 \
       else WIDE(MODE, 2, 4);                            \
@@ -765,7 +770,7 @@ extern "C" int distie_gemm_packed_wide_bf16(const void* x, const void* w_packed,
 
 // The stacked q/k/v product alone, on the ROTARY copy of its weight, for 17 rows of x and more against a weight large
 // enough for the wide kernel: y as distie_gemm_packed_wide_bf16 writes it (columns in the weight's own order; float32
-// [slices, M, N] when K is cut, distie_gemm_packed_wide_slices(M, N, K) says), bias on the first slice. Rotation and
+// [slices, M, N] when K is cut, distie_gemm_packed_wide_slices(N, K) says), bias on the first slice. Rotation and
 // cache write are the caller's next kernel.
 extern "C" int distie_gemm_packed_wide_qkv_bf16(const void* x, const void* w_packed, const float* bias, void* y,
                                                 int y_dtype, int M, int K, int heads, int kv_heads, int dim,

@@ -247,7 +247,7 @@ class HipOps(Ops):
         o.distie_pack_rows.argtypes = [_P, _P, _P, _I, _I, _P]
         o.distie_gemm_packed_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
         o.distie_gemm_packed_wide_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
-        o.distie_gemm_packed_wide_slices.argtypes = [_I, _I, _I]
+        o.distie_gemm_packed_wide_slices.argtypes = [_I, _I]
         o.distie_gemm_packed_wide_qkv_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         o.distie_gemm_packed_rotary_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         o.distie_decode_norm_fits.argtypes = [_I]
@@ -566,7 +566,7 @@ class HipOps(Ops):
             # more than one group of 16 rows against a weight that fills the chip through the wide kernel: the
             # epilogue kernel would read the weight once per group, so the product runs wide (weights once, K in
             # slices) and the rotation with the cache write behind it adds the slices
-            slices = self._ops.distie_gemm_packed_wide_slices(M, N, K)
+            slices = self._ops.distie_gemm_packed_wide_slices(N, K)
             shape, dtype = ((M, N), torch.bfloat16) if slices == 1 else ((slices, M, N), torch.float32)
             product = torch.empty(shape, dtype=dtype, device=self.device)
             _check(self._ops.distie_gemm_packed_wide_qkv_bf16(
@@ -711,7 +711,7 @@ class HipOps(Ops):
                 N * K > self.ROW_GROUPS_MAX_ELEMENTS:
             if packed.numel() != self._packed_elements(N, K, False):
                 raise KernelError("linear: the packed copy does not belong to this weight")
-            slices = self._ops.distie_gemm_packed_wide_slices(M, N, K)
+            slices = self._ops.distie_gemm_packed_wide_slices(N, K)
             if slices == 1:
                 out = torch.empty((M, N), dtype=out_dtype, device=self.device)
             else:
