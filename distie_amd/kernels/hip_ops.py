@@ -147,10 +147,15 @@ class HipOps(Ops):
     # LDS, in passes of at most 64: up to PACKED_MAX_ROWS in a captured step (measured in the decode step: 9 %
     # faster than the library at 72 rows, 5 % at 96, 4 % slower at 128), and up to PACKED_MAX_ROWS_EAGER in a step
     # that is launched kernel by kernel, which the host bounds at these sizes: the library's products cost it
-    # 18 us each and the activation and rotation kernels beside them more launches (a prompt of 128 tokens:
-    # 2.7 instead of 3.9 ms, of 192: 3.3, of 224: 3.8, of 256: 4.1 instead of 3.9 ms),
+    # 18 us each and the activation and rotation kernels beside them more launches. A portion of n tokens behind
+    # 512, this way and through the library: 1.5B shape 100: 2.8 and 3.4 ms, 160: 3.1 and 3.4, 200: 3.6 and 3.5,
+    # 224: 3.7 and 3.5; 7B shape (weights that are read from memory again in every pass of 64 rows) 100: 6.3 and
+    # 7.2, 128: 6.6 and 7.4, 160: 8.3 and 8.0, 200: 10.1 and 8.9. So up to 192 rows, and up to 128 against a weight
+    # too large for the memory-side cache to hold between passes (more than PACKED_LARGE_ELEMENTS: 64 MB).
     PACKED_MAX_ROWS = 96
-    PACKED_MAX_ROWS_EAGER = 224
+    PACKED_MAX_ROWS_EAGER = 192
+    PACKED_MAX_ROWS_EAGER_LARGE = 128
+    PACKED_LARGE_ELEMENTS = 32 << 20
     # or, for a weight of at most this many elements (too few row blocks to occupy the chip that way),
     # through the one-wave kernel once per 16 rows of x
     ROW_GROUPS_MAX_ELEMENTS = 4 << 20
@@ -498,7 +503,7 @@ class HipOps(Ops):
             out = torch.empty((x.shape[0], N // 2), dtype=torch.bfloat16, device=self.device)
             return self._norm_product(x, packed, None, out, 1, N)
         x = self.dense(x)
-        if packed is None or x.dtype != torch.bfloat16 or x.shape[0] > self._packed_rows():
+        if packed is None or x.dtype != torch.bfloat16 or x.shape[0] > self._packed_rows(gate_up_weight.numel()):
             return self.silu_mul(self.linear(x, gate_up_weight))
         self._own(x)
         M, K = x.shape
@@ -543,7 +548,7 @@ class HipOps(Ops):
                 table, slots, k_cache, v_cache, num_heads, num_kv_heads, head_dim, meta.block_size, 1 if write else 0))
         x = self.dense(x)
         fused = held is not None and held[1] == (num_heads, num_kv_heads, head_dim) and \
-            x.dtype == torch.bfloat16 and x.shape[0] <= self._packed_rows() and \
+            x.dtype == torch.bfloat16 and x.shape[0] <= self._packed_rows(weight.numel()) and \
             inv_freq is not None and 2 * inv_freq.shape[0] == head_dim and k_cache.dtype == torch.bfloat16
         if not fused:
             return self.rope_kv_write(self.linear(x, weight, bias), meta, group, k_cache, v_cache, inv_freq,
@@ -585,8 +590,11 @@ class HipOps(Ops):
             num_kv_heads, head_dim, meta.block_size, 1 if write else 0, self._stream()), "gemm_packed_rotary_bf16")
         return out
 
-    def _packed_rows(self) -> int:
-        return self.PACKED_MAX_ROWS if self.captured else self.PACKED_MAX_ROWS_EAGER
+    def _packed_rows(self, elements: int) -> int:
+        """Most rows of x that go through the kernels on the packed copy of a weight of `elements`."""
+        if self.captured:
+            return self.PACKED_MAX_ROWS
+        return self.PACKED_MAX_ROWS_EAGER if elements <= self.PACKED_LARGE_ELEMENTS else self.PACKED_MAX_ROWS_EAGER_LARGE
 
     def _library(self):
         """The vendor library's products, called directly; loaded at the first large product."""
@@ -707,7 +715,7 @@ class HipOps(Ops):
         packed = packed if both_bf16 else None
         if lazy and packed is not None and self._fused(M) and K % 8 == 0 and out_dtype == torch.bfloat16:
             return PendingProduct(x, weight, bias)
-        if packed is not None and self.SKINNY_MAX_ROWS < M <= self._packed_rows() and K % 8 == 0 and \
+        if packed is not None and self.SKINNY_MAX_ROWS < M <= self._packed_rows(N * K) and K % 8 == 0 and \
                 N * K > self.ROW_GROUPS_MAX_ELEMENTS:
             if packed.numel() != self._packed_elements(N, K, False):
                 raise KernelError("linear: the packed copy does not belong to this weight")
@@ -723,7 +731,7 @@ class HipOps(Ops):
             if slices == 1:
                 return out
             return PartialSums(out, out_dtype) if partial_ok else self.dense(PartialSums(out, out_dtype))
-        if both_bf16 and K % 8 == 0 and (M <= self.SKINNY_MAX_ROWS or (packed is not None and M <= self._packed_rows())):
+        if both_bf16 and K % 8 == 0 and (M <= self.SKINNY_MAX_ROWS or (packed is not None and M <= self._packed_rows(N * K))):
             if packed is not None:
                 if packed.numel() != self._packed_elements(N, K, False):
                     raise KernelError("linear: the packed copy does not belong to this weight")

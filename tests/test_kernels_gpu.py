@@ -143,7 +143,7 @@ def test_gemm_skinny_bf16(ops, M, N, K):
     close(got, want + b.double(), torch.bfloat16, scale=want.abs().max().item())
 
 
-@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 50, 64, 65, 96, 130, 224])
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 50, 64, 65, 96, 130, 192])
 @pytest.mark.parametrize("N,K", [(48, 128), (100, 264), (1536, 1536), (333, 8960), (2050, 72), (16, 8), (7, 40)])
 def test_gemm_packed_bf16(ops, M, N, K):
     """The same products through the weight's packed copy (what `prepare_linear` leaves): rows and
@@ -182,7 +182,7 @@ def test_gemm_packed_bf16(ops, M, N, K):
 
 
 def test_fewer_rows_through_the_packed_kernels_in_a_captured_step(ops):
-    """Launched kernel by kernel, a step of up to 224 tokens is bound by the host and takes the packed
+    """Launched kernel by kernel, a step of up to 192 tokens is bound by the host and takes the packed
     kernels with their fused epilogues; in a captured step only up to 96 rows do, the library's products
     being faster on the device beyond."""
     from distie_amd.kernels.hip_ops import PartialSums
@@ -202,6 +202,17 @@ def test_fewer_rows_through_the_packed_kernels_in_a_captured_step(ops):
     assert not isinstance(captured, PartialSums)
     close(ops.dense(eager), want, torch.bfloat16, scale=want.abs().max().item())
     close(captured, want, torch.bfloat16, scale=want.abs().max().item())
+    # against a weight too large for the memory-side cache to hold between the passes, only up to 128 rows
+    more = rand(150, 1536, dtype=torch.bfloat16, seed=3)
+    assert isinstance(ops.linear(more, w), PartialSums)
+    ops.PACKED_LARGE_ELEMENTS = 0                   # every weight counts as large
+    try:
+        assert isinstance(ops.linear(x, w), PartialSums)
+        through_library = ops.linear(more, w)
+        assert not isinstance(through_library, PartialSums)
+    finally:
+        del ops.PACKED_LARGE_ELEMENTS
+    close(through_library, more.double() @ w.double().T, torch.bfloat16, scale=want.abs().max().item())
 
 
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 40, 64, 81, 96, 150, 192])
