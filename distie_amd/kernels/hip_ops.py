@@ -152,7 +152,11 @@ class HipOps(Ops):
     # 224: 3.7 and 3.5; 7B shape (weights that are read from memory again in every pass of 64 rows) 100: 6.3 and
     # 7.2, 128: 6.6 and 7.4, 160: 8.3 and 8.0, 200: 10.1 and 8.9. So up to 192 rows, and up to 128 against a weight
     # too large for the memory-side cache to hold between passes (more than PACKED_LARGE_ELEMENTS: 64 MB).
+    # In a captured step a large weight keeps the packed kernels up to 128 rows: the 7B shape's decode step at batch
+    # 112 takes 9.2 ms this way and 11.3 with the library's (untimed) choice of kernel, at batch 128 9.7 and 12.2, at
+    # batch 160 13.1 and 12.5; the 1.5B shape's step is the same either way (its weights are small, its head large).
     PACKED_MAX_ROWS = 96
+    PACKED_MAX_ROWS_LARGE = 128
     PACKED_MAX_ROWS_EAGER = 192
     PACKED_MAX_ROWS_EAGER_LARGE = 128
     PACKED_LARGE_ELEMENTS = 32 << 20
@@ -593,7 +597,7 @@ class HipOps(Ops):
     def _packed_rows(self, elements: int) -> int:
         """Most rows of x that go through the kernels on the packed copy of a weight of `elements`."""
         if self.captured:
-            return self.PACKED_MAX_ROWS
+            return self.PACKED_MAX_ROWS if elements <= self.PACKED_LARGE_ELEMENTS else self.PACKED_MAX_ROWS_LARGE
         return self.PACKED_MAX_ROWS_EAGER if elements <= self.PACKED_LARGE_ELEMENTS else self.PACKED_MAX_ROWS_EAGER_LARGE
 
     def _library(self):

@@ -210,6 +210,11 @@ def test_fewer_rows_through_the_packed_kernels_in_a_captured_step(ops):
         assert isinstance(ops.linear(x, w), PartialSums)
         through_library = ops.linear(more, w)
         assert not isinstance(through_library, PartialSums)
+        ops.captured = True                         # ... and in a captured step a large weight keeps them up to 128 rows
+        try:
+            assert isinstance(ops.linear(x, w), PartialSums) and not isinstance(ops.linear(more, w), PartialSums)
+        finally:
+            ops.captured = False
     finally:
         del ops.PACKED_LARGE_ELEMENTS
     close(through_library, more.double() @ w.double().T, torch.bfloat16, scale=want.abs().max().item())
