@@ -143,6 +143,11 @@ class HipOps(Ops):
     # bfloat16 products by rows of x: up to SKINNY_MAX_ROWS the weights are streamed by one wave per block
     # of 16 weight rows, x straight from memory (above that, the library's tiles are faster);
     SKINNY_MAX_ROWS = 16
+    # on a packed copy the one-wave kernel is the faster one only up to 8 rows: at 9 to 16 rows every wave reads all
+    # 16 rows of x beside its weights, and the kernel that shares x through LDS takes over (decode step at batch 12
+    # and 16: 1.5B shape 1.77 -> 1.66 and 1.95 -> 1.81 ms, 7B shape 4.34 -> 3.91 and 4.92 -> 4.14 ms; at batch 8 and
+    # below the one-wave kernel is level or ahead)
+    ONE_WAVE_MAX_ROWS = 8
     # with a packed copy of the weight, more rows go through the kernel that shares the x tile of a workgroup in
     # LDS, in passes of at most 64: up to PACKED_MAX_ROWS in a captured step (measured in the decode step: 9 %
     # faster than the library at 72 rows, 5 % at 96, 4 % slower at 128), and up to PACKED_MAX_ROWS_EAGER in a step
@@ -517,7 +522,7 @@ class HipOps(Ops):
         if packed.numel() != self._packed_elements(N, K, True):
             raise KernelError("linear_silu_mul: the packed copy does not belong to this weight")
         out = torch.empty((M, N // 2), dtype=x.dtype, device=self.device)
-        if M <= self.SKINNY_MAX_ROWS:
+        if M <= self.ONE_WAVE_MAX_ROWS:
             _check(self._ops.distie_gemm_packed_bf16(x.data_ptr(), packed.data_ptr(), None, out.data_ptr(), _code(out),
                                                      M, N, K, 1, self._stream()), "gemm_packed_bf16")
         else:
@@ -719,7 +724,7 @@ class HipOps(Ops):
         packed = packed if both_bf16 else None
         if lazy and packed is not None and self._fused(M) and K % 8 == 0 and out_dtype == torch.bfloat16:
             return PendingProduct(x, weight, bias)
-        if packed is not None and self.SKINNY_MAX_ROWS < M <= self._packed_rows(N * K) and K % 8 == 0 and \
+        if packed is not None and self.ONE_WAVE_MAX_ROWS < M <= self._packed_rows(N * K) and K % 8 == 0 and \
                 N * K > self.ROW_GROUPS_MAX_ELEMENTS:
             if packed.numel() != self._packed_elements(N, K, False):
                 raise KernelError("linear: the packed copy does not belong to this weight")
