@@ -7,7 +7,7 @@
 //    (v_mfma_f32_16x16x32_bf16): a wave owns 16 rows of W and a slice of K, reads W straight from
 //    memory into the A operand (every weight byte is read once), and the small x is the B operand.
 //    Slices of K are written side by side and added, in order, by the kernel that reads them.
-//  * pack_rows + gemm_packed (up to 16 rows of x) and gemm_packed_wide (17 to 64 rows a pass): the same streaming on a
+//  * pack_rows + gemm_packed (up to 16 rows of x a group) and gemm_packed_wide (up to 64 rows a pass): the same streaming on a
 //    second copy of W laid out tile by tile in the matrix cores' lane order, with epilogues that finish
 //    what follows the product (gated activation; bias, rotation and cache write of q/k/v). Described at
 //    their definitions.
