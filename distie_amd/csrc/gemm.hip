@@ -7,7 +7,7 @@
 //    (v_mfma_f32_16x16x32_bf16): a wave owns 16 rows of W and a slice of K, reads W straight from
 //    memory into the A operand (every weight byte is read once), and the small x is the B operand.
 //    Slices of K are written side by side and added, in order, by the kernel that reads them.
-//  * pack_rows + gemm_packed (up to 16 rows of x a group) and gemm_packed_wide (up to 64 rows a pass): the same streaming on a
+//  * pack_rows + gemm_packed (up to 16 rows of x a group) and gemm_packed_wide (up to 96 rows a pass): the same streaming on a
 //    second copy of W laid out tile by tile in the matrix cores' lane order, with epilogues that finish
 //    what follows the product (gated activation; bias, rotation and cache write of q/k/v). Described at
 //    their definitions.
@@ -519,7 +519,7 @@ extern "C" int distie_gemm_packed_bf16(const void* x, const void* w_packed, cons
   return launch_status();
 }
 
-// ---------------------------------------------------------------- packed weights, 17 to 64 rows of x a pass
+// ---------------------------------------------------------------- packed weights, up to 96 rows of x a pass
 // A workgroup of WAVES waves owns as many row blocks (one a wave) and one slice of K. Per k-step of 128 the
 // weights go straight into registers, some k-steps ahead; the x tile ([16 MB rows, 128 k], the same for
 // all waves) is fetched as far ahead, into registers, and put into LDS (two stages) right before it is used,
@@ -541,6 +541,11 @@ constexpr int wd_stages() { return WAVES == 2 && MB == 1 ? 8 : 4; }    // (k-ste
 // elements of an x row in LDS: a stride of 32 bytes more than a multiple of 64 keeps the reads (lane (r, g):
 // row r, byte 16 g) free of bank conflicts; with 16 bytes more every read costs twice (measured)
 constexpr int WD_XROW = SK_KSTEP + 16;
+// blocks of 16 rows of x a pass at most: with seven and eight the registers (x is fetched as far ahead as the weights)
+// leave one wave a SIMD, and eight waves a workgroup spill or gain nothing (7B shape, decode step at batch 128: one
+// pass of 8 blocks 11.4 ms with four waves, 9.7 with eight, as two passes of 4; at batch 80 and 96 one pass of 5 and
+// 6 blocks takes 6.8 and 8.1 ms against 7.7 and 8.3 in two passes, the weights coming from memory once)
+constexpr int WD_MAX_BLOCKS = 6;
 
 // MODE PK_ROTARY here: the weight is the ROTARY copy of a stacked q/k/v weight (rotation partners in one block), the
 // result is the plain product, every sum written to the column its row of W has: the rotation needs the whole
@@ -579,7 +584,7 @@ __global__ __launch_bounds__(64 * WD_WAVES) void gemm_packed_wide_kernel(const b
   // this thread's part of an x tile: rows XROWS p + tid / 16 (p < XP), k 8 (tid % 16) .. + 7 of the step
   const int x_row = tid / 16;
   const int x_chunk = tid % 16;
-  constexpr int XP = MB * 4 / WD_WAVES;                          // pieces of an x tile a thread carries
+  constexpr int XP = (MB * 4 + WD_WAVES - 1) / WD_WAVES;         // pieces of an x tile a thread carries
   constexpr int XROWS = 4 * WD_WAVES;                           // rows of the tile the threads cover at once
   const bf16_t* xsrc[XP];
 #pragma unroll
@@ -624,7 +629,8 @@ __global__ __launch_bounds__(64 * WD_WAVES) void gemm_packed_wide_kernel(const b
 #pragma unroll
     for (int p = 0; p < XP; ++p) {
       const uint4 v = xr[slot][p];
-      *reinterpret_cast<uint4*>(&xs[stage][XROWS * p + x_row][8 * x_chunk]) = uint4{v.x & keep, v.y & keep, v.z & keep, v.w & keep};
+      if (XROWS * (p + 1) <= MB * 16 || XROWS * p + x_row < MB * 16)       // (the last piece may reach past the tile)
+        *reinterpret_cast<uint4*>(&xs[stage][XROWS * p + x_row][8 * x_chunk]) = uint4{v.x & keep, v.y & keep, v.z & keep, v.w & keep};
     }
     __syncthreads();
 #pragma unroll
@@ -722,7 +728,7 @@ extern "C" int distie_gemm_packed_wide_slices(int N, int K) {
   return slices;
 }
 
-// 17 to 256 rows of x, at most 64 a pass. mode 0: y [M, N] of y_dtype, or float32 [slices, M, N] when the plan cuts K
+// Up to 256 rows of x, at most 96 a pass. mode 0: y [M, N] of y_dtype, or float32 [slices, M, N] when the plan cuts K
 // (distie_gemm_packed_wide_slices); 1 (gated): [M, N / 2].
 static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bias, void* y, int y_dtype, int M, int N,
                               int K, int mode, int pass_blocks, hipStream_t stream, HeadRows head_rows = HeadRows{0, 0, 0}) {
@@ -730,11 +736,11 @@ static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bia
   int slices = 1, tiles_per_slice = 4 * ((K + SK_KSTEP - 1) / SK_KSTEP);
   if (mode != PK_GATED) wide_plan(row_blocks, K, &slices, &tiles_per_slice);
   if (slices > 1 && y_dtype != DISTIE_F32) return DISTIE_BAD_ARGUMENT;
-  // pass_blocks: the rows of x are taken in passes of 16 * pass_blocks rows over the weight (0: all at once),
+  // pass_blocks: the rows of x are taken in passes of 16 * pass_blocks rows over the weight (0: 64 rows a pass),
   // with more workgroups and fewer registers and less LDS each; worth it if the weight fits the memory-side
   // cache, from which the later passes then read it (measured at 64 rows in two passes, cold: down 18.3 ->
   // 15.4 us, gate+up 22.4 -> 21.3 us; a weight of 270 MB gets slower, being fetched from memory twice).
-  const int m_group = (pass_blocks >= 1 && pass_blocks <= 4) ? 16 * pass_blocks : 64;
+  const int m_group = (pass_blocks >= 1 && pass_blocks <= WD_MAX_BLOCKS) ? 16 * pass_blocks : 64;
   const int groups = (M + m_group - 1) / m_group;
   const int mb = (std::min(M, m_group) + 15) / 16;
   // two waves a workgroup for the gated product of up to 32 rows; the products whose K is cut are faster with four
@@ -756,7 +762,9 @@ static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bia
       else WIDE(MODE, 2, 4);                            \
       break;                                            \
     case 3: WIDE(MODE, 3, 4); break;                    \
-    default: WIDE(MODE, 4, 4); break;                   \
+    case 4: WIDE(MODE, 4, 4); break;                    \
+    case 5: WIDE(MODE, 5, 4); break;                    \
+    default: WIDE(MODE, 6, 4); break;                   \
   }
   if (mode == PK_GATED) {
     WIDE_MB(PK_GATED);

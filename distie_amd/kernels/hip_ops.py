@@ -149,21 +149,21 @@ class HipOps(Ops):
     # below the one-wave kernel is level or ahead)
     ONE_WAVE_MAX_ROWS = 8
     # with a packed copy of the weight, more rows go through the kernel that shares the x tile of a workgroup in
-    # LDS, in passes of at most 64: up to PACKED_MAX_ROWS in a captured step (measured in the decode step: 9 %
+    # LDS, in passes over the weight: up to PACKED_MAX_ROWS in a captured step (measured in the decode step: 9 %
     # faster than the library at 72 rows, 5 % at 96, 4 % slower at 128), and up to PACKED_MAX_ROWS_EAGER in a step
     # that is launched kernel by kernel, which the host bounds at these sizes: the library's products cost it
-    # 18 us each and the activation and rotation kernels beside them more launches. A portion of n tokens behind
-    # 512, this way and through the library: 1.5B shape 100: 2.8 and 3.4 ms, 160: 3.1 and 3.4, 200: 3.6 and 3.5,
-    # 224: 3.7 and 3.5; 7B shape (weights that are read from memory again in every pass of 64 rows) 100: 6.3 and
-    # 7.2, 128: 6.6 and 7.4, 160: 8.3 and 8.0, 200: 10.1 and 8.9. So up to 192 rows, and up to 128 against a weight
-    # too large for the memory-side cache to hold between passes (more than PACKED_LARGE_ELEMENTS: 64 MB).
-    # In a captured step a large weight keeps the packed kernels up to 128 rows: the 7B shape's decode step at batch
-    # 112 takes 9.2 ms this way and 11.3 with the library's (untimed) choice of kernel, at batch 128 9.7 and 12.2, at
-    # batch 160 13.1 and 12.5; the 1.5B shape's step is the same either way (its weights are small, its head large).
+    # 18 us each and the activation and rotation kernels beside them more launches (a portion of n tokens behind
+    # 512, this way and through the library, 1.5B shape: 100: 2.8 and 3.4 ms, 160: 3.1 and 3.4, 200: 3.6 and 3.5,
+    # 224: 3.7 and 3.5).
+    # A weight of more than PACKED_LARGE_ELEMENTS (64 MB: the memory-side cache does not hold it from one pass to
+    # the next) keeps the packed kernels up to PACKED_MAX_ROWS_LARGE in a captured step too. Its passes are of up
+    # to 96 rows, so 192 rows read it twice. 7B shape, this way and with the library's (untimed) choice of kernel:
+    # decode step at batch 112: 9.2 and 11.3 ms, 128: 9.7 and 12.2, 144: 11.5 and 13.6, 160: 11.9 and 14.4, 192: 13.3
+    # and 13.3; a portion of n tokens behind 512: 144: 7.1 and 9.4 ms, 160: 7.4 and 10.1, 192: 8.3 and 10.8.
+    # The 1.5B shape's captured step is the same either way (its weights are small, its head large).
     PACKED_MAX_ROWS = 96
-    PACKED_MAX_ROWS_LARGE = 128
+    PACKED_MAX_ROWS_LARGE = 192
     PACKED_MAX_ROWS_EAGER = 192
-    PACKED_MAX_ROWS_EAGER_LARGE = 128
     PACKED_LARGE_ELEMENTS = 32 << 20
     # or, for a weight of at most this many elements (too few row blocks to occupy the chip that way),
     # through the one-wave kernel once per 16 rows of x
@@ -175,6 +175,10 @@ class HipOps(Ops):
     # ... and that kernel takes more than 32 rows in two passes of 32 over a weight of at most this many elements
     # (64 MB: the second pass reads it from the memory-side cache; much larger ones would come from memory twice)
     TWO_PASS_MAX_ELEMENTS = 32 << 20
+    # ... and a larger one is read once per pass: as few passes as the kernel's 96 rows a pass allow, of equal size
+    # (7B shape: decode step at batch 80 6.8 ms in one pass of 80 rows, 7.7 as 64 + 16; at batch 96 8.1 and 8.3;
+    # a portion of 160 tokens 7.4 ms in two passes of 80 and 8.4 in three of 64, 64 and 32)
+    WIDE_PASS_MAX_BLOCKS = 6
     # attention over a portion of a prompt: from so many visible keys on, the walk over the keys is cut into so
     # many parts that run side by side (measured at 12 heads of 128, 2,048 new tokens: 3 parts are best up to
     # 4,096 keys, 5 at 8,192, 8 from 16,384 on; the kernel takes up to 16)
@@ -603,7 +607,7 @@ class HipOps(Ops):
         """Most rows of x that go through the kernels on the packed copy of a weight of `elements`."""
         if self.captured:
             return self.PACKED_MAX_ROWS if elements <= self.PACKED_LARGE_ELEMENTS else self.PACKED_MAX_ROWS_LARGE
-        return self.PACKED_MAX_ROWS_EAGER if elements <= self.PACKED_LARGE_ELEMENTS else self.PACKED_MAX_ROWS_EAGER_LARGE
+        return self.PACKED_MAX_ROWS_EAGER
 
     def _library(self):
         """The vendor library's products, called directly; loaded at the first large product."""
@@ -685,7 +689,11 @@ class HipOps(Ops):
     def _pass_blocks(self, rows: int, elements: int) -> int:
         """Blocks of 16 rows of x per pass of the wide product over a weight of `elements` (0: one pass)."""
         if elements > self.TWO_PASS_MAX_ELEMENTS:
-            return 0 if rows <= 64 else 4
+            if rows <= 64:
+                return 0
+            blocks = -(-rows // 16)
+            passes = -(-blocks // self.WIDE_PASS_MAX_BLOCKS)
+            return -(-blocks // passes)
         # (a single pass takes at most 64 rows; beyond 128 rows passes of 48 were 5 % faster than of 32 or 64)
         return 0 if rows <= 32 else (2 if rows <= 128 else 3)
 

@@ -202,22 +202,19 @@ def test_fewer_rows_through_the_packed_kernels_in_a_captured_step(ops):
     assert not isinstance(captured, PartialSums)
     close(ops.dense(eager), want, torch.bfloat16, scale=want.abs().max().item())
     close(captured, want, torch.bfloat16, scale=want.abs().max().item())
-    # against a weight too large for the memory-side cache to hold between the passes, only up to 128 rows
+    # a weight too large for the memory-side cache to hold between the passes keeps them in a captured step too
     more = rand(150, 1536, dtype=torch.bfloat16, seed=3)
     assert isinstance(ops.linear(more, w), PartialSums)
     ops.PACKED_LARGE_ELEMENTS = 0                   # every weight counts as large
+    ops.captured = True
     try:
-        assert isinstance(ops.linear(x, w), PartialSums)
-        through_library = ops.linear(more, w)
-        assert not isinstance(through_library, PartialSums)
-        ops.captured = True                         # ... and in a captured step a large weight keeps them up to 128 rows
-        try:
-            assert isinstance(ops.linear(x, w), PartialSums) and not isinstance(ops.linear(more, w), PartialSums)
-        finally:
-            ops.captured = False
+        large = ops.linear(more, w)
+        assert isinstance(large, PartialSums)
+        assert not isinstance(ops.linear(rand(200, 1536, dtype=torch.bfloat16, seed=4), w), PartialSums)
     finally:
+        ops.captured = False
         del ops.PACKED_LARGE_ELEMENTS
-    close(through_library, more.double() @ w.double().T, torch.bfloat16, scale=want.abs().max().item())
+    close(ops.dense(large), more.double() @ w.double().T, torch.bfloat16, scale=want.abs().max().item())
 
 
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 40, 64, 81, 96, 150, 192])
