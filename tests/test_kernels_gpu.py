@@ -292,6 +292,17 @@ def test_linear_rope_kv_write_fused(ops, M, heads, kv_heads, dim, K, P, with_bia
         at = torch.tensor(slots).cuda()
         assert torch.equal(k1[at // P, :, at % P], view[:, heads:heads + kv_heads])
         assert torch.equal(v1[at // P, :, :, at % P], view[:, heads + kv_heads:])
+    if M > 64 and N * K > ops.ROW_GROUPS_MAX_ELEMENTS:
+        # a weight that the memory-side cache cannot hold between passes is taken in passes of up to 96 rows
+        k4, v4 = k2.clone(), v2.clone()
+        if write:
+            k4[at // P, :, at % P] = 0
+        ops.TWO_PASS_MAX_ELEMENTS = 0
+        try:
+            again = ops.linear_rope_kv_write(x, w, b, meta, 0, k4, v4, inv_freq, heads, kv_heads, dim, write)
+        finally:
+            del ops.TWO_PASS_MAX_ELEMENTS
+        assert torch.equal(again, got) and torch.equal(k4, k1) and torch.equal(v4, v1)
     # unfused (no packed copy), the same within rounding
     w2 = w.clone()
     k3, v3 = k2.clone(), v2.clone()
