@@ -47,7 +47,8 @@ def _engine_options(parser: argparse.ArgumentParser) -> None:
     parser.add_argument("--gpu-mem-fraction", type=float, default=None,
                         help="without --num-blocks: pages of the cache until this share of the card's memory is in use")
     parser.add_argument("--tune-products", action="store_true",
-                        help="at start, let the library time its kernels for the products of a full portion")
+                        help="at start, let the library time its kernels for the products of a full portion and of 65 to 192 rows "
+                             "(more with a larger --max-seqs)")
 
 
 def _build(args):

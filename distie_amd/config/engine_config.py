@@ -57,7 +57,7 @@ class EngineConfig:
     # decoder name "qkv", "attn_out", "gate_up", "down" and "head", another part may name others
     packed_weights: Union[bool, Tuple[str, ...]] = True
     lookahead: bool = True                  # launch the next decode step before this step's tokens reach the host
-    tune_products: bool = False             # at start, let the library time its kernels for a full portion's products
+    tune_products: bool = False             # at start, let the library time its kernels for the products of a full portion and of large batches
     step_stats: int = 0
     seed: int = 0
 

@@ -64,10 +64,12 @@ hipblasLtHandle_t handle = nullptr;
 void* workspace = nullptr;
 int device_of_handle = -1;
 std::unordered_map<Key, Plan, KeyHash> plans;
-// the library's first choice for a class of row counts (the key's M rounded up to ROW_CLASS): a serving run meets
-// a new row count in almost every step with a portion in it, and asking the library to rank its kernels costs
-// more than the product of a short portion
+// the choice for a class of row counts (the key's M rounded up to ROW_CLASS): the library's first, or the kernel
+// found by timing if a shape of the class was timed (the engine times the class's largest row count). A serving
+// run meets a new row count in almost every step with a portion in it, and asking the library to rank its
+// kernels costs more than the product of a short portion
 std::unordered_map<Key, hipblasLtMatmulAlgo_t, KeyHash> class_choice;
+std::unordered_map<Key, bool, KeyHash> class_timed;
 long plans_made = 0, plans_timed = 0, choices_asked = 0, candidates_refused = 0;
 
 bool ok(hipblasStatus_t s) { return s == HIPBLAS_STATUS_SUCCESS; }
@@ -338,13 +340,15 @@ extern "C" int distie_lib_linear(const void* x, const void* w, const void* bias,
         return asked;
       }
       plan.algo = found[0].algo;
-      class_choice[of_class] = plan.algo;
+      if (class_timed.find(of_class) == class_timed.end()) class_choice[of_class] = plan.algo;
     }
     if (tune) {
       const int chosen = choose_by_timing(plan, key, found, x, w, bias, y, stream);
       if (chosen != 0) return chosen;
       plan.timed = true;
       ++plans_timed;
+      class_choice[of_class] = plan.algo;
+      class_timed[of_class] = true;
     }
   }
   const hipblasStatus_t s = run(it->second, it->second.algo, x, w, bias, y, stream);

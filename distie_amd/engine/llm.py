@@ -133,24 +133,47 @@ class LLM:
                   spec.architecture, ec.dtype, self.num_pages, ec.block_size, len(self.cache.groups),
                   self.cache.bytes() / 2 ** 20)
 
+    # row counts whose products are timed beside a full portion's: the largest of each class of 32 rows from 96 on,
+    # up to this many or the largest batch, whichever is more (a class takes about a second)
+    TIMED_ROWS = 192
+    TIMED_ROWS_MOST = 512
+
     def _tune_products(self) -> None:
         """One step with as many tokens as a full portion of a prompt has, while the library is
         allowed to time its candidate kernels for every product shape it meets; afterwards it
-        uses what it found for these shapes and its defaults for all others."""
+        uses what it found for these shapes and its defaults for all others. Then the same for
+        the row counts of large decode batches and short portions, class by class, with the
+        products going where a captured step sends them."""
         tokens = min(self.engine_config.token_budget, self.max_model_len,
                      self.cache.block_size * self.cache.num_blocks)
         if tokens < 1:
             return
         started = time.perf_counter()
+        ids = [i % self.model.spec.vocab_size for i in range(tokens)]
+        most = min(tokens, self.TIMED_ROWS_MOST, max(self.TIMED_ROWS, -(-self.engine_config.max_seqs // 32) * 32))
+        graphs, self.runner.graphs = self.runner.graphs, None        # (timing a kernel cannot be recorded into a graph)
         self.ops.tune_library_products(True)
+        done = False
         try:
-            ids = [i % self.model.spec.vocab_size for i in range(tokens)]
             self.step([StepEntry("__tune__", ids, [tokens - 1])])
+            self.finish("__tune__")
+            # from here on the products of these row counts go where they will go once their kernels are timed
+            self.ops.captured, self.ops.library_timed_rows = True, most
+            for rows in range(96, most + 1, 32):
+                # every row wanted: the head's product has as many rows as a decode step of that batch
+                self.step([StepEntry("__tune__", ids[:rows], list(range(rows)))])
+                self.finish("__tune__")
             torch.cuda.synchronize()
+            done = True
         finally:
+            self.ops.captured = False
+            if not done:
+                self.ops.library_timed_rows = 0
             self.finish("__tune__")
             self.ops.tune_library_products(False)
-        _log.info("library products tuned for portions of %d tokens in %.1f s", tokens, time.perf_counter() - started)
+            self.runner.graphs = graphs
+        _log.info("library products tuned for portions of %d tokens and for 65 to %d rows in %.1f s", tokens, most,
+                  time.perf_counter() - started)
 
     # ------------------------------------------------------------ the step function
     def step(self, entries: Seq[StepEntry]) -> Optional[torch.Tensor]:

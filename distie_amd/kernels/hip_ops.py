@@ -155,14 +155,25 @@ class HipOps(Ops):
     # 18 us each and the activation and rotation kernels beside them more launches (a portion of n tokens behind
     # 512, this way and through the library, 1.5B shape: 100: 2.8 and 3.4 ms, 160: 3.1 and 3.4, 200: 3.6 and 3.5,
     # 224: 3.7 and 3.5).
-    # A weight of more than PACKED_LARGE_ELEMENTS (64 MB: the memory-side cache does not hold it from one pass to
-    # the next) keeps the packed kernels up to PACKED_MAX_ROWS_LARGE in a captured step too. Its passes are of up
-    # to 96 rows, so 192 rows read it twice. 7B shape, this way and with the library's (untimed) choice of kernel:
-    # decode step at batch 112: 9.2 and 11.3 ms, 128: 9.7 and 12.2, 144: 11.5 and 13.6, 160: 11.9 and 14.4, 192: 13.3
-    # and 13.3; a portion of n tokens behind 512: 144: 7.1 and 9.4 ms, 160: 7.4 and 10.1, 192: 8.3 and 10.8.
-    # The 1.5B shape's captured step is the same either way (its weights are small, its head large).
+    # A weight of more than PACKED_LARGE_ELEMENTS (64 MB) is not held by the memory-side cache from one pass to the
+    # next: a pass takes up to 96 rows, and every further one reads the weight from memory again, which the library
+    # does once. Which is faster then goes by the weight's shape (7B shape at 128 rows, the packed kernels in two
+    # passes and the library's best kernel by timing, with the same flush of the caches before each: gate+up
+    # [37888, 3584] 144 and 115 us, the head [152064, 3584] 535 and 297, down [3584, 18944] 75 and 91):
+    #  * K longer than the weight has rows (down): the packed kernels, whose K is cut into slices, up to
+    #    PACKED_MAX_ROWS_LARGE rows, captured or not;
+    #  * more rows than K (gate+up, the head, a large q/k/v): one pass, PACKED_MAX_ROWS_LARGE_WIDE rows. Once the
+    #    library's kernels were timed for a class of row counts (`library_timed_rows`, set by the engine's start with
+    #    `tune_products`), the library takes over from 65 rows on (PACKED_MAX_ROWS_LARGE_WIDE_TIMED): untimed, its
+    #    choice is good at one row count and poor at the next. 7B shape, decode step at batch 72, 80, 96, 112, 128,
+    #    160, 192: 6.4, 6.6, 7.3, 8.1, 8.4, 10.4, 10.9 ms timed; 6.6, 6.8, 8.0, 8.6, 9.6, 11.7, 12.0 untimed; and with
+    #    every large weight on the packed kernels up to 192 rows 6.6, 6.8, 8.0, 9.2, 9.7, 11.9, 13.3. At 24 to 64 rows
+    #    the timed library is 1-3 % ahead as well (gate+up rounded to bfloat16 before the activation): left as it is.
+    # The 1.5B shape's weights are small, its head large: its captured step is the same either way.
     PACKED_MAX_ROWS = 96
     PACKED_MAX_ROWS_LARGE = 192
+    PACKED_MAX_ROWS_LARGE_WIDE = 96
+    PACKED_MAX_ROWS_LARGE_WIDE_TIMED = 64
     PACKED_MAX_ROWS_EAGER = 192
     PACKED_LARGE_ELEMENTS = 32 << 20
     # or, for a weight of at most this many elements (too few row blocks to occupy the chip that way),
@@ -214,6 +225,7 @@ class HipOps(Ops):
         self._compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         self._lib = None
         self._tuning = False
+        self.library_timed_rows = 0
         self._packed_left_out = 0
         self._ops = ctypes.CDLL(str(build.ensure("ops")))
         self._declare()
@@ -278,9 +290,11 @@ class HipOps(Ops):
 
     def tune_library_products(self, on: bool) -> None:
         """While on, every new shape of a large product has the library's candidate kernels timed, and the
-        fastest is kept for that shape from then on; shapes first met while off take the library's first choice.
-        Products of up to `PACKED_MAX_ROWS` rows do not go to the library at all (`PACKED_MAX_ROWS_EAGER`
-        outside captured steps)."""
+        fastest is kept for that shape, and for the other row counts of its class of 32 rows, from then on; shapes
+        first met while off take their class's choice, or the library's first. Products of up to `PACKED_MAX_ROWS`
+        rows do not go to the library at all (`PACKED_MAX_ROWS_EAGER` outside captured steps; large weights:
+        see there). The caller that has had every class up to some number of rows timed says so in
+        `library_timed_rows`: up to there large weights with more rows than K leave the packed kernels at 65 rows."""
         self._tuning = bool(on)
 
     def graphs_supported(self) -> bool:
@@ -516,7 +530,7 @@ class HipOps(Ops):
             out = torch.empty((x.shape[0], N // 2), dtype=torch.bfloat16, device=self.device)
             return self._norm_product(x, packed, None, out, 1, N)
         x = self.dense(x)
-        if packed is None or x.dtype != torch.bfloat16 or x.shape[0] > self._packed_rows(gate_up_weight.numel()):
+        if packed is None or x.dtype != torch.bfloat16 or x.shape[0] > self._packed_rows(x.shape[0], *gate_up_weight.shape):
             return self.silu_mul(self.linear(x, gate_up_weight))
         self._own(x)
         M, K = x.shape
@@ -561,7 +575,7 @@ class HipOps(Ops):
                 table, slots, k_cache, v_cache, num_heads, num_kv_heads, head_dim, meta.block_size, 1 if write else 0))
         x = self.dense(x)
         fused = held is not None and held[1] == (num_heads, num_kv_heads, head_dim) and \
-            x.dtype == torch.bfloat16 and x.shape[0] <= self._packed_rows(weight.numel()) and \
+            x.dtype == torch.bfloat16 and x.shape[0] <= self._packed_rows(x.shape[0], *weight.shape) and \
             inv_freq is not None and 2 * inv_freq.shape[0] == head_dim and k_cache.dtype == torch.bfloat16
         if not fused:
             return self.rope_kv_write(self.linear(x, weight, bias), meta, group, k_cache, v_cache, inv_freq,
@@ -603,11 +617,13 @@ class HipOps(Ops):
             num_kv_heads, head_dim, meta.block_size, 1 if write else 0, self._stream()), "gemm_packed_rotary_bf16")
         return out
 
-    def _packed_rows(self, elements: int) -> int:
-        """Most rows of x that go through the kernels on the packed copy of a weight of `elements`."""
-        if self.captured:
-            return self.PACKED_MAX_ROWS if elements <= self.PACKED_LARGE_ELEMENTS else self.PACKED_MAX_ROWS_LARGE
-        return self.PACKED_MAX_ROWS_EAGER
+    def _packed_rows(self, M: int, N: int, K: int) -> int:
+        """Most rows of x that go through the kernels on the packed copy of an [N, K] weight, for a product of M rows."""
+        if N * K > self.PACKED_LARGE_ELEMENTS:
+            if K > N:
+                return self.PACKED_MAX_ROWS_LARGE
+            return self.PACKED_MAX_ROWS_LARGE_WIDE_TIMED if M <= self.library_timed_rows else self.PACKED_MAX_ROWS_LARGE_WIDE
+        return self.PACKED_MAX_ROWS if self.captured else self.PACKED_MAX_ROWS_EAGER
 
     def _library(self):
         """The vendor library's products, called directly; loaded at the first large product."""
@@ -732,7 +748,7 @@ class HipOps(Ops):
         packed = packed if both_bf16 else None
         if lazy and packed is not None and self._fused(M) and K % 8 == 0 and out_dtype == torch.bfloat16:
             return PendingProduct(x, weight, bias)
-        if packed is not None and self.ONE_WAVE_MAX_ROWS < M <= self._packed_rows(N * K) and K % 8 == 0 and \
+        if packed is not None and self.ONE_WAVE_MAX_ROWS < M <= self._packed_rows(M, N, K) and K % 8 == 0 and \
                 N * K > self.ROW_GROUPS_MAX_ELEMENTS:
             if packed.numel() != self._packed_elements(N, K, False):
                 raise KernelError("linear: the packed copy does not belong to this weight")
@@ -748,7 +764,7 @@ class HipOps(Ops):
             if slices == 1:
                 return out
             return PartialSums(out, out_dtype) if partial_ok else self.dense(PartialSums(out, out_dtype))
-        if both_bf16 and K % 8 == 0 and (M <= self.SKINNY_MAX_ROWS or (packed is not None and M <= self._packed_rows(N * K))):
+        if both_bf16 and K % 8 == 0 and (M <= self.SKINNY_MAX_ROWS or (packed is not None and M <= self._packed_rows(M, N, K))):
             if packed is not None:
                 if packed.numel() != self._packed_elements(N, K, False):
                     raise KernelError("linear: the packed copy does not belong to this weight")

@@ -215,6 +215,23 @@ def test_fewer_rows_through_the_packed_kernels_in_a_captured_step(ops):
         ops.captured = False
         del ops.PACKED_LARGE_ELEMENTS
     close(ops.dense(large), more.double() @ w.double().T, torch.bfloat16, scale=want.abs().max().item())
+    # ... if its K is longer than it has rows; a large weight with more rows than K leaves after one pass of up to 96
+    # rows of x, and after 64 once the library's kernels were timed for that many rows
+    wide, x96 = rand(3072, 1536, dtype=torch.bfloat16, seed=5), rand(96, 1536, dtype=torch.bfloat16, seed=6)
+    ops.prepare_linear(wide)
+    ops.PACKED_LARGE_ELEMENTS = 0
+    try:
+        one_pass = ops.linear(x96, wide)
+        assert isinstance(one_pass, PartialSums) and not isinstance(ops.linear(x[:100], wide), PartialSums)
+        ops.library_timed_rows = 192
+        through_library = ops.linear(x96, wide)
+        assert not isinstance(through_library, PartialSums) and isinstance(ops.linear(x96[:64], wide), PartialSums)
+    finally:
+        ops.library_timed_rows = 0
+        del ops.PACKED_LARGE_ELEMENTS
+    want = x96.double() @ wide.double().T
+    close(ops.dense(one_pass), want, torch.bfloat16, scale=want.abs().max().item())
+    close(through_library, want, torch.bfloat16, scale=want.abs().max().item())
 
 
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 40, 64, 81, 96, 150, 192])

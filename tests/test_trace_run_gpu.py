@@ -150,8 +150,9 @@ def test_generation_through_the_entry_point_and_the_command_line(tmp_path):
 
 def test_tuned_library_products(tmp_path):
     """`tune_products`: the engine starts with one full portion while the library's candidate kernels are
-    timed for the large products; afterwards new shapes take the library's first choice. Results stay within
-    the bounds, with whatever kernels were picked."""
+    timed for the large products, and with steps of 96, 128, 160 and 192 rows for the products of large decode
+    batches and short portions; afterwards new shapes take the choice of their class of 32 rows if one of its
+    shapes was timed, else the library's first. Results stay within the bounds, with whatever kernels were picked."""
     from distie_amd import LLM
     from distie_amd.engine.batch import StepEntry
     from engine_util import check_logits
@@ -162,6 +163,13 @@ def test_tuned_library_products(tmp_path):
               packed_weights=False)                 # without packed copies 400 rows are the library's
     made, timed = llm.ops.library_plans()
     assert timed >= 1 and not llm.ops._tuning       # the full portion's products were timed, and tuning is off again
+    assert llm.ops.library_timed_rows == 192 and not llm.ops.captured
+    for n, seed in ((160, 6), (150, 7), (96, 8)):   # a timed shape, another of its class, a timed shape
+        ids = random_ids(cfg, n, seed)
+        logits = llm.step([StepEntry("c", ids, list(range(n)))]).float().cpu()
+        llm.finish("c")
+        check_logits(logits, weights, cfg, ids, torch.bfloat16, folder)
+    assert llm.ops.library_plans()[1] == timed
     ids = random_ids(cfg, 300, 4)
     logits = llm.step([StepEntry("a", ids, list(range(len(ids))))]).float().cpu()
     llm.finish("a")
