@@ -11,7 +11,7 @@ import torch
 
 import plain_qwen2 as plain
 from distie_amd import LLM, SamplingParams, StepEntry
-from engine_util import build_runner, make_model_dir, random_ids, run_and_keep_logits
+from engine_util import FP32_TOL, build_runner, make_model_dir, random_ids, run_and_keep_logits
 
 pytestmark = pytest.mark.gpu
 
@@ -278,4 +278,58 @@ def test_short_mixed_steps_replay_graphs_and_give_the_plain_logits(tmp_path, nam
     assert graphs.mixed_replays >= len(shapes) + 10            # many steps replayed a graph made by an earlier one
     llm.cache.check()
     assert all(f == pages for f in llm.cache.free_pages()) and llm.cache.slots.num_free == llm.cache.num_slots
+    llm.close()
+
+
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("name,dtype,timed", [("B", "fp32", False), ("C", "fp32", True), ("1.5b", "bf16", False),
+                                              ("1.5b", "bf16", True)])
+def test_decode_batches_beyond_the_packed_kernels_rows(tmp_path, monkeypatch, models, name, dtype, timed):
+    """More live requests than the packed kernels take rows: 70, 100, 130 and 200 requests of 3 to 40 tokens decode
+    together through captured steps, whose products go to the library's kernels, or part of them (`timed`: every
+    weight counts as one that the memory-side cache does not hold, the library's kernels are timed at start, and
+    weights with more rows than K then leave the packed kernels at 65 rows while those with a longer K stay up to
+    192). Every step's rows are the plain model's: in float32 on two tiny configurations, in bfloat16 at the 1.5B
+    model's layer sizes (at a width of a few dozen, single rows among these two thousand sit where rounding is
+    amplified beyond the bound that the tiny models' tests hold: the same request alone is at 4.5 % there)."""
+    import random
+
+    from distie_amd.kernels.hip_ops import HipOps
+
+    if name == "1.5b":
+        folder, weights, cfg = models(name)
+        block = 16
+    else:
+        cfg, block = {"B": (plain.TINY_B, 8), "C": (plain.TINY_C, 16)}[name]
+        folder, weights = make_model_dir(tmp_path, cfg, seed=61, dtype=torch.float32)
+    if timed:
+        monkeypatch.setattr(HipOps, "PACKED_LARGE_ELEMENTS", 0)
+    most, new = 200, 5
+    llm = LLM(folder, dtype=dtype, block_size=block, num_blocks=most * (-(-(40 + new) // block)) + 8, max_seqs=most,
+              token_budget=256, tune_products=timed, lookahead=False, max_model_len=512)
+    assert llm.ops.library_timed_rows == (224 if timed else 0)
+    rng = random.Random(3)
+    for count in (70, 100, 130, 200):
+        seqs = {f"r{i}": random_ids(cfg, rng.randint(3, 40) + new, 900 + 7 * i + count) for i in range(count)}
+        names = list(seqs)
+        for first in range(0, count, 8):                    # the prompts, eight requests a step
+            llm.step([StepEntry(rid, seqs[rid][:-new], []) for rid in names[first:first + 8]])
+        replays = llm.runner.graphs.replays
+        rows = {rid: [] for rid in names}
+        for t in range(new):
+            logits = llm.step([StepEntry(rid, [seqs[rid][len(seqs[rid]) - new + t]], [0]) for rid in names]).float().cpu()
+            for row, rid in enumerate(names):
+                rows[rid].append(logits[row])
+        assert llm.runner.graphs.replays == replays + new, "the decode steps went through captured steps"
+        for rid in names:                                   # judged as everywhere (engine_util.check_logits)
+            ids = seqs[rid]
+            want = plain.forward(weights, cfg, ids, torch.float64, rows=list(range(len(ids) - new, len(ids)))).float().cpu()
+            diff = torch.stack(rows[rid]) - want
+            scale = want.abs().max().item()
+            if dtype == "fp32":
+                assert diff.abs().max().item() < FP32_TOL, (count, rid)
+            else:
+                assert diff.abs().max().item() < scale / 16 and diff.pow(2).mean().sqrt().item() < scale / 64, (count, rid)
+            llm.finish(rid)
+    llm.cache.check()
     llm.close()
