@@ -512,15 +512,58 @@ struct KeyRuns {
   int length;     // keys per run
   int count;      // runs that hold a key
 };
-__device__ __forceinline__ KeyRuns key_runs(int q_pos, int window, int max_splits) {
+// run_len > 0: runs of this length for every request (`decode_run_len_kernel`), so that a long request gets more of them
+// than a short one; the caller made it long enough for the longest request to fit max_splits runs.
+__device__ __forceinline__ KeyRuns key_runs(int q_pos, int window, int max_splits, int run_len = 0) {
   KeyRuns runs;
   runs.first = window > 0 ? max(0, q_pos - window + 1) : 0;
   runs.origin = runs.first / RUN_STEP * RUN_STEP;
   const int span = q_pos - runs.origin + 1;
   const int step = max_splits * RUN_STEP;
-  runs.length = (span + step - 1) / step * RUN_STEP;        // ceil(span / max_splits), rounded up to RUN_STEP
+  runs.length = run_len > 0 ? run_len : (span + step - 1) / step * RUN_STEP;        // ceil(span / max_splits), rounded up to RUN_STEP
   runs.count = (span + runs.length - 1) / runs.length;      // <= max_splits
   return runs;
+}
+
+// One run length for all requests of a step (no window): the shortest, in steps of 64 keys, with which the runs of
+// all requests together are at most `budget` (as many waves as the chip has SIMDs, per kv head: the kernel keeps one
+// wave a SIMD, so a wave more than that waits for a place) and no request has more than `max_splits`. A long
+// request then gets more runs than a short one. With every request cut into the same number of runs the runs of the
+// longest end last, alone: 96 requests of 1,050 to 3,150 keys take 119 us, with one run length 96 (the same keys
+// in requests of one length: 89); requests of one length are cut exactly as without it. It is the same for every
+// layer of a step, so one wave finds it once a step and the attention kernels read it beside their request's
+// length (found by every wave of theirs it cost 3 to 10 us a call).
+__global__ __launch_bounds__(DISTIE_WAVE) void decode_run_len_kernel(const int32_t* __restrict__ kv_len, int num_requests,
+                                                                     int budget, int max_splits, int32_t* __restrict__ run_len) {
+  const int lane = threadIdx.x;
+  int most = 1;
+  for (int i = lane; i < num_requests; i += DISTIE_WAVE) most = max(most, kv_len[i]);
+#pragma unroll
+  for (int o = DISTIE_WAVE / 2; o > 0; o >>= 1) most = max(most, __shfl_xor(most, o, DISTIE_WAVE));
+  // in units of RUN_STEP keys: from what the longest request needs to fit max_splits runs, up to one run a request
+  int lo = (most + max_splits * RUN_STEP - 1) / (max_splits * RUN_STEP);
+  int hi = (most + RUN_STEP - 1) / RUN_STEP;
+  while (lo < hi) {                                     // (the same in every lane)
+    const int mid = (lo + hi) / 2;
+    int runs = 0;
+    for (int i = lane; i < num_requests; i += DISTIE_WAVE) runs += (kv_len[i] + mid * RUN_STEP - 1) / (mid * RUN_STEP);
+#pragma unroll
+    for (int o = DISTIE_WAVE / 2; o > 0; o >>= 1) runs += __shfl_xor(runs, o, DISTIE_WAVE);
+    if (runs <= budget) {
+      hi = mid;
+    } else {
+      lo = mid + 1;
+    }
+  }
+  if (lane == 0) *run_len = lo * RUN_STEP;
+}
+
+// run_len: int32 [1], for a step of num_requests requests that bring one token each.
+extern "C" int distie_attention_decode_run_len(const int32_t* kv_len, int num_requests, int budget, int max_splits,
+                                               int32_t* run_len, hipStream_t stream) {
+  if (num_requests < 1 || budget < 1 || max_splits < 1 || kv_len == nullptr || run_len == nullptr) return DISTIE_BAD_ARGUMENT;
+  decode_run_len_kernel<<<1, DISTIE_WAVE, 0, stream>>>(kv_len, num_requests, budget, max_splits, run_len);
+  return launch_status();
 }
 
 template <int MB>
@@ -529,30 +572,36 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ kv_len, const int32_t* __restrict__ cu_q,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ table_rows, float* __restrict__ part_o,
     float* __restrict__ part_ml, int heads, int kv_heads, int block_size, float scale, int window, int split_hint,
-    int max_splits, int dense_rows) {
+    int max_splits, int dense_rows, const int32_t* __restrict__ shared_run_len) {
   const int lane = threadIdx.x;
   const int r = lane % 16;
   const int g = lane / 16;
   const int group = heads / kv_heads;
   const float scale_log2 = scale * 1.4426950408889634f;
-  const int request = blockIdx.z;
-  const int kh = blockIdx.y;
+  // With a shared run length the run is the slowest index of the grid: the places past a request's last run, whose
+  // waves leave at once, then come after all the others (in front of them they held the SIMDs that the working
+  // waves behind them were waiting for: 64 requests took 106 us instead of 54).
+  const bool shared = shared_run_len != nullptr;
+  const int run = shared ? blockIdx.z : blockIdx.x;
+  const int request = shared ? blockIdx.y : blockIdx.z;
+  const int kh = shared ? blockIdx.x : blockIdx.y;
   const int32_t* table = block_table + static_cast<int64_t>(table_rows != nullptr ? table_rows[request] : request) * table_width;
   // The pages of the run's first chunk are asked for before the request's length says where the run begins:
   // at the place it has if the runs are `split_hint` long and begin at key 0, which the host derives from the
   // longest request of the step (the entry is inside the table either way). Where the guess holds, which it
   // does when few requests of similar length decode, that is one trip to memory less on the way to the keys.
-  const int guess_begin = static_cast<int>(blockIdx.x) * split_hint;
+  const int guess_begin = run * split_hint;
   int pages[DC_BLOCKS];
 #pragma unroll
   for (int b = 0; b < DC_BLOCKS; ++b) pages[b] = table[min((guess_begin + 16 * b) / block_size, table_width - 1)];
   // dense_rows: every request brings one token, so request i's token is row i
+  const int run_len = shared ? *shared_run_len : 0;
   const int token = dense_rows ? request : cu_q[request];
   if (!dense_rows && cu_q[request + 1] - token != 1) return;        // a portion of a prompt: the tiled kernel's
   const int q_pos = kv_len[request] - 1;              // the new token is the last one cached
-  const KeyRuns runs = key_runs(q_pos, window, max_splits);
-  if (static_cast<int>(blockIdx.x) >= runs.count) return;
-  const int run_begin = runs.origin + static_cast<int>(blockIdx.x) * runs.length;
+  const KeyRuns runs = key_runs(q_pos, window, max_splits, run_len);
+  if (run >= runs.count) return;
+  const int run_begin = runs.origin + run * runs.length;
   const int key_begin = max(runs.first, run_begin);
   const int key_end = min(q_pos, run_begin + runs.length - 1);
 
@@ -717,7 +766,7 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
       const float l_col = __shfl(l_run[mb], 4 * g + i, DISTIE_WAVE);
       const float m_col = __shfl(m_run[mb], 4 * g + i, DISTIE_WAVE);
       if (col >= group) continue;
-      const int64_t slot = (static_cast<int64_t>(request) * heads + kh * group + col) * max_splits + blockIdx.x;
+      const int64_t slot = (static_cast<int64_t>(request) * heads + kh * group + col) * max_splits + run;
       float* po = part_o + slot * D;
 #pragma unroll
       for (int db = 0; db < DB16; ++db) po[16 * db + r] = o_acc[mb][db][i];
@@ -745,7 +794,7 @@ template <bool FAST>
 __global__ __launch_bounds__(RD_THREADS) void attn_reduce_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int32_t* __restrict__ kv_len,
     const int32_t* __restrict__ cu_q, bf16_t* __restrict__ out, int heads, int window, int max_splits,
-    int dense_rows) {
+    int dense_rows, const int32_t* __restrict__ shared_run_len) {
   __shared__ float weight_s[FAST ? RD_FAST_RUNS : RD_MAX_RUNS];
   __shared__ float sum_s[RD_WAVES][D];
   __shared__ float scratch[32];
@@ -774,7 +823,7 @@ __global__ __launch_bounds__(RD_THREADS) void attn_reduce_kernel(
   const int token = dense_rows ? request : cu_q[request];
   if (!dense_rows && cu_q[request + 1] - token != 1) return;
   const int q_pos = kv_len[request] - 1;
-  const int runs = key_runs(q_pos, window, max_splits).count;     // the first `runs` places hold results
+  const int runs = key_runs(q_pos, window, max_splits, shared_run_len != nullptr ? *shared_run_len : 0).count;     // the first `runs` places hold results
   const int64_t base = base0;
   bf16_t* o = out + (static_cast<int64_t>(token) * heads + head) * D;
 
@@ -863,26 +912,29 @@ extern "C" int distie_attention_decode_columns() { return 16 * DECODE_MAX_MB; }
 // request. part_o: float32 [requests, heads, max_splits, D], part_ml: float32 [requests, heads, max_splits, 2]:
 // every request's keys are cut into at most max_splits runs by its own length. split_hint, a multiple of 64, is
 // the run length the caller expects of the longest request; it only saves time where it is right.
+// shared_run_len (no window, every request of the step brings one token; else null): int32 [1], one run length for
+// all requests, with which no request has more than max_splits runs (distie_attention_decode_run_len).
 extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, const void* k_cache, const void* v_cache,
                                             const int32_t* kv_len, const int32_t* cu_q, const int32_t* block_table,
                                             int table_width, const int32_t* table_rows, void* out, float* part_o, float* part_ml,
                                             int num_requests, int heads, int kv_heads, int block_size, float scale,
                                             int window, int split_hint, int max_splits, int dense_rows,
-                                            hipStream_t stream) {
+                                            const int32_t* shared_run_len, hipStream_t stream) {
   if (num_requests <= 0) return 0;
   const int group = kv_heads > 0 ? heads / kv_heads : 0;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size % 16 != 0 || table_width < 1 || window < 0 ||
       split_hint < RUN_STEP || split_hint % RUN_STEP != 0 || max_splits < 1 || max_splits > RD_MAX_RUNS ||
-      group > 16 * DECODE_MAX_MB || kv_heads > 65535 || num_requests > 65535 || heads > 65535)
+      group > 16 * DECODE_MAX_MB || kv_heads > 65535 || num_requests > 65535 || heads > 65535 ||
+      (shared_run_len != nullptr && (window > 0 || !dense_rows)))
     return DISTIE_BAD_ARGUMENT;
-  dim3 grid(max_splits, kv_heads, num_requests);
+  const dim3 grid = shared_run_len != nullptr ? dim3(kv_heads, num_requests, max_splits) : dim3(max_splits, kv_heads, num_requests);
   const bf16_t* q = static_cast<const bf16_t*>(qkv);
   const bf16_t* kc = static_cast<const bf16_t*>(k_cache);
   const bf16_t* vc = static_cast<const bf16_t*>(v_cache);
 #define DECODE_LAUNCH(MB)                                                                                             \
   attn_decode_kernel<MB><<<grid, DISTIE_WAVE, 0, stream>>>(q, q_stride, kc, vc, kv_len, cu_q, block_table, table_width, table_rows, \
                                                            part_o, part_ml, heads, kv_heads, block_size, scale, window, \
-                                                           split_hint, max_splits, dense_rows)
+                                                           split_hint, max_splits, dense_rows, shared_run_len)
   if (group <= 16) {
     DECODE_LAUNCH(1);
   } else if (group <= 32) {
@@ -895,10 +947,10 @@ extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, c
   if (status != 0) return status;
   if (max_splits <= RD_FAST_RUNS) {
     attn_reduce_kernel<true><<<dim3(heads, num_requests), RD_THREADS, 0, stream>>>(
-        part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, max_splits, dense_rows);
+        part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, max_splits, dense_rows, shared_run_len);
   } else {
     attn_reduce_kernel<false><<<dim3(heads, num_requests), RD_THREADS, 0, stream>>>(
-        part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, max_splits, dense_rows);
+        part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, max_splits, dense_rows, shared_run_len);
   }
   return launch_status();
 }
@@ -1630,9 +1682,11 @@ extern "C" int distie_attention_decode_columns() { return 0; }
 
 extern "C" int distie_attention_decode_bf16(const void*, int64_t, const void*, const void*, const int32_t*, const int32_t*,
                                             const int32_t*, int, const int32_t*, void*, void*, void*, int, int, int, int, float, int, int,
-                                            int, int, hipStream_t) {
+                                            int, int, const int32_t*, hipStream_t) {
   return DISTIE_BAD_ARGUMENT;
 }
+
+extern "C" int distie_attention_decode_run_len(const int32_t*, int, int, int, int32_t*, hipStream_t) { return DISTIE_BAD_ARGUMENT; }
 
 extern "C" int distie_attention_prefill_bf16(const void*, int64_t, const void*, const void*, const int32_t*, const int32_t*,
                                              const int32_t*, int, const int32_t*, void*, int, int, int, int, int, float, int, int,

@@ -200,6 +200,12 @@ class HipOps(Ops):
     # decode attention cuts the keys into runs so that about DECODE_WAVES waves are at work, with at most
     # DECODE_MAX_RUNS places for partial results per request and head
     DECODE_WAVES = 1024
+    # where the same number of runs for every request leaves more than a fifth of those waves unused (640 pairs: one
+    # run each), the requests of a decode step share one run length instead: the shortest with which their runs
+    # together stay within DECODE_WAVES, so that a long request gets more runs than a short one (7B shape's heads,
+    # contexts of 1,050 to 3,150 keys: 96 requests 121 -> 95 us a layer, 160 requests 223 -> 164; with contexts of one
+    # length it changes nothing). Where the waves are all in use already it lost (64 requests: 61 -> 68 us).
+    DECODE_SHARED_BELOW = 0.8
     DECODE_MAX_RUNS = 256
 
     def __init__(self, device="cuda:0", packed_weights=True) -> None:
@@ -321,7 +327,8 @@ class HipOps(Ops):
                                                           _F, _I, _I, _P, _P, _P, _I, _P]
             lib.distie_attention_prefill_f32.argtypes = lib.distie_attention_prefill_bf16.argtypes
             lib.distie_attention_decode_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I,
-                                                         _I, _F, _I, _I, _I, _I, _P]
+                                                         _I, _F, _I, _I, _I, _I, _P, _P]
+            lib.distie_attention_decode_run_len.argtypes = [_P, _I, _I, _I, _P, _P]
             if lib.distie_attention_head_dim() != head_dim:
                 raise KernelError("attention library was built for another head size")
             self._attn[head_dim] = lib
@@ -877,7 +884,8 @@ class HipOps(Ops):
             # with these sizes: worked out once per step (the layers run one after the other, so they can
             # share the buffers)
             key = ("attention", int(window or 0), num_heads, num_kv_heads, head_dim, meta.max_kv, meta.all_decode,
-                   meta.singles_bound, self.PREFILL_PARTS, self.PREFILL_WORKGROUPS, self.DECODE_WAVES, self.DECODE_MAX_RUNS)
+                   meta.singles_bound, self.PREFILL_PARTS, self.PREFILL_WORKGROUPS, self.DECODE_WAVES, self.DECODE_MAX_RUNS,
+                   self.DECODE_SHARED_BELOW)
             plan = meta.scratch.get(key)
             if plan is None or plan["cu_q"] is not meta.host_cu_q:
                 plan = meta.scratch[key] = self._attention_plan(lib, meta, T, num_heads, num_kv_heads, head_dim, window)
@@ -887,7 +895,9 @@ class HipOps(Ops):
                     meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], rows_ptr, out.data_ptr(),
                     plan["decode_o"].data_ptr(), plan["decode_ml"].data_ptr(), meta.num_requests, num_heads,
                     num_kv_heads, meta.block_size, float(scale), int(window or 0), plan["split_len"],
-                    plan["max_splits"], 1 if meta.all_decode else 0, self._stream()), "attention_decode_bf16")
+                    plan["max_splits"], 1 if meta.all_decode else 0,
+                    plan["run_len"].data_ptr() if plan["run_len"] is not None else None, self._stream()),
+                    "attention_decode_bf16")
             if plan["prefill"]:
                 parts = plan["parts"]
                 _check(lib.distie_attention_prefill_bf16(
@@ -941,8 +951,20 @@ class HipOps(Ops):
             visible = min(meta.max_kv, int(window) + 63) if window else meta.max_kv
             max_splits = max(1, min(self.DECODE_MAX_RUNS, self.DECODE_WAVES // (singles * num_kv_heads),
                                     -(-visible // 64)))
-            plan["max_splits"] = max_splits
             plan["split_len"] = -(-visible // (64 * max_splits)) * 64
+            # every request with one token, no window, waves left over: one run length for all of them, so that a
+            # long request gets more runs than a short one (up to twice what every request would get)
+            plan["run_len"] = None
+            pairs = singles * num_kv_heads
+            if meta.all_decode and not window and max_splits * pairs <= self.DECODE_SHARED_BELOW * self.DECODE_WAVES:
+                splits = max_splits
+                max_splits = max(1, min(self.DECODE_MAX_RUNS, 2 * splits, -(-visible // 64)))
+                plan["run_len"] = torch.empty(1, dtype=torch.int32, device=self.device)
+                _check(lib.distie_attention_decode_run_len(meta.kv_len.data_ptr(), meta.num_requests,
+                                                           max(1, self.DECODE_WAVES // num_kv_heads), max_splits,
+                                                           plan["run_len"].data_ptr(), self._stream()),
+                       "attention_decode_run_len")
+            plan["max_splits"] = max_splits
             plan["decode_o"] = torch.empty((meta.num_requests, num_heads, max_splits, head_dim), dtype=torch.float32,
                                            device=self.device)
             plan["decode_ml"] = torch.empty((meta.num_requests, num_heads, max_splits, 2), dtype=torch.float32,

@@ -745,6 +745,46 @@ def test_paged_attention_keys_walked_in_parts(ops, dtype, heads, kv_heads, dim, 
     close(whole, want, dtype, scale=want.abs().max().item())
 
 
+@pytest.mark.parametrize("requests,heads,kv_heads,dim,P", [(65, 8, 4, 64, 16), (100, 28, 4, 128, 16), (200, 12, 2, 128, 32),
+                                                           (150, 4, 4, 48, 16), (700, 3, 1, 32, 16), (80, 10, 5, 80, 64)])
+def test_decode_steps_of_many_requests_share_one_run_length(ops, requests, heads, kv_heads, dim, P):
+    """Where cutting every request into the same number of runs would leave a fifth of the waves unused, the
+    requests of a decode step share one run length, found on the device from the step's lengths: requests of 1 to
+    1,500 keys (a long one gets several runs, a short one a single one, some end on a run's edge), then one far
+    longer than the others (it is what bounds the run length), then all of one length; as launched for these
+    lengths and as in a captured step that was made for far longer ones. Against plain attention."""
+    import random
+
+    rng = random.Random(requests)
+    for lens in ([rng.choice([1, 2, 63, 64, 65, 128, 640, 1280]) if i % 3 == 0 else rng.randint(1, 1500) for i in range(requests)],
+                 [4000] + [rng.randint(1, 90) for _ in range(requests - 1)],
+                 [333] * requests):
+        meta, qkv, k, v = paged_case(heads, kv_heads, dim, P, lens, [1] * requests, torch.bfloat16, seed=requests)
+        assert meta.all_decode
+        want = TorchOps("cuda").paged_attention(qkv.double(), meta, 0, k.double(), v.double(), heads, kv_heads, dim,
+                                                dim ** -0.5, None)
+        for limit in (max(lens), 8192):
+            meta.max_kv = limit
+            meta.scratch.clear()
+            got = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, None)
+            plans = [plan for plan in meta.scratch.values() if isinstance(plan, dict) and "run_len" in plan]
+            assert len(plans) == 1 and plans[0]["run_len"] is not None, "the step did not take the shared run length"
+            run_len = int(plans[0]["run_len"].item())
+            budget, most = ops.DECODE_WAVES // kv_heads, plans[0]["max_splits"]
+            runs = lambda length: sum(-(-n // length) for n in lens)
+            assert run_len % 64 == 0 and max(-(-n // run_len) for n in lens) <= most
+            # the shortest that keeps the runs within the waves, unless the longest request asks for a longer one
+            assert runs(run_len) <= budget or run_len >= -(-max(lens) // 64) * 64
+            assert run_len == 64 or runs(run_len - 64) > budget or -(-max(lens) // (run_len - 64)) > most
+            close(got, want, torch.bfloat16, scale=want.abs().max().item())
+        # under a window, or with fewer requests, every request is cut by its own length as before
+        windowed = ops.paged_attention(qkv, meta, 0, k, v, heads, kv_heads, dim, dim ** -0.5, 100)
+        assert all(plan.get("run_len") is None for key, plan in meta.scratch.items() if isinstance(plan, dict) and key[1] == 100)
+        want = TorchOps("cuda").paged_attention(qkv.double(), meta, 0, k.double(), v.double(), heads, kv_heads, dim,
+                                                dim ** -0.5, 100)
+        close(windowed, want, torch.bfloat16, scale=want.abs().max().item())
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,kv_heads,dim,P,window", ATTENTION_SHAPES)
 def test_paged_attention_decode_step(ops, dtype, heads, kv_heads, dim, P, window):
