@@ -526,13 +526,13 @@ __device__ __forceinline__ KeyRuns key_runs(int q_pos, int window, int max_split
 }
 
 // One run length for all requests of a step (no window): the shortest, in steps of 64 keys, with which the runs of
-// all requests together are at most `budget` (as many waves as the chip has SIMDs, per kv head: the kernel keeps one
-// wave a SIMD, so a wave more than that waits for a place) and no request has more than `max_splits`. A long
-// request then gets more runs than a short one. With every request cut into the same number of runs the runs of the
-// longest end last, alone: 96 requests of 1,050 to 3,150 keys take 119 us, with one run length 96 (the same keys
-// in requests of one length: 89); requests of one length are cut exactly as without it. It is the same for every
-// layer of a step, so one wave finds it once a step and the attention kernels read it beside their request's
-// length (found by every wave of theirs it cost 3 to 10 us a call).
+// all requests together are at most `budget` (the waves the caller wants at work, per kv head) and no request has
+// more than `max_splits`. A long request then gets more runs than a short one; with every request cut into the
+// same number of runs the runs of the longest end last, alone. The caller uses it where that same number would
+// leave many of the waves unused (256 requests of 1,050 to 3,150 keys on 4 kv heads, one run each: 263 us, with one
+// run length 245); requests of one length are cut exactly as without it. It is the same for every layer of a step,
+// so one wave finds it once a step and the attention kernels read it beside their request's length (found by
+// every wave of theirs it cost 3 to 10 us a call).
 __global__ __launch_bounds__(DISTIE_WAVE) void decode_run_len_kernel(const int32_t* __restrict__ kv_len, int num_requests,
                                                                      int budget, int max_splits, int32_t* __restrict__ run_len) {
   const int lane = threadIdx.x;
@@ -566,8 +566,13 @@ extern "C" int distie_attention_decode_run_len(const int32_t* kv_len, int num_re
   return launch_status();
 }
 
+// Two waves a SIMD where the registers allow it without spilling (one block of query heads, head sizes up to 128:
+// 234 registers; left to itself the compiler took a few more and one wave a SIMD). The chip then holds 2,048 waves
+// instead of 1,024, and a batch whose runs are a few more than 1,024, or whose requests differ in length, no
+// longer waits for the last waves to get a place: 7B shape's heads at 2,100 keys, 96 requests 91 -> 83 us a layer,
+// 160 requests 165 -> 130; contexts of 1,050 to 3,150 keys, 96 requests 121 -> 96, 160 requests 222 -> 157.
 template <int MB>
-__global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
+__global__ __launch_bounds__(DISTIE_WAVE, (MB == 1 && D <= 128 ? 2 : 1)) void attn_decode_kernel(
     const bf16_t* __restrict__ qkv, int64_t q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ kv_len, const int32_t* __restrict__ cu_q,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ table_rows, float* __restrict__ part_o,
@@ -579,8 +584,8 @@ __global__ __launch_bounds__(DISTIE_WAVE) void attn_decode_kernel(
   const int group = heads / kv_heads;
   const float scale_log2 = scale * 1.4426950408889634f;
   // With a shared run length the run is the slowest index of the grid: the places past a request's last run, whose
-  // waves leave at once, then come after all the others (in front of them they held the SIMDs that the working
-  // waves behind them were waiting for: 64 requests took 106 us instead of 54).
+  // waves leave at once, then come after all the others (in front of them they held the places on the SIMDs that
+  // the working waves behind them were waiting for: 64 requests took 106 us instead of 54, at one wave a SIMD).
   const bool shared = shared_run_len != nullptr;
   const int run = shared ? blockIdx.z : blockIdx.x;
   const int request = shared ? blockIdx.y : blockIdx.z;

@@ -198,13 +198,15 @@ class HipOps(Ops):
     PACKED_KEEPS_FREE = 0.3          # share of the device's memory that packed weight copies leave free
     PREFILL_F32_MIN_TOKENS = 32      # float32 steps with a portion of at least this many tokens go to the tiled float32 kernel
     # decode attention cuts the keys into runs so that about DECODE_WAVES waves are at work, with at most
-    # DECODE_MAX_RUNS places for partial results per request and head
-    DECODE_WAVES = 1024
-    # where the same number of runs for every request leaves more than a fifth of those waves unused (640 pairs: one
-    # run each), the requests of a decode step share one run length instead: the shortest with which their runs
-    # together stay within DECODE_WAVES, so that a long request gets more runs than a short one (7B shape's heads,
-    # contexts of 1,050 to 3,150 keys: 96 requests 121 -> 95 us a layer, 160 requests 223 -> 164; with contexts of one
-    # length it changes nothing). Where the waves are all in use already it lost (64 requests: 61 -> 68 us).
+    # DECODE_MAX_RUNS places for partial results per request and head. The kernel keeps two waves a SIMD (2,048 on
+    # the chip); 1,536 is what the step likes best (1.5B shape, batch 32 and 64: 2.07 and 2.77 ms with 1,024, 2.02
+    # and 2.71 with 1,536, 2.11 and 2.75 with 2,048; 7B shape, batch 160: 10.85, 10.05, 10.15 ms; batch 1 to 16 the same)
+    DECODE_WAVES = 1536
+    # where the same number of runs for every request leaves more than a fifth of those waves unused (1,024 pairs
+    # of a request and a kv head: one run each), the requests of a decode step share one run length instead: the
+    # shortest with which their runs together stay within DECODE_WAVES, so that a long request gets more runs than a
+    # short one (256 requests on 4 kv heads, contexts of 1,050 to 3,150 keys: 263 -> 245 us a layer; contexts of one
+    # length are cut as before). Everywhere else it is level or behind (32 requests: 30 -> 33 us).
     DECODE_SHARED_BELOW = 0.8
     DECODE_MAX_RUNS = 256
 

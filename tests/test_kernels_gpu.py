@@ -747,14 +747,16 @@ def test_paged_attention_keys_walked_in_parts(ops, dtype, heads, kv_heads, dim, 
 
 @pytest.mark.parametrize("requests,heads,kv_heads,dim,P", [(65, 8, 4, 64, 16), (100, 28, 4, 128, 16), (200, 12, 2, 128, 32),
                                                            (150, 4, 4, 48, 16), (700, 3, 1, 32, 16), (80, 10, 5, 80, 64)])
-def test_decode_steps_of_many_requests_share_one_run_length(ops, requests, heads, kv_heads, dim, P):
-    """Where cutting every request into the same number of runs would leave a fifth of the waves unused, the
-    requests of a decode step share one run length, found on the device from the step's lengths: requests of 1 to
+def test_decode_steps_of_many_requests_share_one_run_length(ops, monkeypatch, requests, heads, kv_heads, dim, P):
+    """Where cutting every request into the same number of runs would leave a fifth of the waves unused (here:
+    wherever no window applies), the requests of a decode step share one run length, found on the device from the
+    step's lengths: requests of 1 to
     1,500 keys (a long one gets several runs, a short one a single one, some end on a run's edge), then one far
     longer than the others (it is what bounds the run length), then all of one length; as launched for these
     lengths and as in a captured step that was made for far longer ones. Against plain attention."""
     import random
 
+    monkeypatch.setattr(type(ops), "DECODE_SHARED_BELOW", 1.01)
     rng = random.Random(requests)
     for lens in ([rng.choice([1, 2, 63, 64, 65, 128, 640, 1280]) if i % 3 == 0 else rng.randint(1, 1500) for i in range(requests)],
                  [4000] + [rng.randint(1, 90) for _ in range(requests - 1)],
