@@ -61,13 +61,25 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void argmax_kernel(const float* __r
 __global__ __launch_bounds__(SAMPLE_THREADS) void argmax_pieces_kernel(const float* __restrict__ logits,
                                                                        float* __restrict__ piece_value,
                                                                        int32_t* __restrict__ piece_index, int vocab,
-                                                                       int piece_len) {
+                                                                       int piece_len, int by_four) {
   __shared__ Best scratch[SAMPLE_THREADS / DISTIE_WAVE];
   const float* row = logits + static_cast<int64_t>(blockIdx.y) * vocab;
   const int begin = blockIdx.x * piece_len;
   const int end = min(vocab, begin + piece_len);
   Best mine{-INFINITY, 0x7fffffff};
-  for (int i = begin + threadIdx.x; i < end; i += blockDim.x) mine = better(mine, Best{row[i], i});
+  if (by_four) {
+    // pieces begin and end at multiples of four and the rows are 16-byte aligned: four logits a load
+    // (64 rows of 151,936: 22.4 -> 10.2 us, 8 rows: 10.0 -> 5.0)
+    for (int i = begin + 4 * static_cast<int>(threadIdx.x); i < end; i += 4 * static_cast<int>(blockDim.x)) {
+      const float4 v = *reinterpret_cast<const float4*>(row + i);
+      mine = better(mine, Best{v.x, i});
+      mine = better(mine, Best{v.y, i + 1});
+      mine = better(mine, Best{v.z, i + 2});
+      mine = better(mine, Best{v.w, i + 3});
+    }
+  } else {
+    for (int i = begin + threadIdx.x; i < end; i += blockDim.x) mine = better(mine, Best{row[i], i});
+  }
   const Best best = block_best(mine, scratch);
   if (threadIdx.x == 0) {
     piece_value[blockIdx.y * gridDim.x + blockIdx.x] = best.value;
@@ -108,8 +120,10 @@ extern "C" int distie_argmax(const float* logits, int32_t* out, int rows, int vo
     return launch_status();
   }
   if (piece_value == nullptr || piece_index == nullptr) return DISTIE_BAD_ARGUMENT;
-  const int piece_len = (vocab + parts - 1) / parts;
-  argmax_pieces_kernel<<<dim3(parts, rows), SAMPLE_THREADS, 0, stream>>>(logits, piece_value, piece_index, vocab, piece_len);
+  const int by_four = vocab % 4 == 0 && reinterpret_cast<uintptr_t>(logits) % 16 == 0;
+  const int piece_len = by_four ? ((vocab / 4 + parts - 1) / parts) * 4 : (vocab + parts - 1) / parts;
+  argmax_pieces_kernel<<<dim3(parts, rows), SAMPLE_THREADS, 0, stream>>>(logits, piece_value, piece_index, vocab, piece_len,
+                                                                         by_four);
   argmax_combine_kernel<<<rows, DISTIE_WAVE, 0, stream>>>(piece_value, piece_index, out, parts, vocab);
   return launch_status();
 }
@@ -173,8 +187,10 @@ extern "C" int distie_argmax_static(const float* logits, int32_t* out, int rows,
   // every entry that the second launch reads is written by the first: nothing has to be cleared
   float* piece_value = static_cast<float*>(base);
   int32_t* piece_index = reinterpret_cast<int32_t*>(piece_value + DISTIE_ARGMAX_STATIC_ENTRIES);
-  const int piece_len = (vocab + parts - 1) / parts;
-  argmax_pieces_kernel<<<dim3(parts, rows), SAMPLE_THREADS, 0, stream>>>(logits, piece_value, piece_index, vocab, piece_len);
+  const int by_four = vocab % 4 == 0 && reinterpret_cast<uintptr_t>(logits) % 16 == 0;
+  const int piece_len = by_four ? ((vocab / 4 + parts - 1) / parts) * 4 : (vocab + parts - 1) / parts;
+  argmax_pieces_kernel<<<dim3(parts, rows), SAMPLE_THREADS, 0, stream>>>(logits, piece_value, piece_index, vocab, piece_len,
+                                                                         by_four);
   argmax_combine_kernel<<<rows, DISTIE_WAVE, 0, stream>>>(piece_value, piece_index, out, parts, vocab);
   return launch_status();
 }

@@ -984,6 +984,17 @@ def test_argmax_and_sample(ops):
     big[1, 151935] = big[1, 70000] = 9.0           # equals in different pieces of the row
     big[2, 4096] = 8.0
     assert ops.argmax(big).tolist() == [int(big[0].argmax()), 70000, 4096]
+    big[0, 1001] = big[0, 1002] = big[0, 1003] = 11.0      # equals inside one load of four logits
+    assert ops.argmax(big).tolist() == [1001, 70000, 4096]
+    # rows that do not begin at a multiple of 16 bytes, and a vocabulary that is no multiple of four: one logit a load
+    flat = rand(2 * 151936 + 1, seed=12)
+    shifted = flat[1:].view(2, 151936)
+    shifted[1, 151935] = shifted[1, 151934] = 7.0
+    assert shifted.data_ptr() % 16 != 0 and ops.argmax(shifted).tolist() == [int(shifted[0].argmax()), 151934]
+    odd = rand(5, 40001, seed=13)
+    odd[3, 40000] = 9.0
+    odd[4, 17] = odd[4, 39999] = 9.5
+    assert ops.argmax(odd).tolist() == [int(r.argmax()) for r in odd[:3]] + [40000, 17]
     temps = torch.tensor([0.0, 0.7, 1.0, 1.5, 0.3, 2.0], device="cuda")
     hits = 0
     trials = 40
